@@ -1,0 +1,67 @@
+"""The device memory behind the cache manager.
+
+For every entry of the run order that owns a cache: keys ``[pages, Hk, page_size, D]``
+and values ``[pages, Hk, D, page_size]`` (values transposed inside a page so that
+attention reads several positions of one channel with one load), in the engine's
+dtype.  For every entry whose mixer has state of fixed size: ``[slots, *shape]``.
+Page 0 is the null page.  Nothing is zeroed when a page changes hands: reads are
+bounded by a request's length, so a page's old contents are never seen.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import Dict, List, Optional
+
+import torch
+
+from ..parts.base import KVSpec, StateSpec
+
+
+@dataclass
+class LayerCache:
+    """What one entry of the run order sees of the cache."""
+    group: int                 # which block table of a request applies
+    page_size: int
+    owns: bool                 # this entry writes keys and values (False: it reads another entry's)
+    k: Optional[torch.Tensor]
+    v: Optional[torch.Tensor]
+    state: Optional[torch.Tensor] = None    # [slots, *shape]
+
+
+class CacheStorage:
+    def __init__(self, kv_specs: List[Optional[KVSpec]], state_specs: List[Optional[StateSpec]],
+                 cache_of: List[Optional[int]], page_size: int, pages_per_group: int, n_slots: int,
+                 dtype: torch.dtype, device: torch.device):
+        """``kv_specs[i]``/``state_specs[i]``/``cache_of[i]`` describe entry ``i`` of the run order."""
+        self.page_size, self.n_pages, self.n_slots = page_size, pages_per_group + 1, n_slots
+        self.group_specs: List[KVSpec] = []
+        self.layers: List[LayerCache] = []
+        for i, (kv, st) in enumerate(zip(kv_specs, state_specs)):
+            owner = cache_of[i]
+            if owner is not None:
+                src = self.layers[owner]
+                if kv is not None and src.k is not None:
+                    okv = kv_specs[owner]
+                    if (okv.num_kv_heads, okv.head_dim) != (kv.num_kv_heads, kv.head_dim):
+                        raise ValueError(f"run order entry {i} reads the cache of entry {owner}, "
+                                         f"whose heads or head size differ")
+                self.layers.append(LayerCache(src.group, page_size, False, src.k, src.v, None))
+                continue
+            group, k, v = -1, None, None
+            if kv is not None:
+                if kv not in self.group_specs:
+                    self.group_specs.append(kv)
+                group = self.group_specs.index(kv)
+                k = torch.zeros((self.n_pages, kv.num_kv_heads, page_size, kv.head_dim), dtype=dtype, device=device)
+                v = torch.zeros((self.n_pages, kv.num_kv_heads, kv.head_dim, page_size), dtype=dtype, device=device)
+            state = None
+            if st is not None:
+                state = torch.zeros((n_slots,) + tuple(st.shape), dtype=st.dtype, device=device)
+            self.layers.append(LayerCache(group, page_size, True, k, v, state))
+
+    def bytes_per_token(self) -> int:
+        total = 0
+        for lc in self.layers:
+            if lc.owns and lc.k is not None:
+                total += 2 * lc.k.shape[1] * lc.k.shape[3] * lc.k.element_size()
+        return total

@@ -1,0 +1,259 @@
+// Element-wise and row-wise kernels of the forward pass, for float and bfloat16
+// storage: embedding gather, RMSNorm, rotary position encoding fused with the
+// write of keys and values into cache pages, SiLU-gate, residual add, fill.
+// All arithmetic is 32-bit float; only loads and stores see the storage type.
+#include "common.h"
+
+// ---------------------------------------------------------------- embedding
+// x[t] = table[id_t]; an id outside [0, V) reads row 0
+// (/root/reference/src/model.c:6148-6162).
+template <typename TW>
+__global__ void k_embedding(float* __restrict__ out, const TW* __restrict__ table,
+                            const int* __restrict__ ids, int E, int V, float scale) {
+    int t = blockIdx.x;
+    int id = ids[t];
+    if (id < 0 || id >= V) id = 0;
+    const TW* row = table + (size_t)id * E;
+    float* o = out + (size_t)t * E;
+    for (int i = threadIdx.x; i < E; i += blockDim.x) o[i] = ld<TW>(row, i) * scale;
+}
+
+extern "C" int xr_embedding(float* out, const void* table, const int* ids, int T, int E, int V,
+                            float scale, int table_dtype, hipStream_t stream) {
+    XR_REQUIRE(T >= 0 && E > 0 && V > 0, "embedding: bad sizes T=%d E=%d V=%d", T, E, V);
+    XR_REQUIRE(table_dtype == XR_F32 || table_dtype == XR_BF16, "embedding: bad dtype %d", table_dtype);
+    if (T == 0) return XR_OK;
+    if (table_dtype == XR_F32)
+        k_embedding<float><<<T, 256, 0, stream>>>(out, (const float*)table, ids, E, V, scale);
+    else
+        k_embedding<bf16_t><<<T, 256, 0, stream>>>(out, (const bf16_t*)table, ids, E, V, scale);
+    XR_CHECK_LAUNCH("embedding");
+    return XR_OK;
+}
+
+// ---------------------------------------------------------------- RMSNorm
+// y_i = x_i * r * w_i with r = 1/sqrt(mean(x^2) + eps): eps inside the root, added to
+// the mean; multiply order (x*r)*w (/root/reference/src/model.c:3386-3392).
+template <typename TO, typename TW>
+__global__ void k_rmsnorm(TO* __restrict__ out, const float* __restrict__ x, const TW* __restrict__ w,
+                          const int* __restrict__ rows, int E, int ldx, float eps) {
+    __shared__ float part[4];
+    int r = blockIdx.x;
+    int src = rows ? rows[r] : r;
+    const float* xr = x + (size_t)src * ldx;
+    float ss = 0.f;
+    for (int i = threadIdx.x; i < E; i += blockDim.x) {
+        float v = xr[i];
+        ss += v * v;
+    }
+    ss = wave_sum(ss);
+    int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    if (lane == 0) part[wave] = ss;
+    __syncthreads();
+    float tot = part[0] + part[1] + part[2] + part[3];
+    float rinv = 1.0f / sqrtf(tot / (float)E + eps);
+    TO* o = out + (size_t)r * E;
+    if (w) {
+        for (int i = threadIdx.x; i < E; i += blockDim.x) st<TO>(o, i, xr[i] * rinv * ld<TW>(w, i));
+    } else {
+        for (int i = threadIdx.x; i < E; i += blockDim.x) st<TO>(o, i, xr[i] * rinv);
+    }
+}
+
+extern "C" int xr_rmsnorm(void* out, const float* x, const void* w, const int* rows, int R, int E,
+                          int ldx, float eps, int out_dtype, int w_dtype, hipStream_t stream) {
+    XR_REQUIRE(R >= 0 && E > 0 && ldx >= E, "rmsnorm: bad sizes R=%d E=%d ldx=%d", R, E, ldx);
+    XR_REQUIRE(eps >= 0.f, "rmsnorm: eps %g is negative", eps);
+    if (R == 0) return XR_OK;
+#define RN(TO, TW) k_rmsnorm<TO, TW><<<R, 256, 0, stream>>>((TO*)out, x, (const TW*)w, rows, E, ldx, eps)
+    if (out_dtype == XR_F32 && w_dtype == XR_F32) RN(float, float);
+    else if (out_dtype == XR_F32 && w_dtype == XR_BF16) RN(float, bf16_t);
+    else if (out_dtype == XR_BF16 && w_dtype == XR_F32) RN(bf16_t, float);
+    else if (out_dtype == XR_BF16 && w_dtype == XR_BF16) RN(bf16_t, bf16_t);
+    else { xr_set_error("rmsnorm: bad dtypes out=%d w=%d", out_dtype, w_dtype); return XR_BAD_ARG; }
+#undef RN
+    XR_CHECK_LAUNCH("rmsnorm");
+    return XR_OK;
+}
+
+// ---------------------------------------------------------------- rotary + cache write
+// Rotation of pair index j of a head by a = pos * inv_freq[j]:
+//   (x0, x1) -> (x0*c - x1*s, x0*s + x1*c), c = cos(a)*mscale, s = sin(a)*mscale
+// (/root/reference/src/model.c:3514-3532).  Half-split pairs (j, j + rot/2) are what
+// un-permuted checkpoints need; interleaved pairs (2j, 2j+1) are the other option.
+// Keys are cached rotated, values as they are (/root/reference/src/model.c:6300-6311).
+// Cache layout per layer: K [page][kv_head][slot][d], V [page][kv_head][d][slot].
+struct RopeArgs {
+    const float* q_in;      // [T, in_stride] 32-bit
+    const float* k_in;
+    const float* v_in;
+    int in_stride;
+    void* q_out;            // [T, H*D] storage type
+    void* k_cache;
+    void* v_cache;
+    const int* positions;   // [T]
+    const int* req_of_token;// [T]
+    const int* block_table; // [B, table_stride]
+    int table_stride;
+    const float* inv_freq;  // [rot/2] or null
+    int H, Hk, D, rot, interleaved;
+    float mscale;
+    int page_shift, page_mask, page_size;
+};
+
+__device__ inline void rotate_pair(float x0, float x1, int pos, float f, float ms, float& y0, float& y1) {
+    float a = (float)pos * f;
+    float c = cosf(a) * ms, s = sinf(a) * ms;
+    y0 = x0 * c - x1 * s;
+    y1 = x0 * s + x1 * c;
+}
+
+template <typename T>
+__global__ void k_rope_kv_write(RopeArgs a) {
+    int t = blockIdx.x;
+    int hs = blockIdx.y;
+    int pos = a.positions[t];
+    int D = a.D, half = a.rot >> 1;
+    if (hs < a.H) {
+        const float* src = a.q_in + (size_t)t * a.in_stride + (size_t)hs * D;
+        T* dst = (T*)a.q_out + ((size_t)t * a.H + hs) * D;
+        for (int j = threadIdx.x; j < half; j += blockDim.x) {
+            int i0 = a.interleaved ? 2 * j : j;
+            int i1 = a.interleaved ? 2 * j + 1 : j + half;
+            float y0, y1;
+            rotate_pair(src[i0], src[i1], pos, a.inv_freq[j], a.mscale, y0, y1);
+            st<T>(dst, i0, y0);
+            st<T>(dst, i1, y1);
+        }
+        for (int i = a.rot + threadIdx.x; i < D; i += blockDim.x) st<T>(dst, i, src[i]);
+        return;
+    }
+    int kvh = hs - a.H;
+    int req = a.req_of_token[t];
+    PageRef pr = page_of(a.block_table, a.table_stride, req, pos, a.page_shift, a.page_mask);
+    const float* ks = a.k_in + (size_t)t * a.in_stride + (size_t)kvh * D;
+    const float* vs = a.v_in + (size_t)t * a.in_stride + (size_t)kvh * D;
+    T* kd = (T*)a.k_cache + (((size_t)pr.page * a.Hk + kvh) * a.page_size + pr.off) * D;
+    T* vd = (T*)a.v_cache + ((size_t)pr.page * a.Hk + kvh) * D * a.page_size + pr.off;
+    for (int j = threadIdx.x; j < half; j += blockDim.x) {
+        int i0 = a.interleaved ? 2 * j : j;
+        int i1 = a.interleaved ? 2 * j + 1 : j + half;
+        float y0, y1;
+        rotate_pair(ks[i0], ks[i1], pos, a.inv_freq[j], a.mscale, y0, y1);
+        st<T>(kd, i0, y0);
+        st<T>(kd, i1, y1);
+    }
+    for (int i = a.rot + threadIdx.x; i < D; i += blockDim.x) st<T>(kd, i, ks[i]);
+    for (int i = threadIdx.x; i < D; i += blockDim.x) st<T>(vd, (size_t)i * a.page_size, vs[i]);
+}
+
+extern "C" int xr_rope_kv_write(const float* q_in, const float* k_in, const float* v_in, int in_stride,
+                                void* q_out, void* k_cache, void* v_cache, const int* positions,
+                                const int* req_of_token, const int* block_table, int table_stride,
+                                const float* inv_freq, int T, int H, int Hk, int D, int rot,
+                                int interleaved, float mscale, int page_size, int dtype,
+                                hipStream_t stream) {
+    XR_REQUIRE(T >= 0 && H >= 0 && Hk >= 0 && D > 0, "rope_kv_write: bad sizes T=%d H=%d Hk=%d D=%d", T, H, Hk, D);
+    XR_REQUIRE(rot >= 0 && rot <= D && (rot % 2) == 0, "rope_kv_write: rotary width %d must be even and at most head_dim %d", rot, D);
+    XR_REQUIRE(rot == 0 || inv_freq, "rope_kv_write: rotary width %d without a frequency table", rot);
+    int shift = ilog2_exact(page_size);
+    XR_REQUIRE(Hk == 0 || shift >= 0, "rope_kv_write: page size %d is not a power of two", page_size);
+    XR_REQUIRE(Hk == 0 || (k_in && v_in && k_cache && v_cache && block_table && req_of_token),
+               "rope_kv_write: keys and values to cache but a null operand");
+    XR_REQUIRE(H == 0 || (q_in && q_out), "rope_kv_write: queries but a null operand");
+    XR_REQUIRE(dtype == XR_F32 || dtype == XR_BF16, "rope_kv_write: bad dtype %d", dtype);
+    if (T == 0 || H + Hk == 0) return XR_OK;
+    RopeArgs a;
+    a.q_in = q_in; a.k_in = k_in; a.v_in = v_in; a.in_stride = in_stride;
+    a.q_out = q_out; a.k_cache = k_cache; a.v_cache = v_cache;
+    a.positions = positions; a.req_of_token = req_of_token;
+    a.block_table = block_table; a.table_stride = table_stride; a.inv_freq = inv_freq;
+    a.H = H; a.Hk = Hk; a.D = D; a.rot = rot; a.interleaved = interleaved; a.mscale = mscale;
+    a.page_shift = shift < 0 ? 0 : shift; a.page_mask = page_size - 1; a.page_size = page_size;
+    dim3 grid(T, H + Hk);
+    if (dtype == XR_F32) k_rope_kv_write<float><<<grid, 64, 0, stream>>>(a);
+    else k_rope_kv_write<bf16_t><<<grid, 64, 0, stream>>>(a);
+    XR_CHECK_LAUNCH("rope_kv_write");
+    return XR_OK;
+}
+
+// ---------------------------------------------------------------- SiLU gate
+// h = silu(g) * u, silu(g) = g / (1 + exp(-g)) (/root/reference/src/model.c:4451-4452,
+// /root/reference/src/kernels.cu:2868-2874).  gu row = [gate(F) | up(F)].
+template <typename TI, typename TO>
+__global__ void k_silu_mul(TO* __restrict__ out, const TI* __restrict__ gu, int F, int ld_gu, size_t n) {
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    size_t t = i / F;
+    int c = (int)(i - t * F);
+    float g = ld<TI>(gu, t * ld_gu + c);
+    float u = ld<TI>(gu, t * ld_gu + F + c);
+    st<TO>(out, i, (g / (1.0f + expf(-g))) * u);
+}
+
+extern "C" int xr_silu_mul(void* out, const void* gu, int T, int F, int ld_gu, int dtype, hipStream_t stream) {
+    XR_REQUIRE(T >= 0 && F > 0 && ld_gu >= 2 * F, "silu_mul: bad sizes T=%d F=%d ld=%d", T, F, ld_gu);
+    size_t n = (size_t)T * F;
+    if (n == 0) return XR_OK;
+    unsigned blocks = (unsigned)((n + 255) / 256);
+    if (dtype == XR_F32) k_silu_mul<float, float><<<blocks, 256, 0, stream>>>((float*)out, (const float*)gu, F, ld_gu, n);
+    else if (dtype == XR_BF16) k_silu_mul<bf16_t, bf16_t><<<blocks, 256, 0, stream>>>((bf16_t*)out, (const bf16_t*)gu, F, ld_gu, n);
+    else { xr_set_error("silu_mul: bad dtype %d", dtype); return XR_BAD_ARG; }
+    XR_CHECK_LAUNCH("silu_mul");
+    return XR_OK;
+}
+
+// ---------------------------------------------------------------- residual add
+template <typename TY>
+__global__ void k_add(float* __restrict__ x, const TY* __restrict__ y, size_t n) {
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) x[i] = x[i] + ld<TY>(y, i);
+}
+
+extern "C" int xr_add(float* x, const void* y, size_t n, int y_dtype, hipStream_t stream) {
+    if (n == 0) return XR_OK;
+    unsigned blocks = (unsigned)((n + 255) / 256);
+    if (y_dtype == XR_F32) k_add<float><<<blocks, 256, 0, stream>>>(x, (const float*)y, n);
+    else if (y_dtype == XR_BF16) k_add<bf16_t><<<blocks, 256, 0, stream>>>(x, (const bf16_t*)y, n);
+    else { xr_set_error("add: bad dtype %d", y_dtype); return XR_BAD_ARG; }
+    XR_CHECK_LAUNCH("add");
+    return XR_OK;
+}
+
+// ---------------------------------------------------------------- fill (32-bit words)
+__global__ void k_fill_rows(uint32_t* __restrict__ base, const int* __restrict__ rows, size_t row_words,
+                            uint32_t value) {
+    int r = rows ? rows[blockIdx.y] : blockIdx.y;
+    if (r < 0) return;
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < row_words) base[(size_t)r * row_words + i] = value;
+}
+
+// Sets rows[r] (or rows 0..n_rows-1) of a [*, row_words] array of 32-bit words to `value`.
+extern "C" int xr_fill_rows(void* base, const int* rows, int n_rows, size_t row_words, uint32_t value,
+                            hipStream_t stream) {
+    if (n_rows <= 0 || row_words == 0) return XR_OK;
+    dim3 grid((unsigned)((row_words + 255) / 256), n_rows);
+    k_fill_rows<<<grid, 256, 0, stream>>>((uint32_t*)base, rows, row_words, value);
+    XR_CHECK_LAUNCH("fill_rows");
+    return XR_OK;
+}
+
+// ---------------------------------------------------------------- dtype conversion
+template <typename TI, typename TO>
+__global__ void k_convert(TO* __restrict__ out, const TI* __restrict__ in, size_t n) {
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) st<TO>(out, i, ld<TI>(in, i));
+}
+
+extern "C" int xr_convert(void* out, const void* in, size_t n, int in_dtype, int out_dtype, hipStream_t stream) {
+    if (n == 0) return XR_OK;
+    unsigned blocks = (unsigned)((n + 255) / 256);
+    if (in_dtype == XR_F32 && out_dtype == XR_BF16) k_convert<float, bf16_t><<<blocks, 256, 0, stream>>>((bf16_t*)out, (const float*)in, n);
+    else if (in_dtype == XR_BF16 && out_dtype == XR_F32) k_convert<bf16_t, float><<<blocks, 256, 0, stream>>>((float*)out, (const bf16_t*)in, n);
+    else if (in_dtype == XR_F32 && out_dtype == XR_F32) k_convert<float, float><<<blocks, 256, 0, stream>>>((float*)out, (const float*)in, n);
+    else if (in_dtype == XR_BF16 && out_dtype == XR_BF16) k_convert<bf16_t, bf16_t><<<blocks, 256, 0, stream>>>((bf16_t*)out, (const bf16_t*)in, n);
+    else { xr_set_error("convert: bad dtypes %d -> %d", in_dtype, out_dtype); return XR_BAD_ARG; }
+    XR_CHECK_LAUNCH("convert");
+    return XR_OK;
+}

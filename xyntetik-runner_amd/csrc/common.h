@@ -1,0 +1,99 @@
+// Shared declarations of the gfx950 kernel library.
+//
+// Every entry point is extern "C", takes raw device pointers and a HIP stream,
+// checks its operands on the host, launches, and returns 0 or a negative code;
+// xr_last_error() gives the text of the last failure on the calling thread.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+#include <stdarg.h>
+
+#define XR_OK 0
+#define XR_BAD_ARG -1
+#define XR_LAUNCH -2
+
+// dtype codes shared with the Python side
+#define XR_F32 0
+#define XR_BF16 1
+
+#define XR_WAVE 64
+
+typedef uint16_t bf16_t;   // storage only; arithmetic is float
+
+extern "C" const char* xr_last_error();
+void xr_set_error(const char* fmt, ...);
+
+#define XR_REQUIRE(cond, ...)                 \
+    do {                                      \
+        if (!(cond)) {                        \
+            xr_set_error(__VA_ARGS__);        \
+            return XR_BAD_ARG;                \
+        }                                     \
+    } while (0)
+
+#define XR_CHECK_LAUNCH(name)                                                   \
+    do {                                                                        \
+        hipError_t e_ = hipGetLastError();                                      \
+        if (e_ != hipSuccess) {                                                 \
+            xr_set_error("%s: launch failed: %s", name, hipGetErrorString(e_)); \
+            return XR_LAUNCH;                                                   \
+        }                                                                       \
+    } while (0)
+
+// ---- bfloat16 <-> float, round to nearest even --------------------------------
+__host__ __device__ inline float bf16_to_f32(bf16_t h) {
+    union { uint32_t u; float f; } c;
+    c.u = ((uint32_t)h) << 16;
+    return c.f;
+}
+
+__host__ __device__ inline bf16_t f32_to_bf16(float f) {
+    union { uint32_t u; float f; } c;
+    c.f = f;
+    uint32_t u = c.u;
+    if ((u & 0x7fffffffu) > 0x7f800000u) return (bf16_t)((u >> 16) | 0x0040u);   // NaN stays NaN
+    u += 0x7fffu + ((u >> 16) & 1u);
+    return (bf16_t)(u >> 16);
+}
+
+template <typename T> __device__ inline float ld(const T* p, size_t i);
+template <> __device__ inline float ld<float>(const float* p, size_t i) { return p[i]; }
+template <> __device__ inline float ld<bf16_t>(const bf16_t* p, size_t i) { return bf16_to_f32(p[i]); }
+
+template <typename T> __device__ inline void st(T* p, size_t i, float v);
+template <> __device__ inline void st<float>(float* p, size_t i, float v) { p[i] = v; }
+template <> __device__ inline void st<bf16_t>(bf16_t* p, size_t i, float v) { p[i] = f32_to_bf16(v); }
+
+// ---- wave (64 lanes) reductions -------------------------------------------------
+__device__ inline float wave_sum(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+    return v;
+}
+__device__ inline float wave_max(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+    return v;
+}
+
+// Page lookup: logical position of a request -> element offset pieces.
+struct PageRef {
+    int page;
+    int off;
+};
+__device__ inline PageRef page_of(const int* __restrict__ block_table, int table_stride, int req,
+                                  int pos, int page_shift, int page_mask) {
+    PageRef r;
+    r.page = block_table[(size_t)req * table_stride + (pos >> page_shift)];
+    r.off = pos & page_mask;
+    return r;
+}
+
+static inline int ilog2_exact(int v) {   // -1 if v is not a power of two
+    if (v <= 0 || (v & (v - 1))) return -1;
+    int s = 0;
+    while ((1 << s) < v) ++s;
+    return s;
+}

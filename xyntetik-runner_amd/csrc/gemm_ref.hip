@@ -1,0 +1,84 @@
+// Plain matrix product out[M,N] = a[M,K] * w[N,K]^T (+ bias) with 32-bit FMA only:
+// the matrix product of the true 32-bit path, and the yardstick of the MFMA kernels.
+// Weights are [n_out][n_in] row-major as the reference keeps them
+// (/root/reference/src/model.c:193-205); each output is a sum over k in ascending
+// order, whatever the batch, so a row's result does not depend on its neighbours.
+#include "common.h"
+
+#define RBM 64
+#define RBN 64
+#define RBK 16
+
+template <typename TI, typename TO, bool ACC>
+__global__ __launch_bounds__(256) void k_gemm_ref(TO* __restrict__ out, const TI* __restrict__ a,
+                                                   const TI* __restrict__ w, const float* __restrict__ bias,
+                                                   int M, int N, int K, int lda, int ldo) {
+    __shared__ float As[RBK][RBM + 4];
+    __shared__ float Ws[RBK][RBN + 4];
+    int m0 = blockIdx.y * RBM, n0 = blockIdx.x * RBN;
+    int tx = threadIdx.x & 15, ty = threadIdx.x >> 4;
+    float acc[4][4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[i][j] = 0.f;
+
+    for (int k0 = 0; k0 < K; k0 += RBK) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            int idx = threadIdx.x + e * 256;
+            int r = idx >> 4, kk = idx & 15;
+            int gm = m0 + r, gn = n0 + r, gk = k0 + kk;
+            As[kk][r] = (gm < M && gk < K) ? ld<TI>(a, (size_t)gm * lda + gk) : 0.f;
+            Ws[kk][r] = (gn < N && gk < K) ? ld<TI>(w, (size_t)gn * K + gk) : 0.f;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int kk = 0; kk < RBK; ++kk) {
+            float av[4], wv[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) av[i] = As[kk][ty * 4 + i];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) wv[j] = Ws[kk][tx * 4 + j];
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) acc[i][j] = fmaf(av[i], wv[j], acc[i][j]);
+        }
+        __syncthreads();
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        int gm = m0 + ty * 4 + i;
+        if (gm >= M) continue;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            int gn = n0 + tx * 4 + j;
+            if (gn >= N) continue;
+            float v = acc[i][j];
+            if (bias) v += bias[gn];
+            size_t o = (size_t)gm * ldo + gn;
+            if (ACC) v += ld<TO>(out, o);
+            st<TO>(out, o, v);
+        }
+    }
+}
+
+// accumulate != 0: out (float) += product.
+extern "C" int xr_gemm_ref(void* out, const void* a, const void* w, const float* bias, int M, int N, int K,
+                           int lda, int ldo, int in_dtype, int out_dtype, int accumulate, hipStream_t stream) {
+    XR_REQUIRE(M >= 0 && N > 0 && K > 0, "gemm: bad sizes M=%d N=%d K=%d", M, N, K);
+    XR_REQUIRE(lda >= K && ldo >= N, "gemm: row strides lda=%d ldo=%d are shorter than K=%d N=%d", lda, ldo, K, N);
+    XR_REQUIRE(!accumulate || out_dtype == XR_F32, "gemm: accumulation needs a 32-bit output");
+    if (M == 0) return XR_OK;
+    dim3 grid((N + RBN - 1) / RBN, (M + RBM - 1) / RBM);
+#define G(TI, TO, ACC) k_gemm_ref<TI, TO, ACC><<<grid, 256, 0, stream>>>((TO*)out, (const TI*)a, (const TI*)w, bias, M, N, K, lda, ldo)
+    if (in_dtype == XR_F32 && out_dtype == XR_F32) { if (accumulate) G(float, float, true); else G(float, float, false); }
+    else if (in_dtype == XR_BF16 && out_dtype == XR_F32) { if (accumulate) G(bf16_t, float, true); else G(bf16_t, float, false); }
+    else if (in_dtype == XR_BF16 && out_dtype == XR_BF16) G(bf16_t, bf16_t, false);
+    else if (in_dtype == XR_F32 && out_dtype == XR_BF16) G(float, bf16_t, false);
+    else { xr_set_error("gemm: bad dtypes in=%d out=%d", in_dtype, out_dtype); return XR_BAD_ARG; }
+#undef G
+    XR_CHECK_LAUNCH("gemm_ref");
+    return XR_OK;
+}

@@ -1,0 +1,258 @@
+"""The kernels as Python calls on torch tensors.
+
+``load_ops()`` loads the compiled library (building it first if no up-to-date one
+exists) and fails loudly when that is impossible: there is no fallback.  Each
+method checks what only the Python side can know (device, dtype, contiguity), hands
+raw pointers and the current HIP stream to the entry point, and raises
+``KernelError`` with the library's message when it refuses its operands.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import threading
+from typing import Dict, Optional
+
+import torch
+
+from . import build as _build
+
+XR_F32, XR_BF16 = 0, 1
+_CODE = {torch.float32: XR_F32, torch.bfloat16: XR_BF16}
+
+
+class KernelError(RuntimeError):
+    pass
+
+
+def dtype_code(dt: torch.dtype) -> int:
+    try:
+        return _CODE[dt]
+    except KeyError:
+        raise KernelError(f"kernels take float32 or bfloat16, not {dt}") from None
+
+
+_p, _i, _f, _sz, _u32 = C.c_void_p, C.c_int, C.c_float, C.c_size_t, C.c_uint32
+
+_PROTOS = {
+    "xr_embedding": [_p, _p, _p, _i, _i, _i, _f, _i, _p],
+    "xr_rmsnorm": [_p, _p, _p, _p, _i, _i, _i, _f, _i, _i, _p],
+    "xr_rope_kv_write": [_p, _p, _p, _i, _p, _p, _p, _p, _p, _p, _i, _p, _i, _i, _i, _i, _i, _i, _f, _i, _i, _p],
+    "xr_silu_mul": [_p, _p, _i, _i, _i, _i, _p],
+    "xr_add": [_p, _p, _sz, _i, _p],
+    "xr_fill_rows": [_p, _p, _i, _sz, _u32, _p],
+    "xr_convert": [_p, _p, _sz, _i, _i, _p],
+    "xr_gemm_ref": [_p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _p],
+    "xr_attention_ref": [_p, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _f, _i, _i, _p],
+    "xr_sample": [_p, _p, _i, _i, _i, _p, _p, _p, _p, _p, _p, _p, _p, _i, _p, _i, _p],
+}
+
+
+def _ptr(t: Optional[torch.Tensor]) -> Optional[int]:
+    return None if t is None else t.data_ptr()
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+class _Lib:
+    def __init__(self, path: str, protos: Dict[str, list]):
+        self.path = path
+        self.dll = C.CDLL(path)
+        self.dll.xr_last_error.restype = C.c_char_p
+        self.dll.xr_last_error.argtypes = []
+        for name, args in protos.items():
+            fn = getattr(self.dll, name)
+            fn.argtypes = args
+            fn.restype = C.c_int
+            setattr(self, name, fn)
+
+    def check(self, rc: int) -> None:
+        if rc != 0:
+            raise KernelError(self.dll.xr_last_error().decode("utf-8", "replace"))
+
+
+class Ops:
+    """All kernels of the forward pass and of sampling."""
+
+    def __init__(self, lib: _Lib):
+        self.lib = lib
+        self._attn_libs: Dict[int, object] = {}
+        self.use_mfma = True
+
+    # -- checks -----------------------------------------------------------------
+    @staticmethod
+    def _dev(*ts: Optional[torch.Tensor]) -> None:
+        for t in ts:
+            if t is not None and not t.is_cuda:
+                raise KernelError("kernel operand is not on the GPU (there is no CPU path)")
+
+    @staticmethod
+    def _contig(t: torch.Tensor, what: str) -> None:
+        if not t.is_contiguous():
+            raise KernelError(f"{what} must be contiguous")
+
+    # -- element-wise and row-wise ----------------------------------------------
+    def embedding(self, table: torch.Tensor, ids: torch.Tensor, scale: float = 1.0) -> torch.Tensor:
+        """``out[t] = table[ids[t]] * scale`` as 32-bit rows."""
+        self._dev(table, ids)
+        self._contig(table, "embedding table")
+        T, (V, E) = ids.numel(), table.shape
+        out = torch.empty((T, E), dtype=torch.float32, device=table.device)
+        self.lib.check(self.lib.xr_embedding(out.data_ptr(), table.data_ptr(), ids.data_ptr(), T, E, V,
+                                             float(scale), dtype_code(table.dtype), _stream()))
+        return out
+
+    def rmsnorm(self, x: torch.Tensor, w: Optional[torch.Tensor], eps: float, out_dtype: torch.dtype,
+                rows: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """RMSNorm of the rows of 32-bit ``x`` (or of the rows ``rows`` selects)."""
+        self._dev(x, w, rows)
+        if x.dtype != torch.float32 or x.dim() != 2 or x.stride(1) != 1:
+            raise KernelError("rmsnorm input must be float32 [rows, width] with unit column stride")
+        E = x.shape[1]
+        if w is not None and (w.numel() != E or not w.is_contiguous()):
+            raise KernelError(f"rmsnorm weight has {w.numel()} elements, the row has {E}")
+        R = x.shape[0] if rows is None else rows.numel()
+        out = torch.empty((R, E), dtype=out_dtype, device=x.device)
+        self.lib.check(self.lib.xr_rmsnorm(out.data_ptr(), x.data_ptr(), _ptr(w), _ptr(rows), R, E, x.stride(0),
+                                           float(eps), dtype_code(out_dtype),
+                                           dtype_code(w.dtype) if w is not None else XR_F32, _stream()))
+        return out
+
+    def silu_mul(self, gu: torch.Tensor) -> torch.Tensor:
+        """``silu(gu[:, :F]) * gu[:, F:]``."""
+        self._dev(gu)
+        T, F2 = gu.shape
+        F = F2 // 2
+        if gu.stride(1) != 1 or F2 % 2:
+            raise KernelError("silu_mul input must be [rows, 2F] with unit column stride")
+        out = torch.empty((T, F), dtype=gu.dtype, device=gu.device)
+        self.lib.check(self.lib.xr_silu_mul(out.data_ptr(), gu.data_ptr(), T, F, gu.stride(0),
+                                            dtype_code(gu.dtype), _stream()))
+        return out
+
+    def add_(self, x: torch.Tensor, y: torch.Tensor) -> None:
+        """``x += y`` with 32-bit ``x``."""
+        self._dev(x, y)
+        if x.dtype != torch.float32 or x.shape != y.shape:
+            raise KernelError(f"add_: x must be float32 and shapes equal, got {x.dtype} {tuple(x.shape)} {tuple(y.shape)}")
+        self._contig(x, "add_ x")
+        self._contig(y, "add_ y")
+        self.lib.check(self.lib.xr_add(x.data_ptr(), y.data_ptr(), x.numel(), dtype_code(y.dtype), _stream()))
+
+    def fill_rows_(self, base: torch.Tensor, rows: Optional[torch.Tensor], n_rows: int, value_bits: int = 0) -> None:
+        """Set whole rows of ``base`` (first axis) to a 32-bit pattern."""
+        self._dev(base, rows)
+        self._contig(base, "fill_rows_ base")
+        row_bytes = base[0].numel() * base.element_size()
+        if row_bytes % 4:
+            raise KernelError("fill_rows_: a row must be a multiple of 4 bytes")
+        self.lib.check(self.lib.xr_fill_rows(base.data_ptr(), _ptr(rows), int(n_rows), row_bytes // 4,
+                                             value_bits & 0xFFFFFFFF, _stream()))
+
+    def convert(self, x: torch.Tensor, dtype: torch.dtype) -> torch.Tensor:
+        self._dev(x)
+        self._contig(x, "convert input")
+        out = torch.empty(x.shape, dtype=dtype, device=x.device)
+        self.lib.check(self.lib.xr_convert(out.data_ptr(), x.data_ptr(), x.numel(), dtype_code(x.dtype),
+                                           dtype_code(dtype), _stream()))
+        return out
+
+    # -- matrix product ---------------------------------------------------------
+    def linear(self, a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None,
+               out_dtype: Optional[torch.dtype] = None, out: Optional[torch.Tensor] = None,
+               accumulate: bool = False) -> torch.Tensor:
+        """``a [M, K] @ w [N, K]^T (+ bias)``; with ``accumulate`` added into 32-bit ``out``."""
+        self._dev(a, w, bias, out)
+        if a.dim() != 2 or w.dim() != 2 or a.shape[1] != w.shape[1]:
+            raise KernelError(f"linear: shapes {tuple(a.shape)} x {tuple(w.shape)}^T do not fit")
+        if a.dtype != w.dtype:
+            raise KernelError(f"linear: input is {a.dtype}, weight is {w.dtype}")
+        if a.stride(1) != 1:
+            raise KernelError("linear: input must have unit column stride")
+        self._contig(w, "linear weight")
+        M, K = a.shape
+        N = w.shape[0]
+        if out is None:
+            if accumulate:
+                raise KernelError("linear: accumulate needs an output")
+            out = torch.empty((M, N), dtype=out_dtype or a.dtype, device=a.device)
+        elif out.shape != (M, N) or out.stride(1) != 1:
+            raise KernelError(f"linear: output is {tuple(out.shape)}, product is {(M, N)}")
+        if bias is not None and (bias.dtype != torch.float32 or bias.numel() != N):
+            raise KernelError("linear: bias must be float32 [N]")
+        self.lib.check(self.lib.xr_gemm_ref(out.data_ptr(), a.data_ptr(), w.data_ptr(), _ptr(bias), M, N, K,
+                                            a.stride(0), out.stride(0), dtype_code(a.dtype),
+                                            dtype_code(out.dtype), 1 if accumulate else 0, _stream()))
+        return out
+
+    # -- attention --------------------------------------------------------------
+    def rope_kv_write(self, q_in, k_in, v_in, q_out, k_cache, v_cache, positions, req_of_token,
+                      block_table, inv_freq, H: int, Hk: int, D: int, rot: int, interleaved: bool,
+                      mscale: float, page_size: int) -> None:
+        """Rotate queries (into ``q_out``) and keys, and write keys and values to their pages.
+
+        ``q_in``/``k_in``/``v_in`` are 32-bit views with one common row stride.
+        """
+        self._dev(q_in, k_in, v_in, q_out, k_cache, v_cache, positions, req_of_token, block_table, inv_freq)
+        T = positions.numel()
+        ins = [t for t in (q_in, k_in, v_in) if t is not None]
+        if any(t.dtype != torch.float32 or t.stride(-1) != 1 for t in ins):
+            raise KernelError("rope_kv_write: inputs must be float32 with unit column stride")
+        strides = {t.stride(0) for t in ins}
+        if len(strides) > 1:
+            raise KernelError("rope_kv_write: q, k and v inputs must share a row stride")
+        stride = strides.pop() if strides else 0
+        store = q_out if q_out is not None else k_cache
+        if k_cache is not None and q_out is not None and k_cache.dtype != q_out.dtype:
+            raise KernelError("rope_kv_write: query output and cache differ in dtype")
+        self.lib.check(self.lib.xr_rope_kv_write(
+            _ptr(q_in), _ptr(k_in), _ptr(v_in), stride, _ptr(q_out), _ptr(k_cache), _ptr(v_cache),
+            positions.data_ptr(), _ptr(req_of_token), _ptr(block_table),
+            block_table.stride(0) if block_table is not None else 0, _ptr(inv_freq), T, H, Hk, D, rot,
+            1 if interleaved else 0, float(mscale), page_size, dtype_code(store.dtype), _stream()))
+
+    def attention(self, q, k_cache, v_cache, positions, req_of_token, block_table, H: int, Hk: int,
+                  D: int, page_size: int, scale: float, window: Optional[int] = None) -> torch.Tensor:
+        """Causal attention of every token over its request's cached keys and values."""
+        self._dev(q, k_cache, v_cache, positions, req_of_token, block_table)
+        T = positions.numel()
+        self._contig(q, "attention queries")
+        if q.dtype != k_cache.dtype or q.dtype != v_cache.dtype:
+            raise KernelError("attention: queries and cache differ in dtype")
+        out = torch.empty((T, H * D), dtype=q.dtype, device=q.device)
+        self.lib.check(self.lib.xr_attention_ref(
+            out.data_ptr(), q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), positions.data_ptr(),
+            req_of_token.data_ptr(), block_table.data_ptr(), block_table.stride(0), T, H, Hk, D, page_size,
+            float(scale), int(window or 0), dtype_code(q.dtype), _stream()))
+        return out
+
+    # -- sampling ---------------------------------------------------------------
+    def sample(self, logits, temp, draw, top_k=None, top_p=None, min_p=None, repeat_penalty=None,
+               recent=None, n_recent=None, exempt=None) -> torch.Tensor:
+        """One token id per row of 32-bit ``logits`` (rows with a penalty are changed in place)."""
+        self._dev(logits, temp, draw, top_k, top_p, min_p, repeat_penalty, recent, n_recent, exempt)
+        if logits.dtype != torch.float32 or logits.dim() != 2 or logits.stride(1) != 1:
+            raise KernelError("sample: logits must be float32 [rows, vocab]")
+        W, V = logits.shape
+        out = torch.empty((W,), dtype=torch.int32, device=logits.device)
+        self.lib.check(self.lib.xr_sample(
+            out.data_ptr(), logits.data_ptr(), W, V, logits.stride(0), temp.data_ptr(), _ptr(top_k),
+            _ptr(top_p), _ptr(min_p), _ptr(repeat_penalty), draw.data_ptr(), _ptr(recent), _ptr(n_recent),
+            recent.shape[1] if recent is not None else 0, _ptr(exempt),
+            exempt.numel() if exempt is not None else 0, _stream()))
+        return out
+
+
+_LOCK = threading.Lock()
+_OPS: Optional[Ops] = None
+
+
+def load_ops() -> Ops:
+    """The kernel library, loaded once per process (compiled first if it must be)."""
+    global _OPS
+    with _LOCK:
+        if _OPS is None:
+            path = _build.find_built("kernels") or _build.build_unit("kernels")
+            _OPS = Ops(_Lib(path, _PROTOS))
+        return _OPS

@@ -1,0 +1,101 @@
+"""One step's batch as the kernels see it.
+
+A step is a list of entries (request, its next tokens, the places whose logits are
+wanted).  All tokens of all entries are laid out one after another ("rows"); per
+row the device gets its token id, its position in its request and the index of its
+request in this batch; per request and cache group the block table.  One pinned
+host buffer carries all of it to the device in a single copy.
+
+The reference has two narrower primitives, n consecutive tokens of one sequence
+(/root/reference/src/model.h:667-670) and one token each of up to 8 sequences with
+per-column position and cache pointers (/root/reference/src/model.h:796-807,
+/root/reference/src/cuda.c:4213-4236); an entry list covers both and their mixtures.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Hashable, List, Optional, Sequence
+
+import numpy as np
+import torch
+
+
+@dataclass
+class StepEntry:
+    req_id: Hashable
+    tokens: Sequence[int]
+    want: Sequence[int] = ()        # indices into ``tokens`` whose logits are wanted
+
+
+class StepContext:
+    """Device views of one step's metadata, handed to every part."""
+
+    def __init__(self, ops, device, entries: List[StepEntry], request_caches, n_groups: int, pad_to: int = 0):
+        self.ops = ops
+        self.device = device
+        self.entries = entries
+        B = len(entries)
+        q_lens = [len(e.tokens) for e in entries]
+        T = sum(q_lens)
+        self.B, self.T = B, T
+        self.q_lens = q_lens
+        self.starts = [rc.n_tokens for rc in request_caches]            # position of each entry's first token
+        self.seq_lens = [s + n for s, n in zip(self.starts, q_lens)]    # length after this step
+        self.max_q_len = max(q_lens) if q_lens else 0
+        self.max_seq_len = max(self.seq_lens) if B else 0
+        nb = [max((len(rc.tables[g]) for rc in request_caches), default=0) for g in range(n_groups)]
+        self.table_width = [max(1, w) for w in nb]
+        want_rows: List[int] = []
+        row0 = 0
+        for e, n in zip(entries, q_lens):
+            for w in e.want:
+                if not (0 <= w < n):
+                    raise ValueError(f"request {e.req_id!r}: wanted place {w} is outside its {n} tokens")
+                want_rows.append(row0 + w)
+            row0 += n
+        self.n_want = len(want_rows)
+
+        # ---- pack: [token_ids T][positions T][req_of_token T][cu_q B+1][seq_lens B][slots B][fresh B]
+        #            [want W][table g: B * width_g]...
+        sizes = [T, T, T, B + 1, B, B, B, self.n_want] + [B * w for w in self.table_width]
+        offs = np.concatenate([[0], np.cumsum(sizes)]).astype(np.int64)
+        total = int(offs[-1])
+        host = torch.empty((max(total, 1),), dtype=torch.int32, pin_memory=True)
+        h = host.numpy()
+        tok, pos, rot = h[offs[0]:offs[1]], h[offs[1]:offs[2]], h[offs[2]:offs[3]]
+        cu = h[offs[3]:offs[4]]
+        cu[0] = 0
+        r = 0
+        for b, (e, n) in enumerate(zip(entries, q_lens)):
+            tok[r:r + n] = np.asarray(e.tokens, dtype=np.int64).astype(np.int32)
+            pos[r:r + n] = np.arange(self.starts[b], self.starts[b] + n, dtype=np.int32)
+            rot[r:r + n] = b
+            r += n
+            cu[b + 1] = r
+        h[offs[4]:offs[5]] = self.seq_lens
+        h[offs[5]:offs[6]] = [rc.slot for rc in request_caches]
+        h[offs[6]:offs[7]] = [1 if rc.fresh else 0 for rc in request_caches]
+        h[offs[7]:offs[8]] = want_rows
+        for g in range(n_groups):
+            w = self.table_width[g]
+            tab = h[offs[8 + g]:offs[9 + g]].reshape(B, w)
+            tab[:] = -1
+            for b, rc in enumerate(request_caches):
+                t = rc.tables[g]
+                tab[b, :len(t)] = t
+        dev = host.to(device, non_blocking=True)
+        self._host = host      # keep the pinned buffer alive until the copy has run
+        self.token_ids = dev[offs[0]:offs[1]]
+        self.positions = dev[offs[1]:offs[2]]
+        self.req_of_token = dev[offs[2]:offs[3]]
+        self.cu_q = dev[offs[3]:offs[4]]
+        self.seq_lens_dev = dev[offs[4]:offs[5]]
+        self.slots = dev[offs[5]:offs[6]]
+        self.fresh = dev[offs[6]:offs[7]]
+        self.want_rows = dev[offs[7]:offs[8]]
+        self._tables = [dev[offs[8 + g]:offs[9 + g]].view(B, self.table_width[g]) for g in range(n_groups)]
+        self.fresh_slots_host = [rc.slot for rc in request_caches if rc.fresh]
+
+    def block_table(self, group: int) -> torch.Tensor:
+        """``[B, width]`` int32: page of each block of each request of this step, -1 where none."""
+        return self._tables[group]

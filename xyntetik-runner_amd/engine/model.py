@@ -1,0 +1,89 @@
+"""A model: the parts of a ``ModelSpec``, built, bound to their tensors, and run.
+
+The forward pass is the reference's, step by step
+(/root/reference/src/model.c:6148-6483): embedding, the layers in their run order,
+then final norm and output head on the rows whose logits are wanted only
+(:6478-6481).
+"""
+from __future__ import annotations
+
+from typing import Dict, List, Optional
+
+import torch
+
+from ..config import ModelSpec
+from ..parts.base import Block, ParamSpec, Runtime, make_block, make_part
+
+
+class Model:
+    def __init__(self, spec: ModelSpec):
+        spec.validate()
+        self.spec = spec
+        self.embedding = make_part("embedding", spec.embedding)
+        self.blocks: List[Block] = []
+        for ls in spec.layers:
+            self.blocks.append(make_block(
+                ls.block, make_part("norm", ls.mixer_norm), make_part("mixer", ls.mixer),
+                make_part("norm", ls.feed_forward_norm), make_part("feed_forward", ls.feed_forward)))
+        self.final_norm = make_part("norm", spec.final_norm)
+        self.head = make_part("head", spec.head)
+        self.rt: Optional[Runtime] = None
+
+    # ------------------------------------------------------------------ tensors
+    def _named_parts(self):
+        yield self.spec.embedding.prefix, self.embedding
+        for ls, blk in zip(self.spec.layers, self.blocks):
+            yield ls.mixer_norm.prefix, blk.mixer_norm
+            yield ls.mixer.prefix, blk.mixer
+            yield ls.feed_forward_norm.prefix, blk.feed_forward_norm
+            yield ls.feed_forward.prefix, blk.feed_forward
+        yield self.spec.final_norm.prefix, self.final_norm
+        yield self.spec.head.prefix, self.head
+
+    def expected(self) -> Dict[str, ParamSpec]:
+        out: Dict[str, ParamSpec] = {}
+        for prefix, part in self._named_parts():
+            for rel, ps in part.param_specs().items():
+                name = prefix + rel
+                if name in out:
+                    raise ValueError(f"two parts claim the tensor {name}")
+                out[name] = ps
+        return out
+
+    @staticmethod
+    def expected_tensors(spec: ModelSpec) -> Dict[str, ParamSpec]:
+        return Model(spec).expected()
+
+    def bind(self, tensors: Dict[str, torch.Tensor], rt: Runtime) -> None:
+        """Give every part its tensors (``tensors`` is emptied as parts take theirs)."""
+        self.rt = rt
+        for prefix, part in self._named_parts():
+            mine = {rel: tensors.pop(prefix + rel) for rel in part.param_specs() if prefix + rel in tensors}
+            if part is self.head:
+                part.bind(mine, rt, tied_to=getattr(self.embedding, "weight", None))
+            else:
+                part.bind(mine, rt)
+
+    # ------------------------------------------------------------------ what the cache must hold
+    def cache_needs(self):
+        """Per entry of the run order: (KVSpec or None, StateSpec or None, cache_of)."""
+        kv, st, of = [], [], []
+        for step in self.spec.order:
+            mixer = self.blocks[step.layer].mixer
+            kv.append(mixer.kv_spec())
+            st.append(mixer.state_spec() if step.cache_of is None else None)
+            of.append(step.cache_of)
+        return kv, st, of
+
+    # ------------------------------------------------------------------ forward
+    def forward(self, ctx, caches) -> torch.Tensor:
+        """Run the step's tokens through every layer; returns the residual stream ``[T, E]`` (32-bit)."""
+        x = self.embedding.forward(ctx, ctx.token_ids)
+        for i, step in enumerate(self.spec.order):
+            self.blocks[step.layer].forward(ctx, caches[i], x)
+        return x
+
+    def logits(self, ctx, x: torch.Tensor, rows: torch.Tensor) -> torch.Tensor:
+        """32-bit logits ``[len(rows), V]`` of the rows ``rows`` of ``x``."""
+        h = self.final_norm.forward(ctx, x, rows=rows)
+        return self.head.forward(ctx, h)

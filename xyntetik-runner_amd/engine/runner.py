@@ -1,0 +1,128 @@
+"""The step function: run a batch of (request, its next tokens) from the cache.
+
+``ModelRunner.step`` takes entries cut anywhere: portions of prompts beside single
+decoded tokens.  It reserves pages, runs only the tokens it is given as one batch,
+records that the requests have grown, and returns 32-bit logits at the wanted
+places, in the order of the entries and of each entry's ``want``.
+"""
+from __future__ import annotations
+
+import os
+from typing import Dict, Hashable, List, Optional, Sequence
+
+import torch
+
+from ..cache import CacheManager, CacheStorage, OutOfPages
+from ..config import ModelSpec, load_config
+from ..csrc.ops import load_ops
+from ..parts.base import Runtime
+from ..weights import SafetensorsStore, load_state, load_tensors
+from .batch import StepContext, StepEntry
+from .model import Model
+
+_DTYPES = {"float32": torch.float32, "fp32": torch.float32, "bfloat16": torch.bfloat16, "bf16": torch.bfloat16}
+
+
+def parse_dtype(name) -> torch.dtype:
+    if isinstance(name, torch.dtype):
+        if name not in (torch.float32, torch.bfloat16):
+            raise ValueError(f"the engine runs in float32 or bfloat16, not {name}")
+        return name
+    try:
+        return _DTYPES[str(name)]
+    except KeyError:
+        raise ValueError(f"dtype {name!r}: expected bfloat16 or float32") from None
+
+
+class ModelRunner:
+    def __init__(self, spec: ModelSpec, tensors_or_store, dtype, max_tokens: int, page_size: int = 64,
+                 max_requests: int = 64, device: str = "cuda:0"):
+        if not torch.cuda.is_available():
+            raise RuntimeError("no GPU: this engine runs on an MI355X only and has no CPU path")
+        self.device = torch.device(device)
+        torch.cuda.set_device(self.device)
+        self.dtype = parse_dtype(dtype)
+        self.spec = spec
+        self.ops = load_ops()
+        self.rt = Runtime(self.device, self.dtype, self.ops)
+        self.model = Model(spec)
+        expected = self.model.expected()
+        if isinstance(tensors_or_store, SafetensorsStore):
+            tensors = load_tensors(tensors_or_store, expected, self.dtype, self.device)
+        else:
+            tensors = load_state(tensors_or_store, expected, self.dtype, self.device)
+        self.model.bind(tensors, self.rt)
+        del tensors
+        kv, st, of = self.model.cache_needs()
+        pages = max(1, -(-int(max_tokens) // page_size))
+        self.page_size = page_size
+        self.storage = CacheStorage(kv, st, of, page_size, pages, max_requests, self.dtype, self.device)
+        self.manager = CacheManager(self.storage.group_specs, page_size, pages, max_requests)
+        self.vocab_size = spec.vocab_size
+
+    @classmethod
+    def from_folder(cls, model_dir: str, dtype="bfloat16", **kw) -> "ModelRunner":
+        arch, cfg = load_config(model_dir)
+        spec = arch.build_spec(cfg)
+        store = SafetensorsStore.open_folder(model_dir)
+        try:
+            return cls(spec, store, dtype, **kw)
+        finally:
+            store.close()
+
+    # ------------------------------------------------------------------ requests
+    def has(self, req_id: Hashable) -> bool:
+        return req_id in self.manager.requests
+
+    def start(self, req_id: Hashable) -> None:
+        self.manager.admit(req_id)
+
+    def finish(self, req_id: Hashable) -> None:
+        self.manager.release(req_id)
+
+    def length(self, req_id: Hashable) -> int:
+        return self.manager.get(req_id).n_tokens
+
+    # ------------------------------------------------------------------ the step
+    def step(self, entries: Sequence[StepEntry]) -> Optional[torch.Tensor]:
+        """Run ``entries`` as one batch; logits ``[wanted, V]`` float32 on the device (None if nothing is wanted)."""
+        entries = [e for e in entries if len(e.tokens) > 0]
+        if not entries:
+            return None
+        seen = set()
+        for e in entries:
+            if e.req_id in seen:
+                raise ValueError(f"request {e.req_id!r} appears twice in one step")
+            seen.add(e.req_id)
+            if not self.has(e.req_id):
+                self.start(e.req_id)
+        mgr = self.manager
+        rcs = [mgr.get(e.req_id) for e in entries]
+        # reserve for all or for none
+        spare = [0] * len(mgr.groups)
+        for e, rc in zip(entries, rcs):
+            need = mgr.pages_needed(e.req_id, rc.n_tokens + len(e.tokens))
+            spare = [s + n for s, n in zip(spare, need)]
+        for gi, g in enumerate(mgr.groups):
+            if spare[gi] > g.pool.n_free:
+                raise OutOfPages(f"this step needs {spare[gi]} new pages in group {gi}, {g.pool.n_free} of {g.pool.size} are free")
+        for e, rc in zip(entries, rcs):
+            mgr.reserve(e.req_id, rc.n_tokens + len(e.tokens))
+        ctx = StepContext(self.ops, self.device, entries, rcs, len(mgr.groups))
+        self._zero_fresh_state(ctx)
+        x = self.model.forward(ctx, self.storage.layers)
+        out = self.model.logits(ctx, x, ctx.want_rows) if ctx.n_want else None
+        for e, rc in zip(entries, rcs):
+            mgr.advance(e.req_id, rc.n_tokens + len(e.tokens))
+        return out
+
+    def _zero_fresh_state(self, ctx: StepContext) -> None:
+        if not ctx.fresh_slots_host:
+            return
+        rows = None
+        for lc in self.storage.layers:
+            if lc.state is None:
+                continue
+            if rows is None:
+                rows = torch.tensor(ctx.fresh_slots_host, dtype=torch.int32, device=self.device)
+            self.ops.fill_rows_(lc.state, rows, len(ctx.fresh_slots_host), 0)

@@ -1,0 +1,114 @@
+"""Grouped-query attention over the paged cache.
+
+Per token: ``q = Wq h``, ``k = Wk h``, ``v = Wv h`` (optional biases); the position
+encoding rotates q and k; k and v go to the cache (k rotated, v as it is); query head
+``h`` reads key/value head ``h // (H / Hk)``; scores are ``(q . k) * scale`` with
+``scale = 1/sqrt(head_dim)`` unless given, causal by construction, limited to the last
+``window`` keys if the layer has a window; softmax in 32-bit; ``a = Wo o``
+(/root/reference/src/model.c:6243-6338, ``attn_heads`` :3548-3589, window bound :6326).
+
+The three input projections are kept as one ``[Q + 2K, E]`` matrix.  A layer that
+reads another layer's cache (``kv_shared``) has no key or value projection and writes
+nothing (/root/reference/src/model.h:492-494).
+"""
+from __future__ import annotations
+
+import math
+from typing import Dict, Optional
+
+import torch
+
+from .base import KVSpec, Mixer, ParamSpec, make_part, register_mixer
+
+
+class PagedAttention(Mixer):
+    def __init__(self, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int,
+                 position=None, window: Optional[int] = None, scale: Optional[float] = None,
+                 bias: bool = False, out_bias: Optional[bool] = None, kv_shared: bool = False,
+                 q_name: str = "q_proj", k_name: str = "k_proj", v_name: str = "v_proj",
+                 o_name: str = "o_proj"):
+        if num_heads % num_kv_heads:
+            raise ValueError(f"{num_heads} query heads are not a multiple of {num_kv_heads} key/value heads")
+        if window is not None and window < 1:
+            raise ValueError(f"attention window {window} must be at least 1")
+        self.hidden_size, self.num_heads = int(hidden_size), int(num_heads)
+        self.num_kv_heads, self.head_dim = int(num_kv_heads), int(head_dim)
+        self.window = int(window) if window is not None else None
+        self.scale = float(scale) if scale is not None else 1.0 / math.sqrt(self.head_dim)
+        self.bias = bool(bias)
+        self.out_bias = self.bias if out_bias is None else bool(out_bias)
+        self.kv_shared = bool(kv_shared)
+        self.names = (q_name, k_name, v_name, o_name)
+        self.position = make_part("position", position) if position is not None else None
+        self.q_size = self.num_heads * self.head_dim
+        self.kv_size = self.num_kv_heads * self.head_dim
+        self.w_in = self.b_in = self.w_out = self.b_out = None
+
+    # what the cache manager must keep
+    def kv_spec(self) -> Optional[KVSpec]:
+        return KVSpec(self.num_kv_heads, self.head_dim, self.window)
+
+    def param_specs(self) -> Dict[str, ParamSpec]:
+        E, Q, K = self.hidden_size, self.q_size, self.kv_size
+        q, k, v, o = self.names
+        specs = {f"{q}.weight": ParamSpec((Q, E)), f"{o}.weight": ParamSpec((E, Q))}
+        if not self.kv_shared:
+            specs[f"{k}.weight"] = ParamSpec((K, E))
+            specs[f"{v}.weight"] = ParamSpec((K, E))
+        if self.bias:
+            specs[f"{q}.bias"] = ParamSpec((Q,), role="vector", init="normal")
+            if not self.kv_shared:
+                specs[f"{k}.bias"] = ParamSpec((K,), role="vector", init="normal")
+                specs[f"{v}.bias"] = ParamSpec((K,), role="vector", init="normal")
+        if self.out_bias:
+            specs[f"{o}.bias"] = ParamSpec((E,), role="vector", init="normal")
+        return specs
+
+    def bind(self, tensors, rt) -> None:
+        self.rt = rt
+        q, k, v, o = self.names
+        mats = [tensors[f"{q}.weight"]]
+        if not self.kv_shared:
+            mats += [tensors[f"{k}.weight"], tensors[f"{v}.weight"]]
+        self.w_in = torch.cat(mats, dim=0).contiguous() if len(mats) > 1 else mats[0]
+        self.w_out = tensors[f"{o}.weight"]
+        if self.bias:
+            bs = [tensors[f"{q}.bias"]]
+            if not self.kv_shared:
+                bs += [tensors[f"{k}.bias"], tensors[f"{v}.bias"]]
+            self.b_in = torch.cat([b.float() for b in bs]).contiguous()
+        if self.out_bias:
+            self.b_out = tensors[f"{o}.bias"].float().contiguous()
+        if self.position is not None:
+            self.position.bind({}, rt)
+
+    def _attend(self, ctx, cache, h):
+        ops, rt = self.rt.ops, self.rt
+        Q, K, H, Hk, D = self.q_size, self.kv_size, self.num_heads, self.num_kv_heads, self.head_dim
+        T = h.shape[0]
+        proj = ops.linear(h, self.w_in, bias=self.b_in, out_dtype=torch.float32)
+        writes = not self.kv_shared and cache.owns
+        q_in = proj[:, :Q]
+        k_in = proj[:, Q:Q + K] if writes else None
+        v_in = proj[:, Q + K:Q + 2 * K] if writes else None
+        rot = self.position.rotary() if self.position is not None else None
+        if self.position is not None and rot is None:
+            self.position.apply(ctx, q_in.unflatten(1, (H, D)), k_in.unflatten(1, (Hk, D)) if writes else None)
+        q = torch.empty((T, Q), dtype=rt.dtype, device=h.device)
+        table = ctx.block_table(cache.group)
+        ops.rope_kv_write(q_in, k_in, v_in, q, cache.k if writes else None, cache.v if writes else None,
+                          ctx.positions, ctx.req_of_token, table,
+                          rot.inv_freq if rot else None, H, Hk if writes else 0, D,
+                          rot.rotary_dim if rot else 0, rot.interleaved if rot else False,
+                          rot.mscale if rot else 1.0, cache.page_size)
+        return ops.attention(q, cache.k, cache.v, ctx.positions, ctx.req_of_token, table, H, Hk, D,
+                             cache.page_size, self.scale, self.window)
+
+    def forward(self, ctx, cache, h):
+        return self.rt.ops.linear(self._attend(ctx, cache, h), self.w_out, bias=self.b_out)
+
+    def forward_add(self, ctx, cache, h, residual) -> None:
+        self.rt.ops.linear(self._attend(ctx, cache, h), self.w_out, bias=self.b_out, out=residual, accumulate=True)
+
+
+register_mixer("paged_attention", PagedAttention)

@@ -1,0 +1,213 @@
+"""Interfaces of the parts a model is put together from.
+
+A part is built from a ``PartSpec`` (its sizes and constants), names the tensors
+it needs, is given them by ``bind`` and is then called by the step function.  No
+part knows which architecture it is in; an architecture's builder chooses parts
+layer by layer.
+
+Families and what each must offer:
+
+* ``Norm``: ``forward(ctx, x, rows=None) -> h``.  ``x`` is the 32-bit residual
+  stream ``[T, E]``; ``h`` is in the compute dtype.  ``rows`` (device int32)
+  selects rows of ``x``.
+* ``PositionEncoding``: ``rotary()`` returns the parameters of a rotation that
+  the attention kernels apply themselves, or ``None``; then ``apply(ctx, q, k)``
+  is called on the 32-bit queries and keys before they are cached.
+* ``Mixer``: ``kv_spec()`` and ``state_spec()`` say what the cache manager must
+  keep for it; ``forward(ctx, cache, h) -> y`` returns ``[T, E]`` in the compute
+  dtype; ``forward_add(ctx, cache, h, residual)`` adds it into the 32-bit
+  residual stream (the default calls ``forward``; a part with a fused epilogue
+  overrides it).
+* ``FeedForward``: ``forward(ctx, h) -> y`` and ``forward_add(ctx, h, residual)``.
+* ``Block``: the arrangement; ``forward(ctx, cache, x)`` updates ``x`` in place.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Any, Callable, Dict, Optional, Tuple
+
+import torch
+
+
+@dataclass(frozen=True)
+class ParamSpec:
+    """One tensor a part reads from the checkpoint.
+
+    ``role``: "matrix" tensors are kept in the engine's compute dtype; "vector"
+    tensors keep 32 bits if the file stores them so (bfloat16 otherwise, in a
+    bfloat16 engine); "int" tensors become int32.
+    ``init`` tells the random-weights mode what to write: "normal", "ones",
+    "ones_jitter" (1 + N(0, jitter)) or "zeros".
+    """
+    shape: Tuple[int, ...]
+    role: str = "matrix"
+    init: str = "normal"
+    optional: bool = False
+
+
+@dataclass(frozen=True)
+class KVSpec:
+    """What a mixer with keys and values asks of the cache manager.
+
+    Layers whose specs are equal share a group: one pool of pages and one block
+    table per request.  ``window`` = None keeps every key; a number keeps only
+    the pages that the last ``window`` positions touch.
+    """
+    num_kv_heads: int
+    head_dim: int
+    window: Optional[int] = None
+
+
+@dataclass(frozen=True)
+class StateSpec:
+    """Fixed-size state per request (one slot per live request)."""
+    shape: Tuple[int, ...]
+    dtype: torch.dtype = torch.float32
+
+
+class Part:
+    """Common base: parameters by relative name."""
+
+    def param_specs(self) -> Dict[str, ParamSpec]:
+        return {}
+
+    def bind(self, tensors: Dict[str, torch.Tensor], rt: "Runtime") -> None:
+        """Take the loaded tensors (already on the device, in the dtype their role asks for)."""
+        self.rt = rt
+        for k, v in tensors.items():
+            setattr(self, "w_" + k.replace(".", "_"), v)
+
+
+class Norm(Part):
+    def forward(self, ctx, x: torch.Tensor, rows: Optional[torch.Tensor] = None) -> torch.Tensor:
+        raise NotImplementedError
+
+
+@dataclass(frozen=True)
+class RotaryParams:
+    """A rotation the attention kernels apply to queries and keys themselves."""
+    inv_freq: torch.Tensor      # [rotary_dim / 2] float32, on the device
+    rotary_dim: int
+    interleaved: bool           # False: pairs (j, j + rotary_dim/2); True: pairs (2j, 2j+1)
+    mscale: float = 1.0
+
+
+class PositionEncoding(Part):
+    def rotary(self) -> Optional[RotaryParams]:
+        return None
+
+    def apply(self, ctx, q: torch.Tensor, k: Optional[torch.Tensor]) -> None:
+        """Transform 32-bit ``q [T, H, D]`` and ``k [T, Hk, D]`` in place (default: nothing)."""
+        return None
+
+
+class Mixer(Part):
+    def kv_spec(self) -> Optional[KVSpec]:
+        return None
+
+    def state_spec(self) -> Optional[StateSpec]:
+        return None
+
+    def forward(self, ctx, cache, h: torch.Tensor) -> torch.Tensor:
+        raise NotImplementedError
+
+    def forward_add(self, ctx, cache, h: torch.Tensor, residual: torch.Tensor) -> None:
+        ctx.ops.add_(residual, self.forward(ctx, cache, h))
+
+
+class FeedForward(Part):
+    def forward(self, ctx, h: torch.Tensor) -> torch.Tensor:
+        raise NotImplementedError
+
+    def forward_add(self, ctx, h: torch.Tensor, residual: torch.Tensor) -> None:
+        ctx.ops.add_(residual, self.forward(ctx, h))
+
+
+class Block:
+    """An arrangement of two norms, a mixer and a feed-forward around the residual stream."""
+
+    def __init__(self, mixer_norm: Norm, mixer: Mixer, feed_forward_norm: Norm, feed_forward: FeedForward):
+        self.mixer_norm = mixer_norm
+        self.mixer = mixer
+        self.feed_forward_norm = feed_forward_norm
+        self.feed_forward = feed_forward
+
+    def parts(self):
+        return {"mixer_norm": self.mixer_norm, "mixer": self.mixer,
+                "feed_forward_norm": self.feed_forward_norm, "feed_forward": self.feed_forward}
+
+    def forward(self, ctx, cache, x: torch.Tensor) -> None:
+        raise NotImplementedError
+
+
+@dataclass
+class Runtime:
+    """What every part needs at run time: the device, the dtypes, and the kernels."""
+    device: torch.device
+    dtype: torch.dtype              # compute dtype: torch.float32 or torch.bfloat16
+    ops: Any                        # xyntetik_runner_amd.csrc.ops.Ops
+
+    @property
+    def is_fp32(self) -> bool:
+        return self.dtype == torch.float32
+
+
+# --------------------------------------------------------------------------- registries
+
+_REGISTRIES: Dict[str, Dict[str, Callable[..., Any]]] = {
+    "norm": {}, "position": {}, "mixer": {}, "feed_forward": {}, "block": {}, "embedding": {}, "head": {},
+}
+
+
+def _register(family: str, kind: str, factory: Callable[..., Any], replace: bool = False) -> None:
+    reg = _REGISTRIES[family]
+    if kind in reg and not replace:
+        raise ValueError(f"{family} part {kind!r} is already registered")
+    reg[kind] = factory
+
+
+def register_norm(kind, factory, replace=False):
+    _register("norm", kind, factory, replace)
+
+
+def register_position(kind, factory, replace=False):
+    _register("position", kind, factory, replace)
+
+
+def register_mixer(kind, factory, replace=False):
+    _register("mixer", kind, factory, replace)
+
+
+def register_feed_forward(kind, factory, replace=False):
+    _register("feed_forward", kind, factory, replace)
+
+
+def register_block(kind, factory, replace=False):
+    _register("block", kind, factory, replace)
+
+
+def register_embedding(kind, factory, replace=False):
+    _register("embedding", kind, factory, replace)
+
+
+def register_head(kind, factory, replace=False):
+    _register("head", kind, factory, replace)
+
+
+def unregister(family: str, kind: str) -> None:
+    _REGISTRIES[family].pop(kind, None)
+
+
+def make_part(family: str, spec) -> Any:
+    """Build the part a ``PartSpec`` describes."""
+    reg = _REGISTRIES[family]
+    if spec.kind not in reg:
+        raise ValueError(f"no {family} part of kind {spec.kind!r}; registered: {sorted(reg)}")
+    return reg[spec.kind](**spec.params)
+
+
+def make_block(kind: str, mixer_norm, mixer, feed_forward_norm, feed_forward) -> Block:
+    reg = _REGISTRIES["block"]
+    if kind not in reg:
+        raise ValueError(f"no block arrangement {kind!r}; registered: {sorted(reg)}")
+    return reg[kind](mixer_norm, mixer, feed_forward_norm, feed_forward)

@@ -1,0 +1,34 @@
+"""The output head: ``logits = W h`` in 32-bit, with ``W`` its own tensor or the
+embedding table when the model ties them (/root/reference/src/model.c:2353-2366, :6481).
+"""
+from __future__ import annotations
+
+from typing import Dict
+
+import torch
+
+from .base import Part, ParamSpec, register_head
+
+
+class LinearHead(Part):
+    def __init__(self, vocab_size: int, hidden_size: int, tied: bool = False, weight_name: str = "weight"):
+        self.vocab_size, self.hidden_size, self.tied = int(vocab_size), int(hidden_size), bool(tied)
+        self.weight_name = weight_name
+        self.weight = None
+
+    def param_specs(self) -> Dict[str, ParamSpec]:
+        if self.tied:
+            return {}
+        return {self.weight_name: ParamSpec((self.vocab_size, self.hidden_size), role="matrix")}
+
+    def bind(self, tensors, rt, tied_to=None) -> None:
+        self.rt = rt
+        self.weight = tied_to if self.tied else tensors[self.weight_name]
+        if self.weight is None:
+            raise ValueError("a tied head needs the embedding table")
+
+    def forward(self, ctx, h):
+        return self.rt.ops.linear(h, self.weight, out_dtype=torch.float32)
+
+
+register_head("linear", LinearHead)

@@ -1,0 +1,58 @@
+"""Gated feed-forward: ``down(act(gate(h)) * up(h))`` with act = SiLU
+(/root/reference/src/model.c:6399-6407, ``gated_act`` :4451-4452).
+
+``gate`` and ``up`` are kept as one ``[2F, E]`` matrix so that one product makes both;
+the reference does the reverse for a checkpoint that stores them fused
+(``slice_rows``, /root/reference/src/model.c:238-248).
+"""
+from __future__ import annotations
+
+from typing import Dict
+
+import torch
+
+from .base import FeedForward, ParamSpec, register_feed_forward
+
+
+class GatedMLP(FeedForward):
+    def __init__(self, hidden_size: int, intermediate_size: int, activation: str = "silu", bias: bool = False,
+                 gate_name: str = "gate_proj", up_name: str = "up_proj", down_name: str = "down_proj"):
+        if activation != "silu":
+            raise ValueError(f"gated feed-forward: activation {activation!r} is not supported (silu)")
+        self.hidden_size, self.intermediate_size = int(hidden_size), int(intermediate_size)
+        self.bias = bool(bias)
+        self.names = (gate_name, up_name, down_name)
+        self.w_gate_up = self.w_down = self.b_gate_up = self.b_down = None
+
+    def param_specs(self) -> Dict[str, ParamSpec]:
+        E, F = self.hidden_size, self.intermediate_size
+        g, u, d = self.names
+        specs = {f"{g}.weight": ParamSpec((F, E)), f"{u}.weight": ParamSpec((F, E)),
+                 f"{d}.weight": ParamSpec((E, F))}
+        if self.bias:
+            specs.update({f"{g}.bias": ParamSpec((F,), role="vector", init="normal"),
+                          f"{u}.bias": ParamSpec((F,), role="vector", init="normal"),
+                          f"{d}.bias": ParamSpec((E,), role="vector", init="normal")})
+        return specs
+
+    def bind(self, tensors, rt) -> None:
+        self.rt = rt
+        g, u, d = self.names
+        self.w_gate_up = torch.cat([tensors[f"{g}.weight"], tensors[f"{u}.weight"]], dim=0).contiguous()
+        self.w_down = tensors[f"{d}.weight"]
+        if self.bias:
+            self.b_gate_up = torch.cat([tensors[f"{g}.bias"], tensors[f"{u}.bias"]]).float().contiguous()
+            self.b_down = tensors[f"{d}.bias"].float().contiguous()
+
+    def _hidden(self, ctx, h):
+        ops = self.rt.ops
+        return ops.silu_mul(ops.linear(h, self.w_gate_up, bias=self.b_gate_up))
+
+    def forward(self, ctx, h):
+        return self.rt.ops.linear(self._hidden(ctx, h), self.w_down, bias=self.b_down)
+
+    def forward_add(self, ctx, h, residual) -> None:
+        self.rt.ops.linear(self._hidden(ctx, h), self.w_down, bias=self.b_down, out=residual, accumulate=True)
+
+
+register_feed_forward("gated_mlp", GatedMLP)
