@@ -10,3 +10,7 @@ sampling (``sampling``), hand-written gfx950 kernels (``csrc``), a command line
 __version__ = "0.1.0"
 
 from . import config, parts, architectures    # noqa: F401,E402  (fills the registries)
+from .sampling import SamplingParams    # noqa: E402
+from .llm import LLM    # noqa: E402
+
+__all__ = ["LLM", "SamplingParams", "config", "parts", "architectures", "__version__"]

@@ -1,0 +1,42 @@
+"""A generation request as the scheduler sees it."""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Hashable, List, Optional
+
+from ..sampling.params import SamplerState, SamplingParams
+
+WAITING, RUNNING, FINISHED = "waiting", "running", "finished"
+
+
+class Request:
+    def __init__(self, req_id: Hashable, prompt: List[int], params: SamplingParams):
+        if not prompt:
+            raise ValueError("a request needs at least one prompt token")
+        self.id = req_id
+        self.prompt = [int(t) for t in prompt]
+        self.params = params
+        self.output: List[int] = []
+        self.n_computed = 0          # tokens of prompt + output whose keys and values are cached
+        self.status = WAITING
+        self.finish_reason: Optional[str] = None
+        self.sampler = SamplerState(params)
+        self.n_accepted = 0          # tokens already recorded in the sampler's recent window
+        self.n_preempted = 0
+
+    @property
+    def tokens(self) -> List[int]:
+        return self.prompt + self.output
+
+    @property
+    def n_tokens(self) -> int:
+        return len(self.prompt) + len(self.output)
+
+    @property
+    def remaining(self) -> int:
+        """Tokens that still have to run before the next one can be sampled."""
+        return self.n_tokens - self.n_computed
+
+    @property
+    def finished(self) -> bool:
+        return self.status == FINISHED
