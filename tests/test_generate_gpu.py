@@ -1,0 +1,185 @@
+"""Generation on the GPU: greedy and sampled decoding through the entry points, the
+sampling kernel against the plain sampler, preemption, and the command line."""
+import os
+import subprocess
+import sys
+
+import numpy as np
+import pytest
+
+import plain_llama as P
+from tiny import make_model, prompt_ids
+
+pytestmark = pytest.mark.gpu
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+@pytest.fixture(scope="module")
+def folders(tmp_path_factory):
+    return {w: make_model(w, str(tmp_path_factory.mktemp("gen" + w))) for w in ("A", "B")}
+
+
+def near_argmax(cfg, w, prompt, out, frac):
+    """Every generated token is the plain model's argmax for its prefix, or within ``frac`` of the range of it."""
+    toks = list(prompt)
+    for t in out:
+        lg = P.forward(cfg, w, toks)[-1]
+        assert lg.max() - lg[t] <= frac * (lg.max() - lg.min()), (len(toks), t, int(lg.argmax()))
+        toks.append(t)
+
+
+@pytest.mark.parametrize("which,lens,n_new", [("A", [5, 17, 33], 16), ("B", [1, 9, 40, 64, 100], 24)])
+def test_greedy_through_the_entry_point(folders, which, lens, n_new):
+    from xyntetik_runner_amd import LLM, SamplingParams
+    cfg, w = P.load_folder(folders[which])
+    prompts = [prompt_ids(n, cfg["vocab_size"], 50 + i) for i, n in enumerate(lens)]
+    llm = LLM(folders[which], dtype="float32", max_tokens=1024, page_size=16, max_batched_tokens=48)
+    outs = llm.generate(prompts, SamplingParams(temperature=0.0, max_new_tokens=n_new))
+    for p, o in zip(prompts, outs):
+        assert len(o) == n_new
+        assert o == P.greedy(cfg, w, p, n_new)
+    llm.runner.manager.check()
+    del llm
+    llm = LLM(folders[which], dtype="bfloat16", max_tokens=1024, page_size=64, max_batched_tokens=64)
+    outs = llm.generate(prompts, SamplingParams(temperature=0.0, max_new_tokens=n_new))
+    for p, o in zip(prompts, outs):
+        assert len(o) == n_new
+        near_argmax(cfg, w, p, o, 0.02)
+
+
+def test_sampled_tokens_depend_on_the_request_alone(folders):
+    from xyntetik_runner_amd import LLM, SamplingParams
+    cfg, w = P.load_folder(folders["B"])
+    prompts = [prompt_ids(n, 384, 70 + i) for i, n in enumerate([1, 9, 40, 64, 100])]
+    sp = [SamplingParams(temperature=0.8, seed=1000 + i, max_new_tokens=24) for i in range(5)]
+    llm = LLM(folders["B"], dtype="float32", max_tokens=2048, page_size=16, max_batched_tokens=32)
+    together = llm.generate(prompts, sp)
+    again = llm.generate(prompts, sp)
+    assert together == again
+    alone = [llm.generate([p], s)[0] for p, s in zip(prompts, sp)]
+    assert alone == together
+    other_seed = llm.generate(prompts[2:3], SamplingParams(temperature=0.8, seed=5, max_new_tokens=24))[0]
+    assert other_seed != together[2]
+    # each token is what the plain sampler picks from the plain logits with the same draw
+    for p, s, out in zip(prompts, sp, together):
+        state, toks = s.seed, list(p)
+        for t in out:
+            state, r = P.rng_f32(state)
+            assert P.sample_pick(P.forward(cfg, w, toks)[-1], 0.8, r) == t
+            toks.append(t)
+
+
+def test_sampling_kernel_matches_plain_sampler():
+    import torch
+    from xyntetik_runner_amd.csrc.ops import load_ops
+    ops = load_ops()
+    rng = np.random.default_rng(0)
+    cases = []
+    for V in (8, 333, 5000):
+        for _ in range(6):
+            lg = (rng.normal(size=V) * rng.choice([0.5, 3.0])).astype(np.float32)
+            if rng.random() < 0.5:
+                lg[rng.integers(0, V, size=V // 3)] = lg[0]             # exact ties
+            kw = dict(temp=float(rng.choice([0.0, 0.3, 0.8, 1.5])), draw=float(np.float32(rng.random())),
+                      top_k=int(rng.choice([0, 1, 5, 40])), top_p=float(rng.choice([1.0, 0.9, 0.5])),
+                      min_p=float(rng.choice([0.0, 0.05, 0.3])), repeat_penalty=float(rng.choice([1.0, 1.3])),
+                      recent=[int(t) for t in rng.integers(-2, V + 2, size=rng.integers(0, 20))])
+            cases.append((V, lg, kw))
+    all_equal = np.full(64, 1.25, dtype=np.float32)
+    cases.append((64, all_equal, dict(temp=1.0, draw=0.5, top_k=0, top_p=1.0, min_p=0.0, repeat_penalty=1.0, recent=[])))
+    cases.append((64, all_equal, dict(temp=1.0, draw=0.99, top_k=10, top_p=1.0, min_p=0.0, repeat_penalty=1.0, recent=[])))
+    cases.append((64, all_equal, dict(temp=0.0, draw=0.99, top_k=0, top_p=1.0, min_p=0.0, repeat_penalty=1.0, recent=[])))
+    exempt = [3]
+    for V, lg, kw in cases:
+        want = P.sample_pick(lg, kw["temp"], kw["draw"], kw["top_k"], kw["top_p"], kw["min_p"],
+                             kw["repeat_penalty"], kw["recent"], exempt)
+        dev = torch.device("cuda:0")
+        rec = torch.zeros((1, 256), dtype=torch.int32)
+        rec[0, :len(kw["recent"])] = torch.tensor(kw["recent"], dtype=torch.int32)
+        t = torch.tensor(lg, device=dev).unsqueeze(0).contiguous()
+        before = t.clone()
+        got = ops.sample(t, torch.tensor([kw["temp"]], device=dev), torch.tensor([kw["draw"]], device=dev),
+                         top_k=torch.tensor([kw["top_k"]], dtype=torch.int32, device=dev),
+                         top_p=torch.tensor([kw["top_p"]], device=dev), min_p=torch.tensor([kw["min_p"]], device=dev),
+                         repeat_penalty=torch.tensor([kw["repeat_penalty"]], device=dev), recent=rec.to(dev),
+                         n_recent=torch.tensor([len(kw["recent"])], dtype=torch.int32, device=dev),
+                         exempt=torch.tensor(exempt, dtype=torch.int32, device=dev))
+        assert int(got[0]) == want, (V, kw, int(got[0]), want)
+        if kw["temp"] <= 0:
+            assert torch.equal(t, before)                              # greedy leaves the logits untouched
+
+
+def test_sampling_kernel_distribution_and_many_rows():
+    import torch
+    from xyntetik_runner_amd.csrc.ops import load_ops
+    ops = load_ops()
+    dev = torch.device("cuda:0")
+    V, n = 8192, 4000
+    lg = np.full(V, -20.0, dtype=np.float32)
+    lg[[5, 100, 4000]] = [6.0, 5.4, 4.8]
+    z = np.exp(lg.astype(np.float64)); z /= z.sum()
+    s, draws = 42, []
+    for _ in range(n):
+        s, r = P.rng_f32(s)
+        draws.append(r)
+    rows = torch.tensor(lg, device=dev).repeat(n, 1).contiguous()
+    got = ops.sample(rows, torch.ones(n, device=dev), torch.tensor(draws, dtype=torch.float32, device=dev)).cpu().numpy()
+    for t in (5, 100, 4000):
+        assert abs((got == t).mean() - z[t]) < 0.03
+    mixed_t = torch.tensor([0.0, 1.0] * (n // 2), device=dev)
+    got2 = ops.sample(rows, mixed_t, torch.tensor(draws, dtype=torch.float32, device=dev)).cpu().numpy()
+    assert np.all(got2[0::2] == 5) and np.array_equal(got2[1::2], got[1::2])
+
+
+def test_preemption_gives_the_same_tokens(folders):
+    """A pool too small for all requests at once: some are preempted and recomputed, and
+    every request still gets the tokens it gets when it has the cache to itself."""
+    from xyntetik_runner_amd import LLM, SamplingParams
+    cfg, w = P.load_folder(folders["A"])
+    prompts = [prompt_ids(n, 256, 90 + i) for i, n in enumerate([30, 22, 41, 9])]
+    sp = [SamplingParams(temperature=0.7 if i % 2 else 0.0, seed=77 + i, max_new_tokens=40) for i in range(4)]
+    big = LLM(folders["A"], dtype="float32", max_tokens=1024, page_size=8, max_batched_tokens=24)
+    want = big.generate(prompts, sp)
+    assert big.engine.stats.preemptions == 0
+    small = LLM(folders["A"], dtype="float32", max_tokens=160, page_size=8, max_batched_tokens=24)
+    got = small.generate(prompts, sp)
+    assert small.engine.stats.preemptions > 0
+    assert got == want
+    small.runner.manager.check()
+    assert small.runner.manager.free_pages() == small.runner.manager.pages_per_group
+
+
+def test_stop_token_ends_a_request(folders):
+    from xyntetik_runner_amd.engine import Engine, ModelRunner
+    from xyntetik_runner_amd.sampling import SamplingParams
+    cfg, w = P.load_folder(folders["A"])
+    prompt = prompt_ids(12, 256, 3)
+    ref = P.greedy(cfg, w, prompt, 10)
+    runner = ModelRunner.from_folder(folders["A"], dtype="float32", max_tokens=256, page_size=16)
+    eng = Engine(runner, stop_ids=[ref[4]])
+    first = ref.index(ref[4])
+    assert eng.generate([prompt], SamplingParams(max_new_tokens=10)) == [ref[:first]]    # the stop token is not kept
+    eng = Engine(runner, stop_ids=[ref[4]])
+    assert eng.generate([prompt], SamplingParams(max_new_tokens=10, ignore_eos=True)) == [ref]
+
+
+def test_command_line(folders):
+    cfg, w = P.load_folder(folders["A"])
+    prompt = prompt_ids(7, 256, 11)
+    want = P.greedy(cfg, w, prompt, 6)
+    cmd = [sys.executable, os.path.join(ROOT, "bin", "runner"), "-m", folders["A"], "--ids",
+           ",".join(map(str, prompt)), "-n", "6", "--temp", "0", "--dtype", "float32"]
+    p = subprocess.run(cmd, capture_output=True, text=True, timeout=120)
+    assert p.returncode == 0, p.stderr
+    assert p.stdout.strip() == ",".join(map(str, prompt + want))
+    assert "prompt: 7 tok" in p.stderr and "gen: 6 tok" in p.stderr
+    # text prompt: bytes are ids; same seed gives the same text
+    cmd = [sys.executable, os.path.join(ROOT, "bin", "runner"), "-m", folders["A"], "-p", "hi\\n", "-n", "5",
+           "--temp", "0.9", "-s", "3", "--top-k", "50", "--dtype", "float32"]
+    a = subprocess.run(cmd, capture_output=True, timeout=120)
+    b = subprocess.run(cmd, capture_output=True, timeout=120)
+    assert a.returncode == 0 and a.stdout == b.stdout and a.stdout.startswith(b"hi\n")
+    bad = subprocess.run(cmd[:-2] + ["-s", "0"], capture_output=True, text=True, timeout=120)
+    assert bad.returncode == 1 and "not a usable seed" in bad.stderr
+    long = subprocess.run(cmd[:4] + ["--ids", ",".join(["1"] * 200), "-c", "100"], capture_output=True, text=True, timeout=120)
+    assert long.returncode == 1 and "does not fit a context of 100" in long.stderr

@@ -1,0 +1,163 @@
+"""Trace replay on the GPU against the plain implementation, in 32-bit and in bfloat16:
+the same requests whole, with the last 32 tokens one by one, in portions of changing
+size, and mixed with other requests in a pool so small that pages are used again."""
+import json
+import os
+import subprocess
+import sys
+
+import numpy as np
+import pytest
+
+import plain_llama as P
+import traces
+from tiny import MAKE, logit_error, make_model, prompt_ids
+
+pytestmark = pytest.mark.gpu
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+# fraction of the mean logit range: (max, mean)
+TOL = {"float32": (1e-5, 1e-6), "bfloat16": (1e-2, 1e-3)}
+WORKLOAD = {
+    # prompt lengths and given decoded tokens (the two tiny workloads, plus lengths that
+    # end exactly on a page and a long request)
+    "A": ([5, 17, 33, 64, 150], 16),
+    "B": ([1, 9, 40, 64, 100], 24),
+    "C": ([3, 31, 70], 40),
+}
+
+
+@pytest.fixture(scope="module")
+def models(tmp_path_factory):
+    out = {}
+    for which in WORKLOAD:
+        d = make_model(which, str(tmp_path_factory.mktemp("model" + which)))
+        cfg, w = P.load_folder(d)
+        lens, extra = WORKLOAD[which]
+        reqs = {f"r{i}": prompt_ids(n + extra, cfg["vocab_size"], 100 + i) for i, n in enumerate(lens)}
+        plens = {f"r{i}": n for i, n in enumerate(lens)}
+        want = {rid: P.forward(cfg, w, toks) for rid, toks in reqs.items()}
+        out[which] = (d, cfg, reqs, plens, want)
+    return out
+
+
+def run_replay(model_dir, dtype, steps, tmp_path, page_size, max_tokens=None):
+    from xyntetik_runner_amd.engine.runner import ModelRunner
+    from xyntetik_runner_amd.trace import replay
+    mt = max_tokens or traces.max_live_tokens(steps, max(64, page_size))
+    runner = ModelRunner.from_folder(model_dir, dtype=dtype, max_tokens=mt, page_size=page_size, max_requests=4)
+    out = str(tmp_path / "out")
+    import io
+    replay(runner, traces.to_lines(steps), out, report=io.StringIO())
+    runner.manager.check()
+    assert not runner.manager.requests and runner.manager.free_pages() == runner.manager.pages_per_group
+    return out, runner
+
+
+def check(got, want, dtype, what):
+    assert set(got) == set(want)
+    for rid in want:
+        assert got[rid].shape == want[rid].shape, (what, rid)
+        assert np.abs(got[rid]).max() > 0, "all-zero logits"
+        mx, mean = logit_error(got[rid], want[rid])
+        tmax, tmean = TOL[dtype]
+        if not (mx <= tmax and mean <= tmean):
+            d = np.abs(got[rid] - want[rid]).max(axis=1)
+            first = int(np.argmax(d > tmax * float(np.mean(want[rid].max(-1) - want[rid].min(-1)))))
+            raise AssertionError(f"{what} {dtype} request {rid}: max {mx:.3e} mean {mean:.3e} of the logit range "
+                                 f"(allowed {tmax:.0e} / {tmean:.0e}); first wrong position {first}")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("which", ["A", "B", "C"])
+@pytest.mark.parametrize("schedule", ["whole", "tail", "portions", "mixed"])
+def test_schedules_match_plain(models, tmp_path, which, dtype, schedule):
+    d, cfg, reqs, plens, want = models[which]
+    page_size = {"A": 16, "B": 64, "C": 4}[which]
+    if schedule == "whole":
+        steps = traces.whole(reqs)
+    elif schedule == "tail":
+        steps = traces.tail_one_by_one(reqs, 32)
+    elif schedule == "portions":
+        steps = traces.portions(reqs)
+    else:
+        steps = traces.mixed(reqs, plens, max_live=4 if which != "A" else 3, seed=len(which))
+    out, runner = run_replay(d, dtype, steps, tmp_path, page_size)
+    got = traces.collect(steps, out, cfg["vocab_size"])
+    check(got, want, dtype, f"{which}/{schedule}")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_pages_are_used_again_and_old_contents_never_show(models, tmp_path, dtype):
+    """The pool holds barely more than the live requests; every page is poisoned with NaN before
+    the replay, so a read beyond a request's length, or of a page it does not own, shows."""
+    import torch
+    from xyntetik_runner_amd.engine.runner import ModelRunner
+    from xyntetik_runner_amd.trace import replay
+    import io
+    d, cfg, reqs, plens, want = models["B"]
+    steps = traces.mixed(reqs, plens, max_live=2, seed=5)
+    mt = traces.max_live_tokens(steps, 64)
+    runner = ModelRunner.from_folder(d, dtype=dtype, max_tokens=mt, page_size=8, max_requests=2)
+    for lc in runner.storage.layers:
+        lc.k.fill_(float("nan")); lc.v.fill_(float("nan"))
+    seen = set()
+    orig_step = runner.step
+
+    def spying_step(entries):
+        r = orig_step(entries)
+        for rc in runner.manager.requests.values():
+            seen.update((id(rc), p) for p in rc.tables[0])
+        return r
+    runner.step = spying_step
+    out = str(tmp_path / "o")
+    replay(runner, traces.to_lines(steps), out, report=io.StringIO())
+    pages_by_req = {}
+    for rid, p in seen:
+        pages_by_req.setdefault(p, set()).add(rid)
+    assert any(len(v) > 1 for v in pages_by_req.values()), "no page was used by two requests"
+    check(traces.collect(steps, out, cfg["vocab_size"]), want, dtype, "B/reuse")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_trace_run_program(models, tmp_path, dtype):
+    """bin/trace_run as a user runs it: a child process, steps on stdin, 'done <step>' lines back."""
+    d, cfg, reqs, plens, want = models["A"]
+    steps = traces.mixed(reqs, plens, max_live=4, seed=9)
+    # a step in which nothing is wanted writes no file
+    steps[0]["entries"][0]["want"] = []
+    mt = traces.max_live_tokens(steps, 64)
+    out = str(tmp_path / "out")
+    p = subprocess.Popen([sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", d, "--dtype", dtype,
+                          "--out", out, "--max-tokens", str(mt)], stdin=subprocess.PIPE, stdout=subprocess.PIPE,
+                         text=True)
+    for st in steps:
+        p.stdin.write(json.dumps(st) + "\n")
+        p.stdin.flush()
+        assert p.stdout.readline().strip() == f"done {st['step']}"
+    p.stdin.close()
+    assert p.wait(timeout=60) == 0
+    got = traces.collect(steps, out, cfg["vocab_size"])
+    first = steps[0]["entries"][0]
+    n0 = len(first["tokens"])
+    w = dict(want)
+    w[first["id"]] = want[first["id"]][n0:]
+    check(got, w, dtype, "trace_run")
+
+
+def test_out_of_pages_is_an_error_that_changes_nothing(models):
+    from xyntetik_runner_amd.cache import OutOfPages
+    from xyntetik_runner_amd.engine.batch import StepEntry
+    from xyntetik_runner_amd.engine.runner import ModelRunner
+    d, cfg, reqs, plens, want = models["A"]
+    runner = ModelRunner.from_folder(d, dtype="float32", max_tokens=64, page_size=16, max_requests=2)
+    toks = reqs["r3"]
+    runner.step([StepEntry("a", toks[:40], [])])
+    free = runner.manager.free_pages()
+    with pytest.raises(OutOfPages):
+        runner.step([StepEntry("a", toks[40:60], []), StepEntry("b", toks[:30], [])])
+    assert runner.manager.free_pages() == free and runner.length("a") == 40
+    got = runner.step([StepEntry("a", toks[40:64], list(range(24)))]).cpu().numpy()
+    mx, mean = logit_error(got, want["r3"][40:64])
+    assert mx <= TOL["float32"][0]
+    runner.manager.check()
