@@ -1,0 +1,359 @@
+"""Each kernel alone against a plain PyTorch float32/float64 reference of the same
+operation, at sizes other than the tiny models': widths and vocabularies that are no
+powers of two, head sizes in steps of 16, any number of heads and groups, several page
+sizes, windows.  Where random inputs would hide a fault the inputs are made so that it
+shows: one far key whose score stands out, keys at a page's edge, a window's edge."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from xyntetik_runner_amd.csrc.ops import load_ops
+    return load_ops()
+
+
+DEV = "cuda:0"
+DT = {"float32": torch.float32, "bfloat16": torch.bfloat16}
+
+
+def rel(got, want):
+    return (got.double() - want.double()).abs().max().item() / max(want.double().abs().max().item(), 1e-30)
+
+
+# ------------------------------------------------------------------ small kernels
+@pytest.mark.parametrize("V,E", [(100, 72), (333, 4100)])
+@pytest.mark.parametrize("dt", ["float32", "bfloat16"])
+def test_embedding(ops, V, E, dt):
+    table = torch.randn(V, E, device=DEV).to(DT[dt])
+    ids = torch.tensor([0, V - 1, 5, -3, V, 17], dtype=torch.int32, device=DEV)
+    got = ops.embedding(table, ids, scale=1.0)
+    want = table.float()[torch.tensor([0, V - 1, 5, 0, 0, 17], device=DEV)]       # out of range reads row 0
+    assert got.dtype == torch.float32 and torch.equal(got, want)
+    assert torch.equal(ops.embedding(table, ids, scale=2.0), want * 2)
+
+
+@pytest.mark.parametrize("E", [8, 100, 4096, 5000])
+@pytest.mark.parametrize("out", ["float32", "bfloat16"])
+@pytest.mark.parametrize("wdt", ["float32", "bfloat16"])
+def test_rmsnorm(ops, E, out, wdt):
+    x = torch.randn(7, E, device=DEV) * 3
+    w = (1 + 0.1 * torch.randn(E, device=DEV)).to(DT[wdt])
+    for eps in (1e-5, 1e-2):
+        want = x.double() / torch.sqrt((x.double() ** 2).mean(-1, keepdim=True) + eps) * w.double()
+        got = ops.rmsnorm(x, w, eps, DT[out])
+        assert rel(got, want) < (2e-6 if out == "float32" else 5e-3)
+    rows = torch.tensor([6, 0, 3], dtype=torch.int32, device=DEV)
+    got = ops.rmsnorm(x, w, 1e-5, DT[out], rows=rows)
+    assert torch.equal(got, ops.rmsnorm(x, w, 1e-5, DT[out])[rows.long()])
+    # eps placement shows on a near-zero row
+    tiny = torch.full((1, E), 1e-4, device=DEV)
+    got = ops.rmsnorm(tiny, None, 1e-6, torch.float32)
+    assert abs(got[0, 0].item() - 1e-4 / math.sqrt(1e-8 + 1e-6)) < 1e-7
+
+
+@pytest.mark.parametrize("dt", ["float32", "bfloat16"])
+def test_silu_mul_add_convert_fill(ops, dt):
+    T, F = 5, 301
+    gu = (torch.randn(T, 2 * F, device=DEV) * 4).to(DT[dt])
+    gu[0, 0] = -200.0
+    g, u = gu[:, :F].double(), gu[:, F:].double()
+    want = g / (1 + torch.exp(-g)) * u
+    got = ops.silu_mul(gu)
+    assert torch.isfinite(got.float()).all() and rel(got, want) < (1e-6 if dt == "float32" else 5e-3)
+    x = torch.randn(T, F, device=DEV)
+    y = torch.randn(T, F, device=DEV).to(DT[dt])
+    want = x + y.float()
+    ops.add_(x, y)
+    assert torch.equal(x, want)
+    c = ops.convert(x, torch.bfloat16)
+    assert torch.equal(c, x.bfloat16()) and torch.equal(ops.convert(c, torch.float32), c.float())
+    st = torch.randn(6, 3, 5, device=DEV)
+    keep = st.clone()
+    ops.fill_rows_(st, torch.tensor([4, 1], dtype=torch.int32, device=DEV), 2)
+    assert (st[4] == 0).all() and (st[1] == 0).all() and torch.equal(st[[0, 2, 3, 5]], keep[[0, 2, 3, 5]])
+
+
+# ------------------------------------------------------------------ matrix products
+@pytest.mark.parametrize("M", [1, 5, 16, 17, 33, 64, 65, 130, 300])
+@pytest.mark.parametrize("N,K", [(48, 64), (100, 72), (333, 264), (1000, 1032)])
+def test_linear_bf16_mfma(ops, M, N, K):
+    a = (torch.randn(M, K, device=DEV) * 0.5).bfloat16()
+    w = (torch.randn(N, K, device=DEV) * 0.1).bfloat16()
+    b = torch.randn(N, device=DEV) * 0.1
+    want = a.double() @ w.double().T + b.double()
+    assert rel(ops.linear(a, w, bias=b, out_dtype=torch.float32), want) < 1e-5       # 32-bit accumulation
+    assert rel(ops.linear(a, w, bias=b), want) < 6e-3                                  # rounded once to bfloat16
+    base = torch.randn(M, N, device=DEV)
+    out = base.clone()
+    ops.linear(a, w, out=out, accumulate=True)
+    assert rel(out, base.double() + a.double() @ w.double().T) < 1e-5
+    w2 = (torch.randn(2 * N, K, device=DEV) * 0.1).bfloat16()
+    b2 = torch.randn(2 * N, device=DEV) * 0.1
+    r = a.double() @ w2.double().T + b2.double()
+    want = r[:, :N] / (1 + torch.exp(-r[:, :N])) * r[:, N:]
+    assert rel(ops.linear_swiglu(a, w2, bias=b2), want) < 6e-3
+    if M > 64:
+        assert rel(ops.linear(a, w, bias=b, out_dtype=torch.float32, variant=3), a.double() @ w.double().T + b.double()) < 1e-5
+
+
+@pytest.mark.parametrize("M,N,K", [(1, 7, 5), (9, 100, 77), (70, 65, 130)])
+@pytest.mark.parametrize("dt", ["float32", "bfloat16"])
+def test_linear_plain_kernel(ops, M, N, K, dt):
+    """Sizes the MFMA kernels refuse (K not a multiple of 8) and the whole 32-bit path."""
+    a = torch.randn(M, K, device=DEV).to(DT[dt])
+    w = torch.randn(N, K, device=DEV).to(DT[dt])
+    b = torch.randn(N, device=DEV)
+    want = a.double() @ w.double().T + b.double()
+    assert rel(ops.linear(a, w, bias=b, out_dtype=torch.float32), want) < 2e-6
+    base = torch.randn(M, N, device=DEV)
+    out = base.clone()
+    ops.linear(a, w, out=out, accumulate=True)
+    assert rel(out, base.double() + a.double() @ w.double().T) < 2e-6
+
+
+def test_linear_one_hot_rows_pick_weight_rows(ops):
+    """A one-hot input returns the matching weight column: a transposed or mis-strided operand fails."""
+    N, K = 96, 64
+    w = torch.randn(N, K, device=DEV).bfloat16()
+    for M in (3, 100):
+        a = torch.zeros(M, K, device=DEV).bfloat16()
+        cols = [(7 * i + 3) % K for i in range(M)]
+        for i, c in enumerate(cols):
+            a[i, c] = 1.0
+        got = ops.linear(a, w, out_dtype=torch.float32)
+        assert torch.equal(got, w.float()[:, cols].T.contiguous())
+
+
+def test_linear_refuses_bad_operands(ops):
+    from xyntetik_runner_amd.csrc.ops import KernelError
+    a = torch.randn(4, 16, device=DEV).bfloat16()
+    with pytest.raises(KernelError):
+        ops.linear(a, torch.randn(8, 24, device=DEV).bfloat16())
+    with pytest.raises(KernelError):
+        ops.linear(a, torch.randn(8, 16, device=DEV))
+    with pytest.raises(KernelError):
+        ops.linear(a.cpu(), torch.randn(8, 16).bfloat16())
+
+
+# ------------------------------------------------------------------ rotary + cache write + attention
+class FakeCtx:
+    """The part of a step's context that the attention kernels read."""
+
+    def __init__(self, starts, q_lens, tables, page_size):
+        from xyntetik_runner_amd.engine.batch import plan_attention, AttentionPlan
+        self.starts, self.q_lens = list(starts), list(q_lens)
+        pos, rot, cu = [], [], [0]
+        for b, (s, n) in enumerate(zip(starts, q_lens)):
+            pos += list(range(s, s + n)); rot += [b] * n; cu.append(cu[-1] + n)
+        i32 = lambda v: torch.tensor(v, dtype=torch.int32, device=DEV)
+        self.positions, self.req_of_token, self.cu_q, self.starts_dev = i32(pos), i32(rot), i32(cu), i32(list(starts))
+        width = max(len(t) for t in tables)
+        tab = torch.full((len(tables), width), -1, dtype=torch.int32)
+        for b, t in enumerate(tables):
+            tab[b, :len(t)] = torch.tensor(t, dtype=torch.int32)
+        self._table = tab.to(DEV)
+        self._plan_fn, self._Plan = plan_attention, AttentionPlan
+
+    def block_table(self, group):
+        return self._table
+
+    def attention_plan(self, group, G, window, Hk):
+        items, jobs, n_slots = self._plan_fn(self.starts, self.q_lens, G, window, Hk)
+        it = torch.tensor([v for i in items for v in i], dtype=torch.int32, device=DEV)
+        jb = torch.tensor([v for j in jobs for v in j], dtype=torch.int32, device=DEV) if jobs else None
+        return self._Plan(it, len(items), jb, len(jobs), n_slots)
+
+
+def scatter_pages(n_req_lens, page_size, seed):
+    """Random, interleaved pages for each request (never page 0)."""
+    rng = np.random.default_rng(seed)
+    need = [-(-n // page_size) for n in n_req_lens]
+    perm = rng.permutation(sum(need) + 3) + 1
+    tables, k = [], 0
+    for n in need:
+        tables.append([int(p) for p in perm[k:k + n]]); k += n
+    return tables, int(perm.max()) + 1
+
+
+def ref_rope(x, pos, inv_freq, interleaved):
+    T, H, D = x.shape
+    half = inv_freq.numel()
+    ang = pos.double()[:, None] * inv_freq.double()[None, :]
+    c, s = torch.cos(ang)[:, None, :], torch.sin(ang)[:, None, :]
+    y = x.double().clone()
+    i0 = torch.arange(half) * 2 if interleaved else torch.arange(half)
+    i1 = i0 + 1 if interleaved else i0 + half
+    y[..., i0] = x.double()[..., i0] * c - x.double()[..., i1] * s
+    y[..., i1] = x.double()[..., i0] * s + x.double()[..., i1] * c
+    return y
+
+
+@pytest.mark.parametrize("dt", ["float32", "bfloat16"])
+@pytest.mark.parametrize("H,Hk,D,rot,inter", [(4, 2, 16, 16, False), (3, 1, 48, 32, False), (6, 3, 80, 80, True), (8, 8, 128, 64, True)])
+def test_rope_kv_write(ops, dt, H, Hk, D, rot, inter):
+    ps = 8
+    starts, q_lens = [0, 13, 40], [9, 3, 1]
+    tables, n_pages = scatter_pages([s + n for s, n in zip(starts, q_lens)], ps, 1)
+    ctx = FakeCtx(starts, q_lens, tables, ps)
+    T = sum(q_lens)
+    Q, K = H * D, Hk * D
+    qkv = torch.randn(T, Q + 2 * K + 5, device=DEV)[:, :Q + 2 * K]          # a row stride that is not the width
+    inv = (10000.0 ** (-torch.arange(rot // 2, dtype=torch.float64) * 2 / rot)).float().to(DEV)
+    q_out = torch.empty(T, Q, device=DEV, dtype=DT[dt])
+    kc = torch.full((n_pages, Hk, ps, D), float("nan"), device=DEV, dtype=DT[dt])
+    vc = torch.full((n_pages, Hk, D, ps), float("nan"), device=DEV, dtype=DT[dt])
+    ops.rope_kv_write(qkv[:, :Q], qkv[:, Q:Q + K], qkv[:, Q + K:], q_out, kc, vc, ctx.positions, ctx.req_of_token,
+                      ctx.block_table(0), inv, H, Hk, D, rot, inter, 1.0, ps)
+    pos = ctx.positions.cpu()
+    want_q = ref_rope(qkv[:, :Q].cpu().reshape(T, H, D), pos, inv.cpu(), inter)
+    want_k = ref_rope(qkv[:, Q:Q + K].cpu().reshape(T, Hk, D), pos, inv.cpu(), inter)
+    tol = 2e-6 if dt == "float32" else 5e-3
+    assert rel(q_out.cpu().reshape(T, H, D), want_q) < tol
+    written = torch.zeros(n_pages, ps, dtype=torch.bool)
+    t = 0
+    for b, (s, n) in enumerate(zip(starts, q_lens)):
+        for p in range(s, s + n):
+            page, off = tables[b][p // ps], p % ps
+            assert rel(kc[page, :, off, :].cpu(), want_k[t]) < tol
+            assert rel(vc[page, :, :, off].cpu(), qkv[t, Q + K:].cpu().reshape(Hk, D).to(DT[dt])) == 0   # values as they are
+            written[page, off] = True
+            t += 1
+    assert torch.isnan(kc.float().cpu().permute(0, 2, 1, 3)[~written]).all()      # nothing else was touched
+    if rot < D:                                                               # channels beyond the rotary width pass through
+        assert torch.equal(q_out.cpu().reshape(T, H, D)[..., rot:], qkv[:, :Q].cpu().reshape(T, H, D)[..., rot:].to(DT[dt]))
+
+
+def ref_attention(q, k_seq, v_seq, starts, q_lens, scale, window):
+    """float64 attention per request; k_seq/v_seq[b]: [len, Hk, D] of the whole request."""
+    outs = []
+    t = 0
+    for b, (s, n) in enumerate(zip(starts, q_lens)):
+        k, v = k_seq[b].double(), v_seq[b].double()
+        H, Hk = q.shape[1], k.shape[1]
+        for i in range(n):
+            p = s + i
+            lo = max(0, p - window + 1) if window else 0
+            kk = k[lo:p + 1].repeat_interleave(H // Hk, dim=1)
+            vv = v[lo:p + 1].repeat_interleave(H // Hk, dim=1)
+            sc = torch.einsum("hd,thd->ht", q[t].double(), kk) * scale
+            pr = torch.softmax(sc, dim=-1)
+            outs.append(torch.einsum("ht,thd->hd", pr, vv))
+            t += 1
+    return torch.stack(outs)
+
+
+def fill_cache(k_seq, v_seq, tables, n_pages, ps, dt):
+    Hk, D = k_seq[0].shape[1:]
+    kc = torch.full((n_pages, Hk, ps, D), float("nan"), dtype=dt)
+    vc = torch.full((n_pages, Hk, D, ps), float("nan"), dtype=dt)
+    for b, (k, v) in enumerate(zip(k_seq, v_seq)):
+        for p in range(k.shape[0]):
+            kc[tables[b][p // ps], :, p % ps, :] = k[p].to(dt)
+            vc[tables[b][p // ps], :, :, p % ps] = v[p].to(dt)
+    return kc.to(DEV), vc.to(DEV)
+
+
+ATTN_CASES = [
+    # H, Hk, D, page, window, starts, q_lens
+    (4, 2, 16, 16, None, [0, 5, 100], [33, 1, 1]),
+    (3, 1, 32, 64, None, [0, 63, 64, 200], [70, 1, 2, 1]),
+    (8, 2, 128, 16, None, [300, 0, 17], [1, 40, 5]),
+    (6, 3, 48, 32, 24, [0, 90, 31], [50, 1, 3]),
+    (4, 4, 64, 16, 7, [40, 0], [1, 20]),
+    (5, 5, 80, 4, None, [10, 0], [3, 9]),          # small pages: the 32-bit kernel serves bfloat16 too
+    (2, 1, 24, 8, 5, [0, 30], [12, 1]),            # head size no multiple of 16
+    (32, 8, 128, 64, None, [2047, 1000], [1, 1]),  # decoding, long
+]
+
+
+@pytest.mark.parametrize("dt", ["float32", "bfloat16"])
+@pytest.mark.parametrize("case", ATTN_CASES)
+def test_attention(ops, dt, case):
+    H, Hk, D, ps, window, starts, q_lens = case
+    torch.manual_seed(H * 100 + D)
+    lens = [s + n for s, n in zip(starts, q_lens)]
+    tables, n_pages = scatter_pages(lens, ps, D)
+    ctx = FakeCtx(starts, q_lens, tables, ps)
+    T = sum(q_lens)
+    q = torch.randn(T, H, D).to(DT[dt])
+    k_seq = [torch.randn(n, Hk, D).to(DT[dt]) for n in lens]
+    v_seq = [torch.randn(n, Hk, D).to(DT[dt]) for n in lens]
+    kc, vc = fill_cache(k_seq, v_seq, tables, n_pages, ps, DT[dt])
+    scale = 1 / math.sqrt(D)
+    want = ref_attention(q.float(), [k.float() for k in k_seq], [v.float() for v in v_seq], starts, q_lens, scale, window)
+    got = ops.attention(q.to(DEV).reshape(T, H * D).contiguous(), kc, vc, ctx, 0, H, Hk, D, ps, scale, window)
+    got = got.cpu().reshape(T, H, D)
+    assert torch.isfinite(got.float()).all(), "read a slot no request owns"
+    assert rel(got, want) < (3e-6 if dt == "float32" else 1.2e-2)
+
+
+@pytest.mark.parametrize("dt", ["float32", "bfloat16"])
+@pytest.mark.parametrize("far", [0, 15, 16, 31, 32, 63, 64, 255, 256, 700, 1023])
+def test_attention_finds_one_far_key(ops, dt, far):
+    """One key among a thousand is made to stand out: the output must be its value row.
+    The key sits at the first slot, at page and tile edges, and at the last position."""
+    H, Hk, D, ps = 4, 2, 64, 16
+    n = 1024
+    torch.manual_seed(far)
+    tables, n_pages = scatter_pages([n], ps, far)
+    k = torch.randn(n, Hk, D) * 0.1
+    v = torch.randn(n, Hk, D)
+    q = torch.randn(1, H, D) * 0.1
+    q[0, :, :] += 4.0
+    k[far, :, :] += 4.0                      # score of `far` stands out by ~ 4*4*64/8
+    kc, vc = fill_cache([k], [v], tables, n_pages, ps, DT[dt])
+    ctx = FakeCtx([n - 1], [1], tables, ps)
+    got = ops.attention(q.to(DT[dt]).to(DEV).reshape(1, H * D), kc, vc, ctx, 0, H, Hk, D, ps, 1 / math.sqrt(D))
+    want = v.to(DT[dt]).float()[far].repeat_interleave(H // Hk, dim=0)
+    assert rel(got.cpu().reshape(H, D), want) < (1e-5 if dt == "float32" else 1e-2)
+
+
+@pytest.mark.parametrize("dt", ["float32", "bfloat16"])
+def test_attention_window_edge(ops, dt):
+    """The key just outside the window is made huge: it must not be seen; the one just inside must."""
+    H, Hk, D, ps, window = 2, 1, 32, 16, 20
+    n = 100
+    tables, n_pages = scatter_pages([n], ps, 3)
+    k = torch.randn(n, Hk, D) * 0.1
+    v = torch.randn(n, Hk, D)
+    q = torch.full((1, H, D), 2.0)
+    outside, inside = n - 1 - window, n - window
+    k[outside] += 50.0
+    kc, vc = fill_cache([k], [v], tables, n_pages, ps, DT[dt])
+    ctx = FakeCtx([n - 1], [1], tables, ps)
+    run = lambda kc_: ops.attention(q.to(DT[dt]).to(DEV).reshape(1, H * D), kc_, vc, ctx, 0, H, Hk, D, ps, 1 / math.sqrt(D), window).cpu().reshape(H, D)
+    got = run(kc)
+    assert rel(got, v.to(DT[dt]).float()[outside].expand(H, D)) > 0.1          # the outside key is not what we got
+    want = ref_attention(q.to(DT[dt]).float(), [k.to(DT[dt]).float()], [v.to(DT[dt]).float()], [n - 1], [1], 1 / math.sqrt(D), window)[0]
+    assert rel(got, want) < (3e-6 if dt == "float32" else 1.2e-2)
+    k2 = k.clone(); k2[inside] += 50.0
+    kc2, _ = fill_cache([k2], [v], tables, n_pages, ps, DT[dt])
+    assert rel(run(kc2), v.to(DT[dt]).float()[inside].expand(H, D)) < (1e-5 if dt == "float32" else 1e-2)
+
+
+def test_attention_plan_covers_every_key_once():
+    from xyntetik_runner_amd.engine.batch import plan_attention
+    for starts, q_lens, G, window, Hk in [([0, 100, 4000], [70, 1, 1], 4, None, 8), ([5000], [1], 4, None, 8),
+                                          ([0], [2048], 4, None, 8), ([300, 2], [1, 9], 2, 50, 1)]:
+        items, jobs, n_slots = plan_attention(starts, q_lens, G, window, Hk)
+        by_block = {}
+        for b, row0, k0, k1, slot, *_ in items:
+            assert k0 % 32 == 0 and k0 < k1
+            by_block.setdefault((b, row0), []).append((k0, k1, slot))
+        for (b, row0), parts in by_block.items():
+            parts.sort()
+            n = q_lens[b]
+            hi = starts[b] + min(n - 1, (row0 + 31) // G) + 1
+            lo = 0 if not window else max(0, starts[b] + row0 // G - window + 1)
+            assert parts[0][0] <= lo and parts[-1][1] == hi
+            assert all(a[1] == c[0] for a, c in zip(parts, parts[1:]))
+            assert (len(parts) == 1) == (parts[0][2] == -1)
+        slots = sorted(s for it in items if (s := it[4]) >= 0)
+        assert slots == list(range(n_slots))
+        assert sum(j[3] for j in jobs) == n_slots

@@ -1,0 +1,294 @@
+// Paged grouped-query attention on the gfx950 matrix cores, bfloat16 storage, for prompt
+// portions and decoded tokens in one launch.  Compiled once per head size (XR_HEAD_DIM,
+// a multiple of 16 up to 256).
+//
+// The formulas are the reference's (/root/reference/src/model.c:3548-3589: scores (q.k)*scale
+// over the keys a position may see, softmax with the maximum taken out, weighted values;
+// window bound :6326); the arrangement is not.  The query rows that share one key/value
+// head -- (token, head-in-group) pairs of one request -- are packed 32 to a block, so the
+// 4 heads of a decoded token, or 8 tokens x 4 heads of a prompt portion, read each key
+// and value once.  A wave takes one work item: a row block and a range of keys, listed
+// by the host.  For every tile of 32 keys it computes, transposed,
+//     S^T[key, row] = K[key, :] . Q[row, :]        v_mfma_f32_32x32x16_bf16, A = K tile
+//     O^T[d, row]  += V^T[d, key] * P^T[key, row]  A = V^T tile (values are cached transposed)
+// so that a lane owns one query row throughout: row maxima and sums are sums over the
+// lane's registers and one exchange with the lane 32 places away, and rescaling O^T is a
+// multiplication by the lane's own factor.  The key a tile row stands for is permuted so
+// that the 8 scores a lane holds for a block of 16 keys are the 8 keys the next MFMA
+// wants from it: P^T goes from accumulator to operand without leaving the lane.
+// Scores, maxima, sums and the output accumulate in 32-bit; P is rounded to bfloat16
+// for the second product.  Items that cover part of a row block's keys write partial
+// results that k_attn_merge combines (/root/reference/src/kernels.cu:2171-2270 does this
+// with 8 fixed slices for decoding).
+#include "common.h"
+
+#ifndef XR_HEAD_DIM
+#error "compile with -DXR_HEAD_DIM=<head size>"
+#endif
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+
+constexpr int HD = XR_HEAD_DIM;
+constexpr int KD = HD / 16;          // k-steps of the score product
+constexpr int DB = (HD + 31) / 32;   // 32-row blocks of O^T
+static_assert(HD % 16 == 0 && HD >= 16 && HD <= 256, "head size must be a multiple of 16 up to 256");
+
+#define ITEM_INTS 8                   // req, row0, k_begin, k_end, slot (-1: final), unused...
+#define ROWS 32
+
+struct AttnArgs {
+    const bf16_t* q;        // [T, H, HD]
+    const bf16_t* kc;       // [pages, Hk, page_size, HD]
+    const bf16_t* vc;       // [pages, Hk, HD, page_size]
+    bf16_t* out;            // [T, H, HD]
+    const int* items;       // [n_items, ITEM_INTS]
+    const int* cu_q;        // [B + 1] first row (token) of each request in this step
+    const int* starts;      // [B] position of each request's first token of this step
+    const int* block_table; // [B, table_stride]
+    int table_stride;
+    float* part_o;          // [slots, Hk, ROWS, HD]
+    float* part_ml;         // [slots, Hk, ROWS, 2]
+    int n_items, H, Hk, page_shift, page_mask, page_size;
+    float scale;
+    int window;
+};
+
+__device__ inline uint4 ldg16(const bf16_t* p) { return *reinterpret_cast<const uint4*>(p); }
+__device__ inline bf16x8 as_bf16x8(uint4 v) {
+    union { uint4 u; bf16x8 b; } c;
+    c.u = v;
+    return c.b;
+}
+__device__ inline uint32_t pack2(float lo, float hi) {
+    return (uint32_t)f32_to_bf16(lo) | ((uint32_t)f32_to_bf16(hi) << 16);
+}
+
+__global__ __launch_bounds__(256) void k_attn_mfma(AttnArgs a) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int item = blockIdx.x * 4 + wave;
+    if (item >= a.n_items) return;
+    const int kvh = blockIdx.y;
+    const int* it = a.items + (size_t)item * ITEM_INTS;
+    const int req = it[0], row0 = it[1], kbeg = it[2], kend = it[3], slot = it[4];
+    const int G = a.H / a.Hk;
+    const int lr = lane & 31, lg = lane >> 5;
+    const int q0 = a.cu_q[req], q_len = a.cu_q[req + 1] - q0;
+    const int start = a.starts[req];
+    const int seq_len = start + q_len;
+    const int* bt = a.block_table + (size_t)req * a.table_stride;
+
+    // this lane's query row
+    const int rho = row0 + lr;
+    const int tok = rho / G, hg = rho - tok * G;
+    const bool row_ok = tok < q_len;
+    const int t = q0 + tok, h = kvh * G + hg;
+    const int pos = start + tok;
+    const int lo = (a.window > 0 && pos - a.window + 1 > 0) ? pos - a.window + 1 : 0;
+
+    const uint4 zero = make_uint4(0, 0, 0, 0);
+    bf16x8 qf[KD];
+    {
+        const bf16_t* qp = a.q + ((size_t)t * a.H + h) * HD + lg * 8;
+#pragma unroll
+        for (int kd = 0; kd < KD; ++kd) qf[kd] = as_bf16x8(row_ok ? ldg16(qp + kd * 16) : zero);
+    }
+    // the key this lane's tile row stands for: r = 8a + 4g + b  ->  16(a/2) + 8g + 4(a%2) + b
+    const int ra = lr >> 3, rg = (lr >> 2) & 1, rb = lr & 3;
+    const int key_off = 16 * (ra >> 1) + 8 * rg + 4 * (ra & 1) + rb;
+
+    f32x16 o[DB];
+#pragma unroll
+    for (int d = 0; d < DB; ++d)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) o[d][e] = 0.f;
+    float m = -INFINITY, l = 0.f;
+
+    for (int kt = kbeg; kt < kend; kt += 32) {
+        // ---- S^T = K Q^T
+        f32x16 s;
+#pragma unroll
+        for (int e = 0; e < 16; ++e) s[e] = 0.f;
+        {
+            const int key = kt + key_off;
+            int page = -1;
+            if (key < seq_len) page = bt[key >> a.page_shift];
+            const bf16_t* kp = a.kc + (((size_t)(page < 0 ? 0 : page) * a.Hk + kvh) * a.page_size + (key & a.page_mask)) * HD + lg * 8;
+            uint4 kf[KD];
+#pragma unroll
+            for (int kd = 0; kd < KD; ++kd) kf[kd] = page >= 0 ? ldg16(kp + kd * 16) : zero;
+#pragma unroll
+            for (int kd = 0; kd < KD; ++kd)
+                s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16x8(kf[kd]), qf[kd], s, 0, 0, 0);
+        }
+        // ---- values for this tile (issued early; used after the softmax)
+        uint4 vf[2][DB];
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            const int k8 = kt + 16 * j + 8 * lg;            // first of this lane's 8 keys
+            int page = -1;
+            if (k8 < seq_len) page = bt[k8 >> a.page_shift];
+#pragma unroll
+            for (int d = 0; d < DB; ++d) {
+                const int dd = d * 32 + lr;
+                uint4 v = zero;
+                if (page >= 0 && dd < HD)
+                    v = ldg16(a.vc + (((size_t)page * a.Hk + kvh) * HD + dd) * a.page_size + (k8 & a.page_mask));
+                if (k8 + 8 > seq_len) {                      // slots past the request's end hold old data
+                    uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+                    for (int e = 0; e < 8; ++e)
+                        if (k8 + e >= seq_len) w[e >> 1] &= (e & 1) ? 0x0000FFFFu : 0xFFFF0000u;
+                    v = make_uint4(w[0], w[1], w[2], w[3]);
+                }
+                vf[j][d] = v;
+            }
+        }
+        // ---- mask, running maximum and sum
+        float p[16];
+        float mt = -INFINITY;
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+            const int key = kt + 16 * (e >> 3) + 8 * lg + (e & 7);
+            const bool ok = row_ok && key <= pos && key >= lo && key < kend;
+            p[e] = ok ? s[e] * a.scale : -INFINITY;
+            mt = fmaxf(mt, p[e]);
+        }
+        mt = fmaxf(mt, __shfl_xor(mt, 32, 64));
+        const float mn = fmaxf(m, mt);
+        const float mu = mn == -INFINITY ? 0.f : mn;
+        const float corr = expf(m - mu);
+        float rs = 0.f;
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+            p[e] = expf(p[e] - mu);
+            rs += p[e];
+        }
+        rs += __shfl_xor(rs, 32, 64);
+        l = l * corr + rs;
+        m = mn;
+#pragma unroll
+        for (int d = 0; d < DB; ++d)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) o[d][e] *= corr;
+        // ---- O^T += V^T P^T
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            uint4 pk = make_uint4(pack2(p[8 * j + 0], p[8 * j + 1]), pack2(p[8 * j + 2], p[8 * j + 3]),
+                                  pack2(p[8 * j + 4], p[8 * j + 5]), pack2(p[8 * j + 6], p[8 * j + 7]));
+            const bf16x8 pf = as_bf16x8(pk);
+#pragma unroll
+            for (int d = 0; d < DB; ++d)
+                o[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16x8(vf[j][d]), pf, o[d], 0, 0, 0);
+        }
+    }
+
+    // ---- write: lane owns row `rho`; register e of block d is channel d*32 + (e/4)*8 + lg*4 + e%4
+    const float inv = l > 0.f ? 1.0f / l : 0.f;
+    if (slot < 0) {
+        if (!row_ok) return;
+        bf16_t* op = a.out + ((size_t)t * a.H + h) * HD;
+#pragma unroll
+        for (int d = 0; d < DB; ++d)
+#pragma unroll
+            for (int e4 = 0; e4 < 4; ++e4) {
+                const int dd = d * 32 + e4 * 8 + lg * 4;
+                if (dd < HD) {
+                    uint2 w = make_uint2(pack2(o[d][e4 * 4 + 0] * inv, o[d][e4 * 4 + 1] * inv),
+                                         pack2(o[d][e4 * 4 + 2] * inv, o[d][e4 * 4 + 3] * inv));
+                    *reinterpret_cast<uint2*>(op + dd) = w;
+                }
+            }
+        return;
+    }
+    float* po = a.part_o + (((size_t)slot * a.Hk + kvh) * ROWS + lr) * HD;
+#pragma unroll
+    for (int d = 0; d < DB; ++d)
+#pragma unroll
+        for (int e4 = 0; e4 < 4; ++e4) {
+            const int dd = d * 32 + e4 * 8 + lg * 4;
+            if (dd < HD)
+                *reinterpret_cast<float4*>(po + dd) = make_float4(o[d][e4 * 4 + 0] * inv, o[d][e4 * 4 + 1] * inv,
+                                                                  o[d][e4 * 4 + 2] * inv, o[d][e4 * 4 + 3] * inv);
+        }
+    if (lg == 0) {
+        float* pm = a.part_ml + (((size_t)slot * a.Hk + kvh) * ROWS + lr) * 2;
+        pm[0] = m;
+        pm[1] = l;
+    }
+}
+
+// One merge job: {req, row0, first_slot, n_slots}.  Slot s holds the normalised output of
+// its keys with their maximum m_s and sum l_s; the whole is sum_s w_s O_s / sum_s w_s with
+// w_s = l_s * exp(m_s - max m).
+struct MergeArgs {
+    const int* jobs;        // [n_jobs, 4]
+    const int* cu_q;
+    const float* part_o;
+    const float* part_ml;
+    bf16_t* out;
+    int H, Hk;
+};
+
+__global__ __launch_bounds__(256) void k_attn_merge(MergeArgs a) {
+    const int* job = a.jobs + (size_t)blockIdx.x * 4;
+    const int req = job[0], row0 = job[1], s0 = job[2], ns = job[3];
+    const int kvh = blockIdx.y;
+    const int G = a.H / a.Hk;
+    const int q0 = a.cu_q[req], q_len = a.cu_q[req + 1] - q0;
+    for (int idx = threadIdx.x; idx < ROWS * (HD / 4); idx += 256) {
+        const int r = idx / (HD / 4), d4 = (idx % (HD / 4)) * 4;
+        const int rho = row0 + r;
+        const int tok = rho / G, hg = rho - tok * G;
+        if (tok >= q_len) continue;
+        float mx = -INFINITY;
+        for (int s = 0; s < ns; ++s) mx = fmaxf(mx, a.part_ml[(((size_t)(s0 + s) * a.Hk + kvh) * ROWS + r) * 2]);
+        float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+        float wsum = 0.f;
+        for (int s = 0; s < ns; ++s) {
+            const size_t base = ((size_t)(s0 + s) * a.Hk + kvh) * ROWS + r;
+            const float ms = a.part_ml[base * 2], ls = a.part_ml[base * 2 + 1];
+            if (!(ls > 0.f)) continue;
+            const float w = ls * expf(ms - mx);
+            const float4 v = *reinterpret_cast<const float4*>(a.part_o + base * HD + d4);
+            acc.x += w * v.x; acc.y += w * v.y; acc.z += w * v.z; acc.w += w * v.w;
+            wsum += w;
+        }
+        const float inv = wsum > 0.f ? 1.0f / wsum : 0.f;
+        bf16_t* op = a.out + ((size_t)(q0 + tok) * a.H + kvh * G + hg) * HD + d4;
+        *reinterpret_cast<uint2*>(op) = make_uint2(pack2(acc.x * inv, acc.y * inv), pack2(acc.z * inv, acc.w * inv));
+    }
+}
+
+extern "C" int xr_attn_head_dim() { return HD; }
+
+extern "C" int xr_attention_mfma(void* out, const void* q, const void* k_cache, const void* v_cache,
+                                 const int* items, int n_items, const int* jobs, int n_jobs, const int* cu_q,
+                                 const int* starts, const int* block_table, int table_stride, float* part_o,
+                                 float* part_ml, int H, int Hk, int D, int page_size, float scale, int window,
+                                 hipStream_t stream) {
+    XR_REQUIRE(D == HD, "attention: this library is compiled for head size %d, got %d", HD, D);
+    XR_REQUIRE(H > 0 && Hk > 0 && H % Hk == 0, "attention: %d query heads are not a multiple of %d key/value heads", H, Hk);
+    int shift = ilog2_exact(page_size);
+    XR_REQUIRE(shift >= 4, "attention: the MFMA kernel needs a page size that is a power of two of at least 16, got %d", page_size);
+    XR_REQUIRE(window >= 0, "attention: window %d is negative", window);
+    XR_REQUIRE(n_items >= 0 && n_jobs >= 0, "attention: negative work counts");
+    XR_REQUIRE(n_jobs == 0 || (part_o && part_ml && jobs), "attention: split work without partial buffers");
+    if (n_items == 0) return XR_OK;
+    AttnArgs a;
+    a.q = (const bf16_t*)q; a.kc = (const bf16_t*)k_cache; a.vc = (const bf16_t*)v_cache; a.out = (bf16_t*)out;
+    a.items = items; a.cu_q = cu_q; a.starts = starts; a.block_table = block_table; a.table_stride = table_stride;
+    a.part_o = part_o; a.part_ml = part_ml; a.n_items = n_items; a.H = H; a.Hk = Hk;
+    a.page_shift = shift; a.page_mask = page_size - 1; a.page_size = page_size; a.scale = scale; a.window = window;
+    dim3 grid((n_items + 3) / 4, Hk);
+    k_attn_mfma<<<grid, 256, 0, stream>>>(a);
+    XR_CHECK_LAUNCH("attention_mfma");
+    if (n_jobs > 0) {
+        MergeArgs mg;
+        mg.jobs = jobs; mg.cu_q = cu_q; mg.part_o = part_o; mg.part_ml = part_ml; mg.out = (bf16_t*)out;
+        mg.H = H; mg.Hk = Hk;
+        k_attn_merge<<<dim3(n_jobs, Hk), 256, 0, stream>>>(mg);
+        XR_CHECK_LAUNCH("attention_merge");
+    }
+    return XR_OK;
+}

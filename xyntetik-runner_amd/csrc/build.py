@@ -35,7 +35,7 @@ HIPCC_FLAGS = [
 UNITS: Dict[str, dict] = {
     "kernels": {
         "sources": ["errors.hip", "basic_kernels.hip", "gemm_ref.hip", "attention_ref.hip",
-                    "sampling.hip"],
+                    "sampling.hip", "gemm_mfma.hip"],
         "defines": [],
     },
 }

@@ -1,0 +1,372 @@
+// bfloat16 matrix products on the gfx950 matrix cores, 32-bit accumulation:
+//   out[M,N] = a[M,K] * w[N,K]^T (+ bias)        (weights [n_out][n_in], row-major)
+// Two kernels share the epilogues:
+//   * k_gemm_tile:   large M (prompt portions).  A workgroup computes a BM x BN tile; both
+//     operands are staged through LDS in 64-wide K slices (16-byte chunks, XOR-swizzled
+//     so that fragment reads do not collide), double-buffered, and fed to
+//     v_mfma_f32_32x32x16_bf16.
+//   * k_gemm_skinny: M <= 64 (decoding).  The product is bound by reading the weights
+//     once, so each wave streams 16 weight rows straight from memory into MFMA fragments
+//     (v_mfma_f32_16x16x32_bf16, weights as the A operand, tokens as the B operand) with
+//     many loads in flight, the few activation rows come through LDS, and the waves of a
+//     workgroup split K among themselves.
+// Epilogues: store (float or bfloat16), add into a float output (the residual stream),
+// and SwiGLU: with w = [gate rows; up rows] the kernel writes silu(gate) * up, so the
+// [M, 2F] intermediate never reaches memory (/root/reference/src/model.c:6399-6404).
+// The reference's float-weight "GEMM" is a multi-column matvec (/root/reference/src/kernels.cu:116-144);
+// its tensor-core kernels (:856) exist for quantised weights only.
+#include "common.h"
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+#define EPI_STORE 0
+#define EPI_ACCUM 1
+#define EPI_SWIGLU 2
+
+struct GemmArgs {
+    const bf16_t* a;   // [M, lda]
+    const bf16_t* w;   // [N or 2N, K]
+    const float* bias; // [N] (or [2N] for SwiGLU) or null
+    void* out;         // [M, ldo]
+    int M, N, K, lda, ldo;
+    int out_bf16;      // storage of out
+    int epi;
+};
+
+__device__ inline uint4 ldg16(const bf16_t* p) { return *reinterpret_cast<const uint4*>(p); }
+__device__ inline bf16x8 as_bf16x8(uint4 v) {
+    union { uint4 u; bf16x8 b; } c;
+    c.u = v;
+    return c.b;
+}
+__device__ inline float silu_f(float g) { return g / (1.0f + expf(-g)); }
+
+__device__ inline void store_out(const GemmArgs& g, int m, int n, float v) {
+    size_t o = (size_t)m * g.ldo + n;
+    if (g.epi == EPI_ACCUM) {
+        float* p = (float*)g.out;
+        p[o] = p[o] + v;
+    } else if (g.out_bf16) {
+        ((bf16_t*)g.out)[o] = f32_to_bf16(v);
+    } else {
+        ((float*)g.out)[o] = v;
+    }
+}
+
+// ------------------------------------------------------------------------------ tile kernel
+// Row r (0..BN-1) of the weight tile of workgroup bx -> row of w.  Plain: n0 + r.  SwiGLU:
+// each wave's 32-column MFMA tiles alternate gate, up, gate, up ... so that the two values
+// of one output column meet in the same lane and register.
+template <int BN, int WN>
+__device__ inline int w_row_of(int r, int bx, int N, int epi, int& out_col) {
+    if (epi != EPI_SWIGLU) {
+        out_col = bx * BN + r;
+        return out_col;
+    }
+    const int wn = r / WN, t = (r % WN) / 32, c = r % 32;
+    out_col = bx * (BN / 2) + (wn * (WN / 64) + t / 2) * 32 + c;
+    return (t & 1) ? N + out_col : out_col;
+}
+
+template <int BM, int BN, int WARPS_M, int WARPS_N>
+__global__ __launch_bounds__(64 * WARPS_M * WARPS_N) void k_gemm_tile(GemmArgs g) {
+    constexpr int THREADS = 64 * WARPS_M * WARPS_N;
+    constexpr int BK = 64, CH = BK / 8;                 // 8 chunks of 16 bytes per row
+    constexpr int WM = BM / WARPS_M, WN = BN / WARPS_N;
+    constexpr int TM = WM / 32, TN = WN / 32;
+    constexpr int A_CHUNKS = BM * CH / THREADS, W_CHUNKS = BN * CH / THREADS;
+    static_assert(BM * CH % THREADS == 0 && BN * CH % THREADS == 0, "tile does not divide among threads");
+    extern __shared__ uint4 lds[];                      // [2][(BM + BN) * CH]
+    constexpr int BUF = (BM + BN) * CH;                 // chunks per buffer; weights follow activations
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm0 = (wave / WARPS_N) * WM, wn0 = (wave % WARPS_N) * WN;
+    const int m0 = blockIdx.y * BM;
+    const int bx = blockIdx.x;
+    const int n_rows = g.epi == EPI_SWIGLU ? 2 * g.N : g.N;
+
+    // which rows this thread stages
+    int a_row[A_CHUNKS], a_c[A_CHUNKS];
+    const bf16_t* a_ptr[A_CHUNKS];
+#pragma unroll
+    for (int i = 0; i < A_CHUNKS; ++i) {
+        int q = tid + i * THREADS;
+        a_row[i] = q / CH; a_c[i] = q % CH;
+        int m = m0 + a_row[i];
+        a_ptr[i] = m < g.M ? g.a + (size_t)m * g.lda + a_c[i] * 8 : nullptr;
+    }
+    int w_row[W_CHUNKS], w_c[W_CHUNKS];
+    const bf16_t* w_ptr[W_CHUNKS];
+#pragma unroll
+    for (int i = 0; i < W_CHUNKS; ++i) {
+        int q = tid + i * THREADS;
+        w_row[i] = q / CH; w_c[i] = q % CH;
+        int oc;
+        int n = w_row_of<BN, WN>(w_row[i], bx, g.N, g.epi, oc);
+        w_ptr[i] = (oc < g.N && n < n_rows) ? g.w + (size_t)n * g.K + w_c[i] * 8 : nullptr;
+    }
+
+    f32x16 acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+
+    uint4 ra[A_CHUNKS], rw[W_CHUNKS];
+    const uint4 zero = make_uint4(0, 0, 0, 0);
+    auto load_global = [&](int k0) {
+#pragma unroll
+        for (int i = 0; i < A_CHUNKS; ++i)
+            ra[i] = (a_ptr[i] && k0 + a_c[i] * 8 < g.K) ? ldg16(a_ptr[i] + k0) : zero;
+#pragma unroll
+        for (int i = 0; i < W_CHUNKS; ++i)
+            rw[i] = (w_ptr[i] && k0 + w_c[i] * 8 < g.K) ? ldg16(w_ptr[i] + k0) : zero;
+    };
+    auto store_lds = [&](int buf) {
+#pragma unroll
+        for (int i = 0; i < A_CHUNKS; ++i) lds[buf * BUF + a_row[i] * CH + (a_c[i] ^ (a_row[i] & 7))] = ra[i];
+#pragma unroll
+        for (int i = 0; i < W_CHUNKS; ++i) lds[buf * BUF + BM * CH + w_row[i] * CH + (w_c[i] ^ (w_row[i] & 7))] = rw[i];
+    };
+
+    const int nk = (g.K + BK - 1) / BK;
+    load_global(0);
+    store_lds(0);
+    __syncthreads();
+    const int lr = lane & 31, lg = lane >> 5;
+    for (int kt = 0; kt < nk; ++kt) {
+        const int buf = kt & 1;
+        if (kt + 1 < nk) load_global((kt + 1) * BK);
+#pragma unroll
+        for (int ks = 0; ks < BK / 16; ++ks) {
+            bf16x8 af[TM], wf[TN];
+            const int c = ks * 2 + lg;
+#pragma unroll
+            for (int i = 0; i < TM; ++i) {
+                int r = wm0 + i * 32 + lr;
+                af[i] = as_bf16x8(lds[buf * BUF + r * CH + (c ^ (r & 7))]);
+            }
+#pragma unroll
+            for (int j = 0; j < TN; ++j) {
+                int r = wn0 + j * 32 + lr;
+                wf[j] = as_bf16x8(lds[buf * BUF + BM * CH + r * CH + (c ^ (r & 7))]);
+            }
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int j = 0; j < TN; ++j)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[i], wf[j], acc[i][j], 0, 0, 0);
+        }
+        if (kt + 1 < nk) store_lds(buf ^ 1);
+        __syncthreads();
+    }
+
+    // epilogue: lane holds column (lane % 32), rows (e/4)*8 + (lane/32)*4 + e%4 of each 32x32 tile
+    if (g.epi == EPI_SWIGLU) {
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j + 1 < TN; j += 2) {
+                int oc;
+                w_row_of<BN, WN>(wn0 + j * 32 + lr, bx, g.N, g.epi, oc);
+                if (oc >= g.N) continue;
+                float bg = g.bias ? g.bias[oc] : 0.f, bu = g.bias ? g.bias[g.N + oc] : 0.f;
+#pragma unroll
+                for (int e = 0; e < 16; ++e) {
+                    int m = m0 + wm0 + i * 32 + (e / 4) * 8 + lg * 4 + (e % 4);
+                    if (m < g.M) store_out(g, m, oc, silu_f(acc[i][j][e] + bg) * (acc[i][j + 1][e] + bu));
+                }
+            }
+        return;
+    }
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+            int n = bx * BN + wn0 + j * 32 + lr;
+            if (n >= g.N) continue;
+            float b = g.bias ? g.bias[n] : 0.f;
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+                int m = m0 + wm0 + i * 32 + (e / 4) * 8 + lg * 4 + (e % 4);
+                if (m < g.M) store_out(g, m, n, acc[i][j][e] + b);
+            }
+        }
+}
+
+// ------------------------------------------------------------------------------ skinny kernel
+// MT: 16-token groups (M <= 16*MT).  RT: groups of 16 weight rows per wave.  KSW: waves per
+// workgroup; they split K into contiguous slices, so a workgroup owns 16*RT output columns
+// and all of K, and no sum crosses workgroups.  A wave issues the weight loads (16 bytes a
+// lane, straight into MFMA A fragments) and the activation loads (B fragments, served by
+// L2) of U k-steps of 32 before it uses them; with N/(16*RT) workgroups of KSW waves this
+// keeps tens of kilobytes in flight on every compute unit.  The slices are summed through
+// LDS in a fixed order.
+template <int MT, int RT, int KSW, int U, bool SWIGLU>
+__global__ __launch_bounds__(64 * KSW) void k_gemm_skinny(GemmArgs g) {
+    constexpr int NWT = SWIGLU ? 2 : 1;  // weight fragments per row group (gate and up)
+    constexpr int MTOK = MT * 16, ROWS = RT * 16, THREADS = 64 * KSW;
+    extern __shared__ float red[];       // [KSW][NWT][ROWS][MTOK]
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int l16 = lane & 15, lq = lane >> 4;
+    const int n_base = blockIdx.x * ROWS;
+    const int steps_total = (g.K + 31) / 32;
+    const int steps_per = (steps_total + KSW - 1) / KSW;
+    const int kbeg = wave * steps_per * 32;
+    const int kend_ = kbeg + steps_per * 32;
+    const int kend = kend_ < g.K ? kend_ : g.K;
+
+    const bf16_t* wp[NWT][RT];
+    bool w_ok[RT];
+#pragma unroll
+    for (int r = 0; r < RT; ++r) {
+        int n = n_base + r * 16 + l16;
+        w_ok[r] = n < g.N;
+        wp[0][r] = g.w + (size_t)(w_ok[r] ? n : 0) * g.K;
+        if (SWIGLU) wp[NWT - 1][r] = g.w + (size_t)(g.N + (w_ok[r] ? n : 0)) * g.K;
+    }
+    const bf16_t* ap[MT];
+    bool a_ok[MT];
+#pragma unroll
+    for (int i = 0; i < MT; ++i) {
+        int tok = i * 16 + l16;
+        a_ok[i] = tok < g.M;
+        ap[i] = g.a + (size_t)(a_ok[i] ? tok : 0) * g.lda;
+    }
+
+    f32x4 acc[NWT][RT][MT];
+#pragma unroll
+    for (int t = 0; t < NWT; ++t)
+#pragma unroll
+        for (int r = 0; r < RT; ++r)
+#pragma unroll
+            for (int i = 0; i < MT; ++i) acc[t][r][i] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    const uint4 zero = make_uint4(0, 0, 0, 0);
+    for (int k0 = kbeg; k0 < kend; k0 += 32 * U) {
+        uint4 wreg[U][NWT][RT], areg[U][MT];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int k = k0 + u * 32 + lq * 8;
+            const bool k_ok = k < kend;
+#pragma unroll
+            for (int r = 0; r < RT; ++r)
+#pragma unroll
+                for (int t = 0; t < NWT; ++t)
+                    wreg[u][t][r] = (k_ok && w_ok[r]) ? ldg16(wp[t][r] + k) : zero;
+#pragma unroll
+            for (int i = 0; i < MT; ++i) areg[u][i] = (k_ok && a_ok[i]) ? ldg16(ap[i] + k) : zero;
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+#pragma unroll
+            for (int i = 0; i < MT; ++i) {
+                const bf16x8 af = as_bf16x8(areg[u][i]);
+#pragma unroll
+                for (int r = 0; r < RT; ++r)
+#pragma unroll
+                    for (int t = 0; t < NWT; ++t)
+                        acc[t][r][i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(wreg[u][t][r]), af,
+                                                                                acc[t][r][i], 0, 0, 0);
+            }
+    }
+
+    // acc[t][r][i][e]: weight row r*16 + 4*(lane/16) + e of the workgroup's ROWS, token i*16 + lane%16
+#pragma unroll
+    for (int t = 0; t < NWT; ++t)
+#pragma unroll
+        for (int r = 0; r < RT; ++r)
+#pragma unroll
+            for (int i = 0; i < MT; ++i)
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                    red[((wave * NWT + t) * ROWS + r * 16 + lq * 4 + e) * MTOK + i * 16 + l16] = acc[t][r][i][e];
+    __syncthreads();
+    for (int q = tid; q < ROWS * MTOK; q += THREADS) {
+        int col = q % ROWS, tok = q / ROWS;          // consecutive threads write consecutive columns
+        int nn = n_base + col;
+        if (tok >= g.M || nn >= g.N) continue;
+        float v[NWT];
+#pragma unroll
+        for (int t = 0; t < NWT; ++t) {
+            float s = 0.f;
+#pragma unroll
+            for (int k = 0; k < KSW; ++k) s += red[((k * NWT + t) * ROWS + col) * MTOK + tok];
+            v[t] = s;
+        }
+        if (SWIGLU) {
+            float bg = g.bias ? g.bias[nn] : 0.f, bu = g.bias ? g.bias[g.N + nn] : 0.f;
+            store_out(g, tok, nn, silu_f(v[0] + bg) * (v[NWT - 1] + bu));
+        } else {
+            store_out(g, tok, nn, v[0] + (g.bias ? g.bias[nn] : 0.f));
+        }
+    }
+}
+
+template <int MT, int RT, int KSW, int U, bool SW>
+static int launch_skinny(const GemmArgs& g, hipStream_t stream) {
+    constexpr int NWT = SW ? 2 : 1;
+    size_t smem = (size_t)KSW * NWT * RT * 16 * MT * 16 * 4;
+    static bool attr_set = false;
+    if (!attr_set) {
+        hipError_t e = hipFuncSetAttribute((const void*)k_gemm_skinny<MT, RT, KSW, U, SW>,
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+        if (e != hipSuccess) { xr_set_error("gemm: cannot reserve %zu bytes of LDS: %s", smem, hipGetErrorString(e)); return XR_LAUNCH; }
+        attr_set = true;
+    }
+    unsigned blocks = (unsigned)((g.N + 16 * RT - 1) / (16 * RT));
+    k_gemm_skinny<MT, RT, KSW, U, SW><<<blocks, 64 * KSW, smem, stream>>>(g);
+    XR_CHECK_LAUNCH("gemm_skinny");
+    return XR_OK;
+}
+
+template <int BM, int BN, int WM_, int WN_>
+static int launch_tile(const GemmArgs& g, hipStream_t stream) {
+    size_t smem = (size_t)2 * (BM + BN) * 8 * 16;
+    static bool attr_set = false;
+    if (!attr_set) {
+        hipError_t e = hipFuncSetAttribute((const void*)k_gemm_tile<BM, BN, WM_, WN_>,
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+        if (e != hipSuccess) { xr_set_error("gemm: cannot reserve %zu bytes of LDS: %s", smem, hipGetErrorString(e)); return XR_LAUNCH; }
+        attr_set = true;
+    }
+    int n_out_tile = g.epi == EPI_SWIGLU ? BN / 2 : BN;
+    dim3 grid((g.N + n_out_tile - 1) / n_out_tile, (g.M + BM - 1) / BM);
+    k_gemm_tile<BM, BN, WM_, WN_><<<grid, 64 * WM_ * WN_, smem, stream>>>(g);
+    XR_CHECK_LAUNCH("gemm_tile");
+    return XR_OK;
+}
+
+// epi: 0 store, 1 add into float out, 2 SwiGLU (w has 2N rows: gate rows then up rows).
+// variant: 0 = choose by M; 1 = skinny; 2 = tile 128x128; 3 = tile 256x128.
+extern "C" int xr_gemm_bf16(void* out, const void* a, const void* w, const float* bias, int M, int N, int K,
+                            int lda, int ldo, int out_dtype, int epi, int variant, hipStream_t stream) {
+    XR_REQUIRE(M >= 0 && N > 0 && K > 0, "gemm: bad sizes M=%d N=%d K=%d", M, N, K);
+    XR_REQUIRE(lda >= K && ldo >= N, "gemm: row strides lda=%d ldo=%d are shorter than K=%d N=%d", lda, ldo, K, N);
+    XR_REQUIRE(K % 8 == 0 && lda % 8 == 0, "gemm: the MFMA kernels need K (%d) and the row stride (%d) to be multiples of 8", K, lda);
+    XR_REQUIRE(((uintptr_t)a % 16) == 0 && ((uintptr_t)w % 16) == 0, "gemm: operands must be 16-byte aligned");
+    XR_REQUIRE(epi >= 0 && epi <= 2, "gemm: unknown epilogue %d", epi);
+    XR_REQUIRE(epi != EPI_ACCUM || out_dtype == XR_F32, "gemm: accumulation needs a 32-bit output");
+    XR_REQUIRE(out_dtype == XR_F32 || out_dtype == XR_BF16, "gemm: bad output dtype %d", out_dtype);
+    if (M == 0) return XR_OK;
+    GemmArgs g;
+    g.a = (const bf16_t*)a; g.w = (const bf16_t*)w; g.bias = bias; g.out = out;
+    g.M = M; g.N = N; g.K = K; g.lda = lda; g.ldo = ldo; g.out_bf16 = out_dtype == XR_BF16; g.epi = epi;
+    const bool sw = epi == EPI_SWIGLU;
+    if (variant == 0) variant = M <= 64 ? 1 : 2;
+    if (variant == 1) {
+        XR_REQUIRE(M <= 64, "gemm: the skinny kernel takes at most 64 rows, got %d", M);
+        if (M <= 16) return sw ? launch_skinny<1, 1, 16, 8, true>(g, stream) : launch_skinny<1, 1, 16, 8, false>(g, stream);
+        if (M <= 32) return sw ? launch_skinny<2, 1, 16, 8, true>(g, stream) : launch_skinny<2, 1, 16, 8, false>(g, stream);
+        return sw ? launch_skinny<4, 2, 8, 4, true>(g, stream) : launch_skinny<4, 2, 8, 4, false>(g, stream);
+    }
+    if (variant == 2) return launch_tile<128, 128, 2, 2>(g, stream);
+    if (variant == 3) return launch_tile<256, 128, 4, 2>(g, stream);
+    xr_set_error("gemm: unknown variant %d", variant);
+    return XR_BAD_ARG;
+}

@@ -42,6 +42,7 @@ _PROTOS = {
     "xr_fill_rows": [_p, _p, _i, _sz, _u32, _p],
     "xr_convert": [_p, _p, _sz, _i, _i, _p],
     "xr_gemm_ref": [_p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _p],
+    "xr_gemm_bf16": [_p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _p],
     "xr_attention_ref": [_p, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _f, _i, _i, _p],
     "xr_sample": [_p, _p, _i, _i, _i, _p, _p, _p, _p, _p, _p, _p, _p, _i, _p, _i, _p],
 }
@@ -159,10 +160,18 @@ class Ops:
         return out
 
     # -- matrix product ---------------------------------------------------------
+    def _mfma_ok(self, a: torch.Tensor, w: torch.Tensor) -> bool:
+        return (self.use_mfma and a.dtype == torch.bfloat16 and a.shape[1] % 8 == 0 and a.stride(0) % 8 == 0
+                and a.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0)
+
     def linear(self, a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None,
                out_dtype: Optional[torch.dtype] = None, out: Optional[torch.Tensor] = None,
-               accumulate: bool = False) -> torch.Tensor:
-        """``a [M, K] @ w [N, K]^T (+ bias)``; with ``accumulate`` added into 32-bit ``out``."""
+               accumulate: bool = False, variant: int = 0) -> torch.Tensor:
+        """``a [M, K] @ w [N, K]^T (+ bias)``; with ``accumulate`` added into 32-bit ``out``.
+
+        bfloat16 operands run on the matrix cores (32-bit accumulation); float32 operands, and
+        shapes the MFMA kernels do not take, run the plain 32-bit FMA kernel.
+        """
         self._dev(a, w, bias, out)
         if a.dim() != 2 or w.dim() != 2 or a.shape[1] != w.shape[1]:
             raise KernelError(f"linear: shapes {tuple(a.shape)} x {tuple(w.shape)}^T do not fit")
@@ -181,10 +190,35 @@ class Ops:
             raise KernelError(f"linear: output is {tuple(out.shape)}, product is {(M, N)}")
         if bias is not None and (bias.dtype != torch.float32 or bias.numel() != N):
             raise KernelError("linear: bias must be float32 [N]")
+        if self._mfma_ok(a, w):
+            self.lib.check(self.lib.xr_gemm_bf16(out.data_ptr(), a.data_ptr(), w.data_ptr(), _ptr(bias), M, N, K,
+                                                 a.stride(0), out.stride(0), dtype_code(out.dtype),
+                                                 1 if accumulate else 0, variant, _stream()))
+            return out
         self.lib.check(self.lib.xr_gemm_ref(out.data_ptr(), a.data_ptr(), w.data_ptr(), _ptr(bias), M, N, K,
                                             a.stride(0), out.stride(0), dtype_code(a.dtype),
                                             dtype_code(out.dtype), 1 if accumulate else 0, _stream()))
         return out
+
+    def linear_swiglu(self, a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None,
+                      variant: int = 0) -> torch.Tensor:
+        """``silu(a @ w[:F]^T) * (a @ w[F:]^T)`` for ``w [2F, K]`` = gate rows then up rows."""
+        F = w.shape[0] // 2
+        if w.shape[0] % 2:
+            raise KernelError("linear_swiglu: the weight must have an even number of rows")
+        if self._mfma_ok(a, w):
+            self._dev(a, w, bias)
+            self._contig(w, "linear_swiglu weight")
+            M, K = a.shape
+            if K != w.shape[1] or a.stride(1) != 1:
+                raise KernelError(f"linear_swiglu: shapes {tuple(a.shape)} x {tuple(w.shape)}^T do not fit")
+            if bias is not None and (bias.dtype != torch.float32 or bias.numel() != 2 * F):
+                raise KernelError("linear_swiglu: bias must be float32 [2F]")
+            out = torch.empty((M, F), dtype=a.dtype, device=a.device)
+            self.lib.check(self.lib.xr_gemm_bf16(out.data_ptr(), a.data_ptr(), w.data_ptr(), _ptr(bias), M, F, K,
+                                                 a.stride(0), F, dtype_code(out.dtype), 2, variant, _stream()))
+            return out
+        return self.silu_mul(self.linear(a, w, bias=bias))
 
     # -- attention --------------------------------------------------------------
     def rope_kv_write(self, q_in, k_in, v_in, q_out, k_cache, v_cache, positions, req_of_token,
@@ -212,20 +246,51 @@ class Ops:
             block_table.stride(0) if block_table is not None else 0, _ptr(inv_freq), T, H, Hk, D, rot,
             1 if interleaved else 0, float(mscale), page_size, dtype_code(store.dtype), _stream()))
 
-    def attention(self, q, k_cache, v_cache, positions, req_of_token, block_table, H: int, Hk: int,
-                  D: int, page_size: int, scale: float, window: Optional[int] = None) -> torch.Tensor:
-        """Causal attention of every token over its request's cached keys and values."""
+    def attention(self, q, k_cache, v_cache, ctx, group: int, H: int, Hk: int, D: int, page_size: int,
+                  scale: float, window: Optional[int] = None) -> torch.Tensor:
+        """Causal attention of every token of the step over its request's cached keys and values.
+
+        bfloat16 runs on the matrix cores (head sizes in steps of 16 up to 256, pages of at least
+        16 positions); float32, and what the MFMA kernel does not take, runs the 32-bit kernel.
+        """
+        positions, req_of_token, block_table = ctx.positions, ctx.req_of_token, ctx.block_table(group)
         self._dev(q, k_cache, v_cache, positions, req_of_token, block_table)
         T = positions.numel()
         self._contig(q, "attention queries")
         if q.dtype != k_cache.dtype or q.dtype != v_cache.dtype:
             raise KernelError("attention: queries and cache differ in dtype")
+        if H % Hk:
+            raise KernelError(f"attention: {H} query heads are not a multiple of {Hk} key/value heads")
         out = torch.empty((T, H * D), dtype=q.dtype, device=q.device)
+        if self.use_mfma and q.dtype == torch.bfloat16 and D % 16 == 0 and 16 <= D <= 256 and page_size >= 16:
+            lib = self.attention_lib(D)
+            plan = ctx.attention_plan(group, H // Hk, window, Hk)
+            part_o = part_ml = None
+            if plan.n_slots:
+                part_o = torch.empty((plan.n_slots, Hk, 32, D), dtype=torch.float32, device=q.device)
+                part_ml = torch.empty((plan.n_slots, Hk, 32, 2), dtype=torch.float32, device=q.device)
+            lib.check(lib.xr_attention_mfma(
+                out.data_ptr(), q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), plan.items.data_ptr(),
+                plan.n_items, _ptr(plan.jobs), plan.n_jobs, ctx.cu_q.data_ptr(), ctx.starts_dev.data_ptr(),
+                block_table.data_ptr(), block_table.stride(0), _ptr(part_o), _ptr(part_ml), H, Hk, D, page_size,
+                float(scale), int(window or 0), _stream()))
+            return out
         self.lib.check(self.lib.xr_attention_ref(
             out.data_ptr(), q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), positions.data_ptr(),
             req_of_token.data_ptr(), block_table.data_ptr(), block_table.stride(0), T, H, Hk, D, page_size,
             float(scale), int(window or 0), dtype_code(q.dtype), _stream()))
         return out
+
+    def attention_lib(self, D: int) -> "_Lib":
+        """The MFMA attention library for head size ``D`` (compiled at first use)."""
+        lib = self._attn_libs.get(D)
+        if lib is None:
+            unit = f"attn_d{D}"
+            path = _build.find_built(unit) or _build.build_unit(unit)
+            lib = _Lib(path, {"xr_attention_mfma": [_p, _p, _p, _p, _p, _i, _p, _i, _p, _p, _p, _i, _p, _p,
+                                                    _i, _i, _i, _i, _f, _i, _p]})
+            self._attn_libs[D] = lib
+        return lib
 
     # -- sampling ---------------------------------------------------------------
     def sample(self, logits, temp, draw, top_k=None, top_p=None, min_p=None, repeat_penalty=None,

@@ -21,6 +21,63 @@ import torch
 
 
 @dataclass
+class AttentionPlan:
+    """The work list of the MFMA attention kernel for one step, cache group, group size and window.
+
+    ``items [n, 8]`` int32 on the device: request, first row of a 32-row block, first key,
+    end key, partial slot (-1: the item covers all keys of its block and writes the output).
+    ``jobs [m, 4]``: request, first row, first slot, number of slots to merge.
+    """
+    items: torch.Tensor
+    n_items: int
+    jobs: Optional[torch.Tensor]
+    n_jobs: int
+    n_slots: int
+
+
+ATTN_ROWS = 32          # query rows (token x head-in-group) per work item
+ATTN_TILE = 32          # keys per tile; items begin and end on tile edges
+ATTN_TARGET_WAVES = 2048
+ATTN_MIN_TILES = 4
+
+
+def plan_attention(starts, q_lens, group_size: int, window: Optional[int], n_kv_heads: int):
+    """Host side of ``AttentionPlan``: lists of items and merge jobs (plain Python ints)."""
+    blocks = []
+    total_tiles = 0
+    for b, (s, n) in enumerate(zip(starts, q_lens)):
+        rows = n * group_size
+        for row0 in range(0, rows, ATTN_ROWS):
+            tok_lo = row0 // group_size
+            tok_hi = min(n - 1, (row0 + ATTN_ROWS - 1) // group_size)
+            lo = 0 if not window else max(0, s + tok_lo - window + 1)
+            lo = (lo // ATTN_TILE) * ATTN_TILE
+            hi = s + tok_hi + 1
+            tiles = -(-(hi - lo) // ATTN_TILE)
+            blocks.append((b, row0, lo, hi, tiles))
+            total_tiles += tiles
+    chunk = 1 << 30
+    if blocks and len(blocks) * n_kv_heads < ATTN_TARGET_WAVES:
+        chunk = max(ATTN_MIN_TILES, -(-total_tiles * n_kv_heads // ATTN_TARGET_WAVES))
+    items, jobs, slot = [], [], 0
+    for b, row0, lo, hi, tiles in blocks:
+        parts = -(-tiles // chunk)
+        if parts <= 1:
+            items.append((b, row0, lo, hi, -1, 0, 0, 0))
+            continue
+        per = -(-tiles // parts)
+        first = slot
+        k = lo
+        while k < hi:
+            e = min(hi, k + per * ATTN_TILE)
+            items.append((b, row0, k, e, slot, 0, 0, 0))
+            slot += 1
+            k = e
+        jobs.append((b, row0, first, slot - first))
+    return items, jobs, slot
+
+
+@dataclass
 class StepEntry:
     req_id: Hashable
     tokens: Sequence[int]
@@ -57,7 +114,7 @@ class StepContext:
 
         # ---- pack: [token_ids T][positions T][req_of_token T][cu_q B+1][seq_lens B][slots B][fresh B]
         #            [want W][table g: B * width_g]...
-        sizes = [T, T, T, B + 1, B, B, B, self.n_want] + [B * w for w in self.table_width]
+        sizes = [T, T, T, B + 1, B, B, B + B, self.n_want] + [B * w for w in self.table_width]
         offs = np.concatenate([[0], np.cumsum(sizes)]).astype(np.int64)
         total = int(offs[-1])
         host = torch.empty((max(total, 1),), dtype=torch.int32, pin_memory=True)
@@ -74,7 +131,8 @@ class StepContext:
             cu[b + 1] = r
         h[offs[4]:offs[5]] = self.seq_lens
         h[offs[5]:offs[6]] = [rc.slot for rc in request_caches]
-        h[offs[6]:offs[7]] = [1 if rc.fresh else 0 for rc in request_caches]
+        h[offs[6]:offs[6] + B] = [1 if rc.fresh else 0 for rc in request_caches]
+        h[offs[6] + B:offs[7]] = self.starts
         h[offs[7]:offs[8]] = want_rows
         for g in range(n_groups):
             w = self.table_width[g]
@@ -91,10 +149,27 @@ class StepContext:
         self.cu_q = dev[offs[3]:offs[4]]
         self.seq_lens_dev = dev[offs[4]:offs[5]]
         self.slots = dev[offs[5]:offs[6]]
-        self.fresh = dev[offs[6]:offs[7]]
+        self.fresh = dev[offs[6]:offs[6] + B]
+        self.starts_dev = dev[offs[6] + B:offs[7]]
         self.want_rows = dev[offs[7]:offs[8]]
         self._tables = [dev[offs[8 + g]:offs[9 + g]].view(B, self.table_width[g]) for g in range(n_groups)]
         self.fresh_slots_host = [rc.slot for rc in request_caches if rc.fresh]
+        self._plans = {}
+
+    def attention_plan(self, group: int, group_size: int, window: Optional[int], n_kv_heads: int) -> AttentionPlan:
+        """The MFMA attention work list, made once per step and shared by all layers that can."""
+        key = (group_size, window, n_kv_heads)
+        plan = self._plans.get(key)
+        if plan is None:
+            items, jobs, n_slots = plan_attention(self.starts, self.q_lens, group_size, window, n_kv_heads)
+            flat = [v for it in items for v in it] + [v for j in jobs for v in j]
+            host = torch.tensor(flat, dtype=torch.int32).pin_memory()
+            dev = host.to(self.device, non_blocking=True)
+            ni, nj = len(items), len(jobs)
+            plan = AttentionPlan(dev[:ni * 8], ni, dev[ni * 8:] if nj else None, nj, n_slots)
+            plan._host = host
+            self._plans[key] = plan
+        return plan
 
     def block_table(self, group: int) -> torch.Tensor:
         """``[B, width]`` int32: page of each block of each request of this step, -1 where none."""

@@ -101,8 +101,8 @@ class PagedAttention(Mixer):
                           rot.inv_freq if rot else None, H, Hk if writes else 0, D,
                           rot.rotary_dim if rot else 0, rot.interleaved if rot else False,
                           rot.mscale if rot else 1.0, cache.page_size)
-        return ops.attention(q, cache.k, cache.v, ctx.positions, ctx.req_of_token, table, H, Hk, D,
-                             cache.page_size, self.scale, self.window)
+        return ops.attention(q, cache.k, cache.v, ctx, cache.group, H, Hk, D, cache.page_size, self.scale,
+                             self.window)
 
     def forward(self, ctx, cache, h):
         return self.rt.ops.linear(self._attend(ctx, cache, h), self.w_out, bias=self.b_out)

@@ -45,8 +45,7 @@ class GatedMLP(FeedForward):
             self.b_down = tensors[f"{d}.bias"].float().contiguous()
 
     def _hidden(self, ctx, h):
-        ops = self.rt.ops
-        return ops.silu_mul(ops.linear(h, self.w_gate_up, bias=self.b_gate_up))
+        return self.rt.ops.linear_swiglu(h, self.w_gate_up, bias=self.b_gate_up)
 
     def forward(self, ctx, h):
         return self.rt.ops.linear(self._hidden(ctx, h), self.w_down, bias=self.b_down)
