@@ -1,0 +1,182 @@
+"""The serving benchmark: decode tokens a second for the Llama-3.1-8B shape with random
+weights on one MI355X, plus the prefill rate at 2,048 tokens and the decode step's
+fraction of the HBM roofline.
+
+    python bench.py --gpus 1 --steps K --warmup W
+
+A "step" is one decode step of the engine (schedule, model step, sampling) for a batch of
+8 requests, each with a 2,048-token prompt already in the cache.  One JSON line goes to
+stdout.  The reference's own bench times a 512-token prompt and 128 greedy tokens of one
+sequence and ignores end-of-text while it does (/root/reference/src/main.c:1435-1515).
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+LLAMA_3_1_8B = {
+    "architectures": ["LlamaForCausalLM"], "model_type": "llama",
+    "num_hidden_layers": 32, "hidden_size": 4096, "num_attention_heads": 32, "num_key_value_heads": 8,
+    "head_dim": 128, "intermediate_size": 14336, "vocab_size": 128256, "rope_theta": 500000.0,
+    "rope_scaling": {"rope_type": "llama3", "factor": 8.0, "low_freq_factor": 1.0, "high_freq_factor": 4.0,
+                     "original_max_position_embeddings": 8192},
+    "rms_norm_eps": 1e-5, "tie_word_embeddings": False, "max_position_embeddings": 8192, "hidden_act": "silu",
+}
+PEAK = {"hbm_gbs": 8000.0, "bf16_flops": 2.5e15, "fp32_flops": 157.3e12}
+
+
+def log(msg):
+    sys.stderr.write(f"[bench] {msg}\n")
+    sys.stderr.flush()
+
+
+def build_runner(cfg, dtype, max_tokens, max_requests, seed=0):
+    import torch
+    from xyntetik_runner_amd.config import config_from_dict
+    from xyntetik_runner_amd.engine import ModelRunner
+    from xyntetik_runner_amd.engine.model import Model
+    from xyntetik_runner_amd.weights import random_state
+    arch, typed = config_from_dict(cfg)
+    spec = arch.build_spec(typed)
+    t0 = time.time()
+    state = random_state(Model.expected_tensors(spec), seed, device=torch.device("cuda:0"))
+    runner = ModelRunner(spec, state, dtype, max_tokens=max_tokens, page_size=64, max_requests=max_requests)
+    del state
+    torch.cuda.synchronize()
+    log(f"model with {len(spec.layers)} layers on the GPU in {time.time() - t0:.1f} s")
+    return spec, runner
+
+
+def matmul_params(cfg, layers):
+    E, H, Hk, D, F, V = (cfg["hidden_size"], cfg["num_attention_heads"], cfg["num_key_value_heads"], cfg["head_dim"],
+                         cfg["intermediate_size"], cfg["vocab_size"])
+    per_layer = E * (H * D + 2 * Hk * D) + H * D * E + 3 * E * F
+    return per_layer * layers, V * E
+
+
+def decode_bytes(cfg, layers, batch, ctx_tokens, elt=2):
+    """Bytes one decode step has to read: every weight it uses once, and the cache of the live requests."""
+    body, head = matmul_params(cfg, layers)
+    norms = (2 * layers + 1) * cfg["hidden_size"]
+    weights = (body + head + norms) * elt + batch * cfg["hidden_size"] * elt     # + one embedding row per request
+    kv = ctx_tokens * 2 * cfg["num_key_value_heads"] * cfg["head_dim"] * layers * elt
+    return weights + kv
+
+
+def prefill_flops(cfg, layers, T):
+    body, head = matmul_params(cfg, layers)
+    attn = 4 * cfg["num_attention_heads"] * cfg["head_dim"] * layers * (T * (T + 1) // 2)
+    return 2 * body * T + 2 * head * 1 + attn
+
+
+def measure_decode(runner, cfg, batch, prompt_len, steps, warmup, seed):
+    """tokens/s of `steps` decode steps with `batch` requests whose prompts are already cached."""
+    import numpy as np
+    import torch
+    from xyntetik_runner_amd.engine import Engine
+    from xyntetik_runner_amd.sampling import SamplingParams
+    eng = Engine(runner, max_batched_tokens=max(2048, prompt_len), max_running=batch,
+                 max_model_len=cfg["max_position_embeddings"], stop_ids=[])
+    rng = np.random.default_rng(seed)
+    sp = SamplingParams(temperature=0.0, max_new_tokens=warmup + steps + 8, ignore_eos=True)
+    ids = [eng.add_request([int(t) for t in rng.integers(0, cfg["vocab_size"], size=prompt_len)], sp) for _ in range(batch)]
+    while any(eng.requests[i].n_computed < prompt_len for i in ids):
+        eng.step()
+    for _ in range(warmup):
+        eng.step()
+    ctx0 = sum(eng.requests[i].n_tokens for i in ids)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        eng.step()
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    ctx1 = sum(eng.requests[i].n_tokens for i in ids)
+    for i in ids:
+        eng.scheduler.abort(eng.requests.pop(i))
+    return batch * steps / dt, dt / steps, (ctx0 + ctx1) / 2
+
+
+def measure_prefill(runner, cfg, T, repeats, seed):
+    import numpy as np
+    import torch
+    from xyntetik_runner_amd.engine.batch import StepEntry
+    rng = np.random.default_rng(seed)
+    best = None
+    for r in range(repeats + 1):
+        toks = [int(t) for t in rng.integers(0, cfg["vocab_size"], size=T)]
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        out = runner.step([StepEntry(("prefill", r), toks, [T - 1])])
+        out.cpu()
+        dt = time.perf_counter() - t0
+        runner.finish(("prefill", r))
+        if r > 0:
+            best = dt if best is None else min(best, dt)
+    return best
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=128)
+    ap.add_argument("--warmup", type=int, default=16)
+    ap.add_argument("--layers", type=int, default=0, help="run fewer layers than the configuration has (named in config)")
+    ap.add_argument("--batch", type=int, default=8)
+    ap.add_argument("--prompt-len", type=int, default=2048)
+    ap.add_argument("--no-points", action="store_true", help="skip decode at batch 1 and 64")
+    ap.add_argument("--dtype", default="bfloat16")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print(f"bench.py measures one GPU only: --gpus {args.gpus} is not supported by this engine", flush=True)
+        return 2
+    cfg = dict(LLAMA_3_1_8B)
+    layers_full = cfg["num_hidden_layers"]
+    layers = args.layers or layers_full
+    cfg["num_hidden_layers"] = layers
+    P, B = args.prompt_len, args.batch
+    span = P + args.warmup + args.steps + 80
+    spec, runner = build_runner(cfg, args.dtype, max_tokens=max(64, B) * (-(-span // 64) * 64) + 4096, max_requests=64)
+
+    pre_s = measure_prefill(runner, cfg, 2048, repeats=3, seed=1)
+    pre_frac = prefill_flops(cfg, layers, 2048) / pre_s / PEAK["bf16_flops" if args.dtype == "bfloat16" else "fp32_flops"]
+    log(f"prefill 2048 tokens: {pre_s * 1e3:.1f} ms")
+
+    tps, step_s, ctx = measure_decode(runner, cfg, B, P, args.steps, args.warmup, seed=2)
+    elt = 2 if args.dtype == "bfloat16" else 4
+    achieved = decode_bytes(cfg, layers, B, ctx, elt) / step_s / 1e9
+    log(f"decode batch {B}: {tps:.1f} tok/s, {step_s * 1e3:.3f} ms/step, {achieved:.0f} GB/s")
+    points = {}
+    if not args.no_points:
+        for b in (1, 64):
+            n = max(8, min(args.steps, 64))
+            t, s, c = measure_decode(runner, cfg, b, P, n, min(args.warmup, 8), seed=3 + b)
+            points[f"decode_b{b}"] = round(t, 1)
+            log(f"decode batch {b}: {t:.1f} tok/s, {s * 1e3:.3f} ms/step, "
+                f"{decode_bytes(cfg, layers, b, c, elt) / s / 1e9:.0f} GB/s")
+    line = {
+        "metric": "decode tokens/s, Llama-3.1-8B shape, batch 8, 2048-token prompts (random weights)",
+        "value": round(tps, 1), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(step_s * 1e3, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16" if args.dtype == "bfloat16" else "fp32", "data": "synthetic",
+        "config": {"model": "Llama-3.1-8B shape", "layers": layers, "layers_in_config": layers_full,
+                   "hidden_size": cfg["hidden_size"], "heads": cfg["num_attention_heads"],
+                   "kv_heads": cfg["num_key_value_heads"], "head_dim": cfg["head_dim"],
+                   "intermediate_size": cfg["intermediate_size"], "vocab_size": cfg["vocab_size"],
+                   "global_batch": B, "seq_len": P, "max_context": cfg["max_position_embeddings"],
+                   "decode_tokens": args.steps, "parallelism": "single GPU"},
+        "prefill": {"value": round(2048 / pre_s, 1), "tokens": 2048, "ms": round(pre_s * 1e3, 3), "frac": round(pre_frac, 4)},
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK["hbm_gbs"], "unit": "GB/s",
+                     "frac": round(achieved / PEAK["hbm_gbs"], 4)},
+        "points": points,
+    }
+    print(json.dumps(line), flush=True)
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -104,24 +104,22 @@ __global__ __launch_bounds__(256) void k_attn_mfma(AttnArgs a) {
         for (int e = 0; e < 16; ++e) o[d][e] = 0.f;
     float m = -INFINITY, l = 0.f;
 
+    // Loads run ahead of their use: the keys of the next tile are requested while the
+    // current tile's softmax and second product run, the values of the current tile before
+    // its scores are computed.
+    auto load_k = [&](int kt, uint4* kf) {
+        const int key = kt + key_off;
+        int page = -1;
+        if (key < seq_len) page = bt[key >> a.page_shift];
+        const bf16_t* kp = a.kc + (((size_t)(page < 0 ? 0 : page) * a.Hk + kvh) * a.page_size + (key & a.page_mask)) * HD + lg * 8;
+#pragma unroll
+        for (int kd = 0; kd < KD; ++kd) kf[kd] = page >= 0 ? ldg16(kp + kd * 16) : zero;
+    };
+    uint4 kf[KD];
+    if (kbeg < kend) load_k(kbeg, kf);
+
     for (int kt = kbeg; kt < kend; kt += 32) {
-        // ---- S^T = K Q^T
-        f32x16 s;
-#pragma unroll
-        for (int e = 0; e < 16; ++e) s[e] = 0.f;
-        {
-            const int key = kt + key_off;
-            int page = -1;
-            if (key < seq_len) page = bt[key >> a.page_shift];
-            const bf16_t* kp = a.kc + (((size_t)(page < 0 ? 0 : page) * a.Hk + kvh) * a.page_size + (key & a.page_mask)) * HD + lg * 8;
-            uint4 kf[KD];
-#pragma unroll
-            for (int kd = 0; kd < KD; ++kd) kf[kd] = page >= 0 ? ldg16(kp + kd * 16) : zero;
-#pragma unroll
-            for (int kd = 0; kd < KD; ++kd)
-                s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16x8(kf[kd]), qf[kd], s, 0, 0, 0);
-        }
-        // ---- values for this tile (issued early; used after the softmax)
+        // ---- values for this tile (used after the softmax)
         uint4 vf[2][DB];
 #pragma unroll
         for (int j = 0; j < 2; ++j) {
@@ -144,6 +142,14 @@ __global__ __launch_bounds__(256) void k_attn_mfma(AttnArgs a) {
                 vf[j][d] = v;
             }
         }
+        // ---- S^T = K Q^T
+        f32x16 s;
+#pragma unroll
+        for (int e = 0; e < 16; ++e) s[e] = 0.f;
+#pragma unroll
+        for (int kd = 0; kd < KD; ++kd)
+            s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16x8(kf[kd]), qf[kd], s, 0, 0, 0);
+        if (kt + 32 < kend) load_k(kt + 32, kf);
         // ---- mask, running maximum and sum
         float p[16];
         float mt = -INFINITY;
@@ -230,29 +236,42 @@ struct MergeArgs {
     int H, Hk;
 };
 
+#define MERGE_MAX 64     // slots whose weights a thread keeps at once
+
 __global__ __launch_bounds__(256) void k_attn_merge(MergeArgs a) {
     const int* job = a.jobs + (size_t)blockIdx.x * 4;
     const int req = job[0], row0 = job[1], s0 = job[2], ns = job[3];
     const int kvh = blockIdx.y;
     const int G = a.H / a.Hk;
     const int q0 = a.cu_q[req], q_len = a.cu_q[req + 1] - q0;
-    for (int idx = threadIdx.x; idx < ROWS * (HD / 4); idx += 256) {
+    const int n_rows = (q_len * G - row0) < ROWS ? (q_len * G - row0) : ROWS;      // rows of this block that exist
+    for (int idx = threadIdx.x; idx < n_rows * (HD / 4); idx += 256) {
         const int r = idx / (HD / 4), d4 = (idx % (HD / 4)) * 4;
         const int rho = row0 + r;
         const int tok = rho / G, hg = rho - tok * G;
-        if (tok >= q_len) continue;
-        float mx = -INFINITY;
-        for (int s = 0; s < ns; ++s) mx = fmaxf(mx, a.part_ml[(((size_t)(s0 + s) * a.Hk + kvh) * ROWS + r) * 2]);
         float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
-        float wsum = 0.f;
-        for (int s = 0; s < ns; ++s) {
-            const size_t base = ((size_t)(s0 + s) * a.Hk + kvh) * ROWS + r;
-            const float ms = a.part_ml[base * 2], ls = a.part_ml[base * 2 + 1];
-            if (!(ls > 0.f)) continue;
-            const float w = ls * expf(ms - mx);
-            const float4 v = *reinterpret_cast<const float4*>(a.part_o + base * HD + d4);
-            acc.x += w * v.x; acc.y += w * v.y; acc.z += w * v.z; acc.w += w * v.w;
-            wsum += w;
+        float wsum = 0.f, mx = -INFINITY;
+        for (int c0 = 0; c0 < ns; c0 += MERGE_MAX) {          // almost always one pass
+            const int nc = (ns - c0) < MERGE_MAX ? (ns - c0) : MERGE_MAX;
+            float ms[MERGE_MAX], ls[MERGE_MAX];
+            float cm = -INFINITY;
+#pragma unroll 8
+            for (int s = 0; s < nc; ++s) {
+                const float2 v = *reinterpret_cast<const float2*>(a.part_ml + (((size_t)(s0 + c0 + s) * a.Hk + kvh) * ROWS + r) * 2);
+                ms[s] = v.x; ls[s] = v.y;
+                cm = fmaxf(cm, v.x);
+            }
+            const float nm = fmaxf(mx, cm);
+            const float resc = (mx == -INFINITY) ? 0.f : expf(mx - nm);
+            acc.x *= resc; acc.y *= resc; acc.z *= resc; acc.w *= resc; wsum *= resc;
+            mx = nm;
+#pragma unroll 8
+            for (int s = 0; s < nc; ++s) {
+                const float w = ls[s] > 0.f ? ls[s] * expf(ms[s] - mx) : 0.f;
+                const float4 v = *reinterpret_cast<const float4*>(a.part_o + (((size_t)(s0 + c0 + s) * a.Hk + kvh) * ROWS + r) * HD + d4);
+                acc.x += w * v.x; acc.y += w * v.y; acc.z += w * v.z; acc.w += w * v.w;
+                wsum += w;
+            }
         }
         const float inv = wsum > 0.f ? 1.0f / wsum : 0.f;
         bf16_t* op = a.out + ((size_t)(q0 + tok) * a.H + kvh * G + hg) * HD + d4;

@@ -60,17 +60,73 @@ __global__ void k_rmsnorm(TO* __restrict__ out, const float* __restrict__ x, con
     }
 }
 
+// Rows whose width is a multiple of 4 (up to 4 * 256 * RN_MAXV): every thread keeps its
+// float4 pieces in registers between the sum and the scaling, and writes 4 values at a time.
+#define RN_MAXV 8
+template <typename TO> __device__ inline void st4(TO* p, size_t i, float a, float b, float c, float d);
+template <> __device__ inline void st4<float>(float* p, size_t i, float a, float b, float c, float d) {
+    *reinterpret_cast<float4*>(p + i) = make_float4(a, b, c, d);
+}
+template <> __device__ inline void st4<bf16_t>(bf16_t* p, size_t i, float a, float b, float c, float d) {
+    uint2 w;
+    w.x = (uint32_t)f32_to_bf16(a) | ((uint32_t)f32_to_bf16(b) << 16);
+    w.y = (uint32_t)f32_to_bf16(c) | ((uint32_t)f32_to_bf16(d) << 16);
+    *reinterpret_cast<uint2*>(p + i) = w;
+}
+
+template <typename TO, typename TW, int NV>
+__global__ __launch_bounds__(256) void k_rmsnorm_v4(TO* __restrict__ out, const float* __restrict__ x,
+                                                    const TW* __restrict__ w, const int* __restrict__ rows,
+                                                    int E, int ldx, float eps) {
+    __shared__ float part[4];
+    const int r = blockIdx.x;
+    const int src = rows ? rows[r] : r;
+    const float4* xr = reinterpret_cast<const float4*>(x + (size_t)src * ldx);
+    const int n4 = E >> 2;
+    float4 v[NV];
+    float ss = 0.f;
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+        const int c = threadIdx.x + i * 256;
+        v[i] = c < n4 ? xr[c] : make_float4(0.f, 0.f, 0.f, 0.f);
+        ss += v[i].x * v[i].x + v[i].y * v[i].y + v[i].z * v[i].z + v[i].w * v[i].w;
+    }
+    ss = wave_sum(ss);
+    if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = ss;
+    __syncthreads();
+    const float tot = part[0] + part[1] + part[2] + part[3];
+    const float rinv = 1.0f / sqrtf(tot / (float)E + eps);
+    TO* o = out + (size_t)r * E;
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+        const int c = threadIdx.x + i * 256;
+        if (c >= n4) continue;
+        float w0 = 1.f, w1 = 1.f, w2 = 1.f, w3 = 1.f;
+        if (w) { w0 = ld<TW>(w, 4 * c); w1 = ld<TW>(w, 4 * c + 1); w2 = ld<TW>(w, 4 * c + 2); w3 = ld<TW>(w, 4 * c + 3); }
+        st4<TO>(o, (size_t)4 * c, v[i].x * rinv * w0, v[i].y * rinv * w1, v[i].z * rinv * w2, v[i].w * rinv * w3);
+    }
+}
+
 extern "C" int xr_rmsnorm(void* out, const float* x, const void* w, const int* rows, int R, int E,
                           int ldx, float eps, int out_dtype, int w_dtype, hipStream_t stream) {
     XR_REQUIRE(R >= 0 && E > 0 && ldx >= E, "rmsnorm: bad sizes R=%d E=%d ldx=%d", R, E, ldx);
     XR_REQUIRE(eps >= 0.f, "rmsnorm: eps %g is negative", eps);
+    XR_REQUIRE((out_dtype == XR_F32 || out_dtype == XR_BF16) && (w_dtype == XR_F32 || w_dtype == XR_BF16),
+               "rmsnorm: bad dtypes out=%d w=%d", out_dtype, w_dtype);
     if (R == 0) return XR_OK;
-#define RN(TO, TW) k_rmsnorm<TO, TW><<<R, 256, 0, stream>>>((TO*)out, x, (const TW*)w, rows, E, ldx, eps)
+    const bool vec = E % 4 == 0 && ldx % 4 == 0 && ((uintptr_t)x % 16) == 0 && ((uintptr_t)out % 16) == 0 &&
+                     E <= 4 * 256 * RN_MAXV;
+#define RN(TO, TW)                                                                                              \
+    do {                                                                                                        \
+        if (!vec) k_rmsnorm<TO, TW><<<R, 256, 0, stream>>>((TO*)out, x, (const TW*)w, rows, E, ldx, eps);        \
+        else if (E <= 4 * 256 * 2) k_rmsnorm_v4<TO, TW, 2><<<R, 256, 0, stream>>>((TO*)out, x, (const TW*)w, rows, E, ldx, eps); \
+        else if (E <= 4 * 256 * 4) k_rmsnorm_v4<TO, TW, 4><<<R, 256, 0, stream>>>((TO*)out, x, (const TW*)w, rows, E, ldx, eps); \
+        else k_rmsnorm_v4<TO, TW, RN_MAXV><<<R, 256, 0, stream>>>((TO*)out, x, (const TW*)w, rows, E, ldx, eps); \
+    } while (0)
     if (out_dtype == XR_F32 && w_dtype == XR_F32) RN(float, float);
     else if (out_dtype == XR_F32 && w_dtype == XR_BF16) RN(float, bf16_t);
     else if (out_dtype == XR_BF16 && w_dtype == XR_F32) RN(bf16_t, float);
-    else if (out_dtype == XR_BF16 && w_dtype == XR_BF16) RN(bf16_t, bf16_t);
-    else { xr_set_error("rmsnorm: bad dtypes out=%d w=%d", out_dtype, w_dtype); return XR_BAD_ARG; }
+    else RN(bf16_t, bf16_t);
 #undef RN
     XR_CHECK_LAUNCH("rmsnorm");
     return XR_OK;

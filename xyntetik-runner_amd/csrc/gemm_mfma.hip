@@ -36,6 +36,13 @@ struct GemmArgs {
 };
 
 __device__ inline uint4 ldg16(const bf16_t* p) { return *reinterpret_cast<const uint4*>(p); }
+// streaming load: the weights of a decode step are read once and must not push the
+// activations out of the caches
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+__device__ inline uint4 ldg16_stream(const bf16_t* p) {
+    u32x4 v = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p));
+    return make_uint4(v.x, v.y, v.z, v.w);
+}
 __device__ inline bf16x8 as_bf16x8(uint4 v) {
     union { uint4 u; bf16x8 b; } c;
     c.u = v;
@@ -206,7 +213,7 @@ __global__ __launch_bounds__(64 * WARPS_M * WARPS_N) void k_gemm_tile(GemmArgs g
 // L2) of U k-steps of 32 before it uses them; with N/(16*RT) workgroups of KSW waves this
 // keeps tens of kilobytes in flight on every compute unit.  The slices are summed through
 // LDS in a fixed order.
-template <int MT, int RT, int KSW, int U, bool SWIGLU>
+template <int MT, int RT, int KSW, int U, bool SWIGLU, bool NT>
 __global__ __launch_bounds__(64 * KSW) void k_gemm_skinny(GemmArgs g) {
     constexpr int NWT = SWIGLU ? 2 : 1;  // weight fragments per row group (gate and up)
     constexpr int MTOK = MT * 16, ROWS = RT * 16, THREADS = 64 * KSW;
@@ -258,7 +265,7 @@ __global__ __launch_bounds__(64 * KSW) void k_gemm_skinny(GemmArgs g) {
             for (int r = 0; r < RT; ++r)
 #pragma unroll
                 for (int t = 0; t < NWT; ++t)
-                    wreg[u][t][r] = (k_ok && w_ok[r]) ? ldg16(wp[t][r] + k) : zero;
+                    wreg[u][t][r] = (k_ok && w_ok[r]) ? (NT ? ldg16_stream(wp[t][r] + k) : ldg16(wp[t][r] + k)) : zero;
 #pragma unroll
             for (int i = 0; i < MT; ++i) areg[u][i] = (k_ok && a_ok[i]) ? ldg16(ap[i] + k) : zero;
         }
@@ -308,19 +315,19 @@ __global__ __launch_bounds__(64 * KSW) void k_gemm_skinny(GemmArgs g) {
     }
 }
 
-template <int MT, int RT, int KSW, int U, bool SW>
+template <int MT, int RT, int KSW, int U, bool SW, bool NT = false>
 static int launch_skinny(const GemmArgs& g, hipStream_t stream) {
     constexpr int NWT = SW ? 2 : 1;
     size_t smem = (size_t)KSW * NWT * RT * 16 * MT * 16 * 4;
     static bool attr_set = false;
     if (!attr_set) {
-        hipError_t e = hipFuncSetAttribute((const void*)k_gemm_skinny<MT, RT, KSW, U, SW>,
+        hipError_t e = hipFuncSetAttribute((const void*)k_gemm_skinny<MT, RT, KSW, U, SW, NT>,
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
         if (e != hipSuccess) { xr_set_error("gemm: cannot reserve %zu bytes of LDS: %s", smem, hipGetErrorString(e)); return XR_LAUNCH; }
         attr_set = true;
     }
     unsigned blocks = (unsigned)((g.N + 16 * RT - 1) / (16 * RT));
-    k_gemm_skinny<MT, RT, KSW, U, SW><<<blocks, 64 * KSW, smem, stream>>>(g);
+    k_gemm_skinny<MT, RT, KSW, U, SW, NT><<<blocks, 64 * KSW, smem, stream>>>(g);
     XR_CHECK_LAUNCH("gemm_skinny");
     return XR_OK;
 }
@@ -365,6 +372,17 @@ extern "C" int xr_gemm_bf16(void* out, const void* a, const void* w, const float
         if (M <= 32) return sw ? launch_skinny<2, 1, 16, 8, true>(g, stream) : launch_skinny<2, 1, 16, 8, false>(g, stream);
         return sw ? launch_skinny<4, 2, 8, 4, true>(g, stream) : launch_skinny<4, 2, 8, 4, false>(g, stream);
     }
+#ifdef XR_GEMM_SWEEP
+#define SK(id, MT, RT, KSW, U, NT) if (variant == id) return sw ? launch_skinny<MT, RT, KSW, U, true, NT>(g, stream) : launch_skinny<MT, RT, KSW, U, false, NT>(g, stream);
+    SK(100, 1, 1, 16, 8, false) SK(101, 1, 1, 8, 8, false) SK(102, 1, 1, 8, 16, false) SK(103, 1, 1, 4, 16, false)
+    SK(104, 1, 1, 4, 8, false) SK(105, 1, 2, 8, 8, false) SK(106, 1, 2, 4, 8, false) SK(107, 1, 1, 16, 4, false)
+    SK(108, 1, 1, 16, 8, true) SK(109, 1, 1, 8, 8, true) SK(110, 1, 1, 8, 16, true) SK(111, 1, 2, 8, 8, true)
+    SK(112, 1, 2, 16, 4, false) SK(113, 1, 4, 4, 4, false) SK(114, 1, 1, 2, 16, false) SK(115, 1, 2, 4, 8, true)
+    SK(140, 4, 2, 8, 4, false) SK(141, 4, 1, 8, 4, false) SK(142, 4, 1, 16, 4, false) SK(143, 4, 2, 4, 4, false)
+    SK(144, 4, 4, 4, 2, false) SK(145, 4, 2, 8, 4, true) SK(146, 4, 1, 8, 8, false) SK(147, 4, 2, 8, 2, false)
+    SK(148, 4, 4, 4, 4, false) SK(149, 4, 4, 8, 2, false)
+#undef SK
+#endif
     if (variant == 2) return launch_tile<128, 128, 2, 2>(g, stream);
     if (variant == 3) return launch_tile<256, 128, 4, 2>(g, stream);
     xr_set_error("gemm: unknown variant %d", variant);

@@ -37,8 +37,8 @@ class AttentionPlan:
 
 ATTN_ROWS = 32          # query rows (token x head-in-group) per work item
 ATTN_TILE = 32          # keys per tile; items begin and end on tile edges
-ATTN_TARGET_WAVES = 2048
-ATTN_MIN_TILES = 4
+ATTN_TARGET_WAVES = 4096
+ATTN_MIN_TILES = 2
 
 
 def plan_attention(starts, q_lens, group_size: int, window: Optional[int], n_kv_heads: int):

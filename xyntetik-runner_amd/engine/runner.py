@@ -36,7 +36,7 @@ def parse_dtype(name) -> torch.dtype:
 
 class ModelRunner:
     def __init__(self, spec: ModelSpec, tensors_or_store, dtype, max_tokens: int, page_size: int = 64,
-                 max_requests: int = 64, device: str = "cuda:0"):
+                 max_requests: int = 64, device: str = "cuda:0", use_graphs: bool = True):
         if not torch.cuda.is_available():
             raise RuntimeError("no GPU: this engine runs on an MI355X only and has no CPU path")
         self.device = torch.device(device)
@@ -59,6 +59,8 @@ class ModelRunner:
         self.storage = CacheStorage(kv, st, of, page_size, pages, max_requests, self.dtype, self.device)
         self.manager = CacheManager(self.storage.group_specs, page_size, pages, max_requests)
         self.vocab_size = spec.vocab_size
+        from .graphs import DecodeGraphs
+        self.graphs = DecodeGraphs(self) if use_graphs else None
 
     @classmethod
     def from_folder(cls, model_dir: str, dtype="bfloat16", **kw) -> "ModelRunner":
@@ -108,13 +110,29 @@ class ModelRunner:
                 raise OutOfPages(f"this step needs {spare[gi]} new pages in group {gi}, {g.pool.n_free} of {g.pool.size} are free")
         for e, rc in zip(entries, rcs):
             mgr.reserve(e.req_id, rc.n_tokens + len(e.tokens))
-        ctx = StepContext(self.ops, self.device, entries, rcs, len(mgr.groups))
-        self._zero_fresh_state(ctx)
-        x = self.model.forward(ctx, self.storage.layers)
-        out = self.model.logits(ctx, x, ctx.want_rows) if ctx.n_want else None
+        if self.graphs is not None and self.graphs.applies(entries):
+            out = self._step_graph(entries, rcs)
+        else:
+            ctx = StepContext(self.ops, self.device, entries, rcs, len(mgr.groups))
+            self._zero_fresh_state(ctx)
+            x = self.model.forward(ctx, self.storage.layers)
+            out = self.model.logits(ctx, x, ctx.want_rows) if ctx.n_want else None
         for e, rc in zip(entries, rcs):
             mgr.advance(e.req_id, rc.n_tokens + len(e.tokens))
         return out
+
+    def _step_graph(self, entries, rcs) -> Optional[torch.Tensor]:
+        """A step of single tokens through a captured graph; the result is valid until the next step."""
+        for e in entries:
+            if any(w != 0 for w in e.want):
+                raise ValueError(f"request {e.req_id!r}: wanted place outside its one token")
+        logits = self.graphs.run(entries, rcs)
+        rows = [i for i, e in enumerate(entries) for _ in e.want]
+        if not rows:
+            return None
+        if rows == list(range(len(entries))):
+            return logits
+        return logits[torch.tensor(rows, dtype=torch.long, device=self.device)]
 
     def _zero_fresh_state(self, ctx: StepContext) -> None:
         if not ctx.fresh_slots_host:
