@@ -98,6 +98,8 @@ def measure_decode(runner, cfg, batch, prompt_len, steps, warmup, seed):
     ctx1 = sum(eng.requests[i].n_tokens for i in ids)
     for i in ids:
         eng.scheduler.abort(eng.requests.pop(i))
+    if runner.graphs is not None:
+        log(f"  graphs: {runner.graphs.captures} captured, {runner.graphs.replays} replays so far")
     return batch * steps / dt, dt / steps, (ctx0 + ctx1) / 2
 
 

@@ -34,7 +34,7 @@ constexpr int KD = HD / 16;          // k-steps of the score product
 constexpr int DB = (HD + 31) / 32;   // 32-row blocks of O^T
 static_assert(HD % 16 == 0 && HD >= 16 && HD <= 256, "head size must be a multiple of 16 up to 256");
 
-#define ITEM_INTS 8                   // req, row0, k_begin, k_end, slot (-1: final), unused...
+#define ITEM_INTS 8                   // req, row0, k_begin, k_end, slot (-1: final), q0, q_len, start
 #define ROWS 32
 
 struct AttnArgs {
@@ -42,7 +42,7 @@ struct AttnArgs {
     const bf16_t* kc;       // [pages, Hk, page_size, HD]
     const bf16_t* vc;       // [pages, Hk, HD, page_size]
     bf16_t* out;            // [T, H, HD]
-    const int* items;       // [n_items, ITEM_INTS]
+    const int* items;       // [n_items, ITEM_INTS]; q0: the request's first row, start: its first position
     const int* cu_q;        // [B + 1] first row (token) of each request in this step
     const int* starts;      // [B] position of each request's first token of this step
     const int* block_table; // [B, table_stride]
@@ -60,9 +60,10 @@ __device__ inline bf16x8 as_bf16x8(uint4 v) {
     c.u = v;
     return c.b;
 }
-__device__ inline uint32_t pack2(float lo, float hi) {
-    return (uint32_t)f32_to_bf16(lo) | ((uint32_t)f32_to_bf16(hi) << 16);
+__device__ inline uint4 keep_if(bool ok, uint4 v) {     // zero unless ok, word by word
+    return make_uint4(ok ? v.x : 0u, ok ? v.y : 0u, ok ? v.z : 0u, ok ? v.w : 0u);
 }
+__device__ inline uint32_t pack2(float lo, float hi) { return pack_bf16x2(lo, hi); }
 
 __global__ __launch_bounds__(256) void k_attn_mfma(AttnArgs a) {
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -70,11 +71,11 @@ __global__ __launch_bounds__(256) void k_attn_mfma(AttnArgs a) {
     if (item >= a.n_items) return;
     const int kvh = blockIdx.y;
     const int* it = a.items + (size_t)item * ITEM_INTS;
+    // everything about the item and its request comes with the item: no second lookup
     const int req = it[0], row0 = it[1], kbeg = it[2], kend = it[3], slot = it[4];
+    const int q0 = it[5], q_len = it[6], start = it[7];
     const int G = a.H / a.Hk;
     const int lr = lane & 31, lg = lane >> 5;
-    const int q0 = a.cu_q[req], q_len = a.cu_q[req + 1] - q0;
-    const int start = a.starts[req];
     const int seq_len = start + q_len;
     const int* bt = a.block_table + (size_t)req * a.table_stride;
 
@@ -89,57 +90,98 @@ __global__ __launch_bounds__(256) void k_attn_mfma(AttnArgs a) {
     const uint4 zero = make_uint4(0, 0, 0, 0);
     bf16x8 qf[KD];
     {
-        const bf16_t* qp = a.q + ((size_t)t * a.H + h) * HD + lg * 8;
+        const bf16_t* qp = a.q + ((size_t)(row_ok ? t : q0) * a.H + h) * HD + lg * 8;
 #pragma unroll
-        for (int kd = 0; kd < KD; ++kd) qf[kd] = as_bf16x8(row_ok ? ldg16(qp + kd * 16) : zero);
+        for (int kd = 0; kd < KD; ++kd) qf[kd] = as_bf16x8(keep_if(row_ok, ldg16(qp + kd * 16)));
     }
     // the key this lane's tile row stands for: r = 8a + 4g + b  ->  16(a/2) + 8g + 4(a%2) + b
     const int ra = lr >> 3, rg = (lr >> 2) & 1, rb = lr & 3;
     const int key_off = 16 * (ra >> 1) + 8 * rg + 4 * (ra & 1) + rb;
+
+    // Page numbers of the item's keys, one per lane, fetched once per 64 pages: inside the
+    // loop a page number comes from another lane's register, not from memory.
+    const bf16_t* __restrict__ kc = a.kc;
+    const bf16_t* __restrict__ vc = a.vc;
+    const int page0 = kbeg >> a.page_shift;
+    int pages_base = page0;
+    int my_page;
+    {
+        const int pi = page0 + lane;
+        const bool in = ((long)pi << a.page_shift) < seq_len;
+        my_page = bt[in ? pi : 0];
+        my_page = in ? my_page : -1;
+    }
+    // Loads are never predicated: a key that does not exist is read from the null page and
+    // its words are replaced by zeros, so whole 16-byte loads stay in flight.
+#define ATTN_LOAD_K(KT, KF)                                                                              \
+    {                                                                                                    \
+        const int key_ = (KT) + key_off;                                                                 \
+        const int pg_ = __shfl(my_page, ((key_ < seq_len ? key_ : (KT)) >> a.page_shift) - pages_base, 64); \
+        const bool ok_ = key_ < seq_len && pg_ >= 0;                                                     \
+        const bf16_t* kp_ = kc + (((size_t)(ok_ ? pg_ : 0) * a.Hk + kvh) * a.page_size + (key_ & a.page_mask)) * HD + lg * 8; \
+        _Pragma("unroll") for (int kd = 0; kd < KD; ++kd) KF[kd] = keep_if(ok_, ldg16(kp_ + kd * 16));   \
+    }
+#define ATTN_LOAD_V(KT, VF)                                                                              \
+    {                                                                                                    \
+        _Pragma("unroll") for (int j = 0; j < 2; ++j) {                                                  \
+            const int k8_ = (KT) + 16 * j + 8 * lg;                                                      \
+            const int pg_ = __shfl(my_page, ((k8_ < seq_len ? k8_ : (KT)) >> a.page_shift) - pages_base, 64); \
+            const bool ok_ = k8_ < seq_len && pg_ >= 0;                                                  \
+            _Pragma("unroll") for (int d = 0; d < DB; ++d) {                                             \
+                const int dd_ = d * 32 + lr;                                                             \
+                const bool okd_ = ok_ && dd_ < HD;                                                       \
+                VF[j][d] = keep_if(okd_, ldg16(vc + (((size_t)(okd_ ? pg_ : 0) * a.Hk + kvh) * HD + (okd_ ? dd_ : 0)) * a.page_size + (k8_ & a.page_mask))); \
+            }                                                                                            \
+        }                                                                                                \
+    }
 
     f32x16 o[DB];
 #pragma unroll
     for (int d = 0; d < DB; ++d)
 #pragma unroll
         for (int e = 0; e < 16; ++e) o[d][e] = 0.f;
-    float m = -INFINITY, l = 0.f;
-
-    // Loads run ahead of their use: the keys of the next tile are requested while the
-    // current tile's softmax and second product run, the values of the current tile before
-    // its scores are computed.
-    auto load_k = [&](int kt, uint4* kf) {
-        const int key = kt + key_off;
-        int page = -1;
-        if (key < seq_len) page = bt[key >> a.page_shift];
-        const bf16_t* kp = a.kc + (((size_t)(page < 0 ? 0 : page) * a.Hk + kvh) * a.page_size + (key & a.page_mask)) * HD + lg * 8;
+    float m = -INFINITY, l = 0.f;      // m in units of log2
+    const float c2 = a.scale * 1.44269504088896340736f;
+    // a tile whose keys lie in [lo_max, pos_min] is visible to every row that exists
+    int pos_min = row_ok ? pos : 0x7fffffff, lo_max = row_ok ? lo : 0;
 #pragma unroll
-        for (int kd = 0; kd < KD; ++kd) kf[kd] = page >= 0 ? ldg16(kp + kd * 16) : zero;
-    };
-    uint4 kf[KD];
-    if (kbeg < kend) load_k(kbeg, kf);
+    for (int o_ = 32; o_ > 0; o_ >>= 1) {
+        pos_min = min(pos_min, __shfl_xor(pos_min, o_, 64));
+        lo_max = max(lo_max, __shfl_xor(lo_max, o_, 64));
+    }
 
+    // Loads run one tile ahead of their use.
+    uint4 kf[KD], vf[2][DB];
+    if (kbeg < kend) {
+        ATTN_LOAD_K(kbeg, kf)
+        ATTN_LOAD_V(kbeg, vf)
+    }
     for (int kt = kbeg; kt < kend; kt += 32) {
-        // ---- values for this tile (used after the softmax)
-        uint4 vf[2][DB];
+        uint4 kn[KD], vn[2][DB];
+        const int nx = kt + 32;
+        if (nx < kend) {
+            if (((nx >> a.page_shift) - pages_base) >= 64) {
+                pages_base = nx >> a.page_shift;
+                const int pi = pages_base + lane;
+                const bool in = ((long)pi << a.page_shift) < seq_len;
+                my_page = bt[in ? pi : 0];
+                my_page = in ? my_page : -1;
+            }
+            ATTN_LOAD_K(nx, kn)
+            ATTN_LOAD_V(nx, vn)
+        }
+        if (kt + 32 > seq_len) {               // the request's last tile: slots past its end hold old data
 #pragma unroll
-        for (int j = 0; j < 2; ++j) {
-            const int k8 = kt + 16 * j + 8 * lg;            // first of this lane's 8 keys
-            int page = -1;
-            if (k8 < seq_len) page = bt[k8 >> a.page_shift];
+            for (int j = 0; j < 2; ++j) {
+                const int k8 = kt + 16 * j + 8 * lg;
+                uint32_t mk[4];
 #pragma unroll
-            for (int d = 0; d < DB; ++d) {
-                const int dd = d * 32 + lr;
-                uint4 v = zero;
-                if (page >= 0 && dd < HD)
-                    v = ldg16(a.vc + (((size_t)page * a.Hk + kvh) * HD + dd) * a.page_size + (k8 & a.page_mask));
-                if (k8 + 8 > seq_len) {                      // slots past the request's end hold old data
-                    uint32_t w[4] = {v.x, v.y, v.z, v.w};
+                for (int e = 0; e < 4; ++e)
+                    mk[e] = (k8 + 2 * e < seq_len ? 0x0000FFFFu : 0u) | (k8 + 2 * e + 1 < seq_len ? 0xFFFF0000u : 0u);
 #pragma unroll
-                    for (int e = 0; e < 8; ++e)
-                        if (k8 + e >= seq_len) w[e >> 1] &= (e & 1) ? 0x0000FFFFu : 0xFFFF0000u;
-                    v = make_uint4(w[0], w[1], w[2], w[3]);
+                for (int d = 0; d < DB; ++d) {
+                    vf[j][d].x &= mk[0]; vf[j][d].y &= mk[1]; vf[j][d].z &= mk[2]; vf[j][d].w &= mk[3];
                 }
-                vf[j][d] = v;
             }
         }
         // ---- S^T = K Q^T
@@ -149,34 +191,55 @@ __global__ __launch_bounds__(256) void k_attn_mfma(AttnArgs a) {
 #pragma unroll
         for (int kd = 0; kd < KD; ++kd)
             s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16x8(kf[kd]), qf[kd], s, 0, 0, 0);
-        if (kt + 32 < kend) load_k(kt + 32, kf);
-        // ---- mask, running maximum and sum
+        // ---- running maximum and sum, in units of log2: p = 2^(s*c - m), c = scale * log2(e)
         float p[16];
-        float mt = -INFINITY;
+        float corr;
+        if (kt + 32 <= kend && kt + 31 <= pos_min && kt >= lo_max) {
+            // every key of the tile is visible to every row: no mask
+            float mt = fmaxf(fmaxf(s[0], s[1]), fmaxf(s[2], s[3]));
 #pragma unroll
-        for (int e = 0; e < 16; ++e) {
-            const int key = kt + 16 * (e >> 3) + 8 * lg + (e & 7);
-            const bool ok = row_ok && key <= pos && key >= lo && key < kend;
-            p[e] = ok ? s[e] * a.scale : -INFINITY;
-            mt = fmaxf(mt, p[e]);
+            for (int e = 4; e < 16; e += 4) mt = fmaxf(mt, fmaxf(fmaxf(s[e], s[e + 1]), fmaxf(s[e + 2], s[e + 3])));
+            mt = fmaxf(mt, __shfl_xor(mt, 32, 64));
+            const float mn = fmaxf(m, mt * c2);
+            corr = __builtin_amdgcn_exp2f(m - mn);
+            float rs = 0.f;
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+                p[e] = __builtin_amdgcn_exp2f(fmaf(s[e], c2, -mn));
+                rs += p[e];
+            }
+            rs += __shfl_xor(rs, 32, 64);
+            l = fmaf(l, corr, rs);
+            m = mn;
+        } else {
+            float mt = -INFINITY;
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+                const int key = kt + 16 * (e >> 3) + 8 * lg + (e & 7);
+                const bool ok = row_ok && key <= pos && key >= lo && key < kend;
+                p[e] = ok ? s[e] * c2 : -INFINITY;
+                mt = fmaxf(mt, p[e]);
+            }
+            mt = fmaxf(mt, __shfl_xor(mt, 32, 64));
+            const float mn = fmaxf(m, mt);
+            const float mu = mn == -INFINITY ? 0.f : mn;
+            corr = __builtin_amdgcn_exp2f(m - mu);
+            float rs = 0.f;
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+                p[e] = __builtin_amdgcn_exp2f(p[e] - mu);
+                rs += p[e];
+            }
+            rs += __shfl_xor(rs, 32, 64);
+            l = fmaf(l, corr, rs);
+            m = mn;
         }
-        mt = fmaxf(mt, __shfl_xor(mt, 32, 64));
-        const float mn = fmaxf(m, mt);
-        const float mu = mn == -INFINITY ? 0.f : mn;
-        const float corr = expf(m - mu);
-        float rs = 0.f;
+        if (__any(corr != 1.0f)) {             // the maximum moved for some row
 #pragma unroll
-        for (int e = 0; e < 16; ++e) {
-            p[e] = expf(p[e] - mu);
-            rs += p[e];
+            for (int d = 0; d < DB; ++d)
+#pragma unroll
+                for (int e = 0; e < 16; ++e) o[d][e] *= corr;
         }
-        rs += __shfl_xor(rs, 32, 64);
-        l = l * corr + rs;
-        m = mn;
-#pragma unroll
-        for (int d = 0; d < DB; ++d)
-#pragma unroll
-            for (int e = 0; e < 16; ++e) o[d][e] *= corr;
         // ---- O^T += V^T P^T
 #pragma unroll
         for (int j = 0; j < 2; ++j) {
@@ -187,12 +250,20 @@ __global__ __launch_bounds__(256) void k_attn_mfma(AttnArgs a) {
             for (int d = 0; d < DB; ++d)
                 o[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16x8(vf[j][d]), pf, o[d], 0, 0, 0);
         }
+        if (nx < kend) {
+#pragma unroll
+            for (int kd = 0; kd < KD; ++kd) kf[kd] = kn[kd];
+#pragma unroll
+            for (int j = 0; j < 2; ++j)
+#pragma unroll
+                for (int d = 0; d < DB; ++d) vf[j][d] = vn[j][d];
+        }
     }
 
     // ---- write: lane owns row `rho`; register e of block d is channel d*32 + (e/4)*8 + lg*4 + e%4
     const float inv = l > 0.f ? 1.0f / l : 0.f;
+    if (!row_ok) return;
     if (slot < 0) {
-        if (!row_ok) return;
         bf16_t* op = a.out + ((size_t)t * a.H + h) * HD;
 #pragma unroll
         for (int d = 0; d < DB; ++d)
@@ -225,8 +296,8 @@ __global__ __launch_bounds__(256) void k_attn_mfma(AttnArgs a) {
 }
 
 // One merge job: {req, row0, first_slot, n_slots}.  Slot s holds the normalised output of
-// its keys with their maximum m_s and sum l_s; the whole is sum_s w_s O_s / sum_s w_s with
-// w_s = l_s * exp(m_s - max m).
+// its keys with their maximum m_s (in units of log2) and sum l_s; the whole is
+// sum_s w_s O_s / sum_s w_s with w_s = l_s * 2^(m_s - max m).
 struct MergeArgs {
     const int* jobs;        // [n_jobs, 4]
     const int* cu_q;
@@ -235,8 +306,6 @@ struct MergeArgs {
     bf16_t* out;
     int H, Hk;
 };
-
-#define MERGE_MAX 64     // slots whose weights a thread keeps at once
 
 __global__ __launch_bounds__(256) void k_attn_merge(MergeArgs a) {
     const int* job = a.jobs + (size_t)blockIdx.x * 4;
@@ -249,29 +318,21 @@ __global__ __launch_bounds__(256) void k_attn_merge(MergeArgs a) {
         const int r = idx / (HD / 4), d4 = (idx % (HD / 4)) * 4;
         const int rho = row0 + r;
         const int tok = rho / G, hg = rho - tok * G;
+        const float* ml = a.part_ml + (((size_t)s0 * a.Hk + kvh) * ROWS + r) * 2;
+        const float* po = a.part_o + (((size_t)s0 * a.Hk + kvh) * ROWS + r) * HD + d4;
+        const size_t ml_step = (size_t)a.Hk * ROWS * 2, po_step = (size_t)a.Hk * ROWS * HD;
+        float mx = -INFINITY;
+#pragma unroll 4
+        for (int s = 0; s < ns; ++s) mx = fmaxf(mx, ml[s * ml_step]);
         float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
-        float wsum = 0.f, mx = -INFINITY;
-        for (int c0 = 0; c0 < ns; c0 += MERGE_MAX) {          // almost always one pass
-            const int nc = (ns - c0) < MERGE_MAX ? (ns - c0) : MERGE_MAX;
-            float ms[MERGE_MAX], ls[MERGE_MAX];
-            float cm = -INFINITY;
-#pragma unroll 8
-            for (int s = 0; s < nc; ++s) {
-                const float2 v = *reinterpret_cast<const float2*>(a.part_ml + (((size_t)(s0 + c0 + s) * a.Hk + kvh) * ROWS + r) * 2);
-                ms[s] = v.x; ls[s] = v.y;
-                cm = fmaxf(cm, v.x);
-            }
-            const float nm = fmaxf(mx, cm);
-            const float resc = (mx == -INFINITY) ? 0.f : expf(mx - nm);
-            acc.x *= resc; acc.y *= resc; acc.z *= resc; acc.w *= resc; wsum *= resc;
-            mx = nm;
-#pragma unroll 8
-            for (int s = 0; s < nc; ++s) {
-                const float w = ls[s] > 0.f ? ls[s] * expf(ms[s] - mx) : 0.f;
-                const float4 v = *reinterpret_cast<const float4*>(a.part_o + (((size_t)(s0 + c0 + s) * a.Hk + kvh) * ROWS + r) * HD + d4);
-                acc.x += w * v.x; acc.y += w * v.y; acc.z += w * v.z; acc.w += w * v.w;
-                wsum += w;
-            }
+        float wsum = 0.f;
+#pragma unroll 4
+        for (int s = 0; s < ns; ++s) {
+            const float2 v2 = *reinterpret_cast<const float2*>(ml + s * ml_step);
+            const float w = v2.y > 0.f ? v2.y * __builtin_amdgcn_exp2f(v2.x - mx) : 0.f;
+            const float4 v = *reinterpret_cast<const float4*>(po + s * po_step);
+            acc.x += w * v.x; acc.y += w * v.y; acc.z += w * v.z; acc.w += w * v.w;
+            wsum += w;
         }
         const float inv = wsum > 0.f ? 1.0f / wsum : 0.f;
         bf16_t* op = a.out + ((size_t)(q0 + tok) * a.H + kvh * G + hg) * HD + d4;

@@ -58,6 +58,23 @@ __host__ __device__ inline bf16_t f32_to_bf16(float f) {
     return (bf16_t)(u >> 16);
 }
 
+// two floats -> two bfloat16 in one word (low half first), round to nearest even, one
+// v_cvt_pk_bf16_f32 on gfx950
+#if defined(__HIP_DEVICE_COMPILE__)
+typedef __bf16 xr_bf16x2 __attribute__((ext_vector_type(2)));
+typedef float xr_f32x2 __attribute__((ext_vector_type(2)));
+__device__ inline uint32_t pack_bf16x2(float lo, float hi) {
+    xr_f32x2 v = {lo, hi};
+    union { xr_bf16x2 b; uint32_t u; } c;
+    c.b = __builtin_convertvector(v, xr_bf16x2);
+    return c.u;
+}
+#else   // the host pass only has to parse the callers
+__host__ __device__ inline uint32_t pack_bf16x2(float lo, float hi) {
+    return (uint32_t)f32_to_bf16(lo) | ((uint32_t)f32_to_bf16(hi) << 16);
+}
+#endif
+
 template <typename T> __device__ inline float ld(const T* p, size_t i);
 template <> __device__ inline float ld<float>(const float* p, size_t i) { return p[i]; }
 template <> __device__ inline float ld<bf16_t>(const bf16_t* p, size_t i) { return bf16_to_f32(p[i]); }

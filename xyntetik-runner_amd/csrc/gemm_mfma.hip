@@ -48,6 +48,10 @@ __device__ inline bf16x8 as_bf16x8(uint4 v) {
     c.u = v;
     return c.b;
 }
+// zero unless ok, word by word (a select between two 16-byte objects goes through memory)
+__device__ inline uint4 keep_if(bool ok, uint4 v) {
+    return make_uint4(ok ? v.x : 0u, ok ? v.y : 0u, ok ? v.z : 0u, ok ? v.w : 0u);
+}
 __device__ inline float silu_f(float g) { return g / (1.0f + expf(-g)); }
 
 __device__ inline void store_out(const GemmArgs& g, int m, int n, float v) {
@@ -94,26 +98,34 @@ __global__ __launch_bounds__(64 * WARPS_M * WARPS_N) void k_gemm_tile(GemmArgs g
     const int bx = blockIdx.x;
     const int n_rows = g.epi == EPI_SWIGLU ? 2 * g.N : g.N;
 
-    // which rows this thread stages
+    // Which chunks this thread stages.  Loads are never predicated: a chunk outside the
+    // matrix is read from a row and column that exist and then replaced by zeros, so the
+    // compiler keeps whole 16-byte global loads in flight.
     int a_row[A_CHUNKS], a_c[A_CHUNKS];
-    const bf16_t* a_ptr[A_CHUNKS];
+    size_t a_off[A_CHUNKS];
+    bool a_ok[A_CHUNKS];
 #pragma unroll
     for (int i = 0; i < A_CHUNKS; ++i) {
         int q = tid + i * THREADS;
         a_row[i] = q / CH; a_c[i] = q % CH;
         int m = m0 + a_row[i];
-        a_ptr[i] = m < g.M ? g.a + (size_t)m * g.lda + a_c[i] * 8 : nullptr;
+        a_ok[i] = m < g.M;
+        a_off[i] = (size_t)(a_ok[i] ? m : 0) * g.lda + a_c[i] * 8;
     }
     int w_row[W_CHUNKS], w_c[W_CHUNKS];
-    const bf16_t* w_ptr[W_CHUNKS];
+    size_t w_off[W_CHUNKS];
+    bool w_ok[W_CHUNKS];
 #pragma unroll
     for (int i = 0; i < W_CHUNKS; ++i) {
         int q = tid + i * THREADS;
         w_row[i] = q / CH; w_c[i] = q % CH;
         int oc;
         int n = w_row_of<BN, WN>(w_row[i], bx, g.N, g.epi, oc);
-        w_ptr[i] = (oc < g.N && n < n_rows) ? g.w + (size_t)n * g.K + w_c[i] * 8 : nullptr;
+        w_ok[i] = oc < g.N && n < n_rows;
+        w_off[i] = (size_t)(w_ok[i] ? n : 0) * g.K + w_c[i] * 8;
     }
+    const bf16_t* __restrict__ gA = g.a;
+    const bf16_t* __restrict__ gW = g.w;
 
     f32x16 acc[TM][TN];
 #pragma unroll
@@ -125,29 +137,35 @@ __global__ __launch_bounds__(64 * WARPS_M * WARPS_N) void k_gemm_tile(GemmArgs g
 
     uint4 ra[A_CHUNKS], rw[W_CHUNKS];
     const uint4 zero = make_uint4(0, 0, 0, 0);
-    auto load_global = [&](int k0) {
-#pragma unroll
-        for (int i = 0; i < A_CHUNKS; ++i)
-            ra[i] = (a_ptr[i] && k0 + a_c[i] * 8 < g.K) ? ldg16(a_ptr[i] + k0) : zero;
-#pragma unroll
-        for (int i = 0; i < W_CHUNKS; ++i)
-            rw[i] = (w_ptr[i] && k0 + w_c[i] * 8 < g.K) ? ldg16(w_ptr[i] + k0) : zero;
-    };
-    auto store_lds = [&](int buf) {
-#pragma unroll
-        for (int i = 0; i < A_CHUNKS; ++i) lds[buf * BUF + a_row[i] * CH + (a_c[i] ^ (a_row[i] & 7))] = ra[i];
-#pragma unroll
-        for (int i = 0; i < W_CHUNKS; ++i) lds[buf * BUF + BM * CH + w_row[i] * CH + (w_c[i] ^ (w_row[i] & 7))] = rw[i];
-    };
+#define TILE_LOAD_GLOBAL(K0)                                                                     \
+    {                                                                                            \
+        _Pragma("unroll") for (int i = 0; i < A_CHUNKS; ++i) {                                   \
+            const bool in_k = (K0) + a_c[i] * 8 < g.K;                                           \
+            const uint4 v = ldg16(gA + a_off[i] + (in_k ? (K0) : 0));                            \
+            ra[i] = keep_if(a_ok[i] && in_k, v);                                                 \
+        }                                                                                        \
+        _Pragma("unroll") for (int i = 0; i < W_CHUNKS; ++i) {                                   \
+            const bool in_k = (K0) + w_c[i] * 8 < g.K;                                           \
+            const uint4 v = ldg16(gW + w_off[i] + (in_k ? (K0) : 0));                            \
+            rw[i] = keep_if(w_ok[i] && in_k, v);                                                 \
+        }                                                                                        \
+    }
+#define TILE_STORE_LDS(BUFI)                                                                     \
+    {                                                                                            \
+        _Pragma("unroll") for (int i = 0; i < A_CHUNKS; ++i)                                     \
+            lds[(BUFI) * BUF + a_row[i] * CH + (a_c[i] ^ (a_row[i] & 7))] = ra[i];               \
+        _Pragma("unroll") for (int i = 0; i < W_CHUNKS; ++i)                                     \
+            lds[(BUFI) * BUF + BM * CH + w_row[i] * CH + (w_c[i] ^ (w_row[i] & 7))] = rw[i];     \
+    }
 
     const int nk = (g.K + BK - 1) / BK;
-    load_global(0);
-    store_lds(0);
+    TILE_LOAD_GLOBAL(0)
+    TILE_STORE_LDS(0)
     __syncthreads();
     const int lr = lane & 31, lg = lane >> 5;
     for (int kt = 0; kt < nk; ++kt) {
         const int buf = kt & 1;
-        if (kt + 1 < nk) load_global((kt + 1) * BK);
+        if (kt + 1 < nk) TILE_LOAD_GLOBAL((kt + 1) * BK)
 #pragma unroll
         for (int ks = 0; ks < BK / 16; ++ks) {
             bf16x8 af[TM], wf[TN];
@@ -168,9 +186,11 @@ __global__ __launch_bounds__(64 * WARPS_M * WARPS_N) void k_gemm_tile(GemmArgs g
                 for (int j = 0; j < TN; ++j)
                     acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[i], wf[j], acc[i][j], 0, 0, 0);
         }
-        if (kt + 1 < nk) store_lds(buf ^ 1);
+        if (kt + 1 < nk) TILE_STORE_LDS(buf ^ 1)
         __syncthreads();
     }
+#undef TILE_LOAD_GLOBAL
+#undef TILE_STORE_LDS
 
     // epilogue: lane holds column (lane % 32), rows (e/4)*8 + (lane/32)*4 + e%4 of each 32x32 tile
     if (g.epi == EPI_SWIGLU) {
@@ -261,13 +281,14 @@ __global__ __launch_bounds__(64 * KSW) void k_gemm_skinny(GemmArgs g) {
         for (int u = 0; u < U; ++u) {
             const int k = k0 + u * 32 + lq * 8;
             const bool k_ok = k < kend;
+            const int ks = k_ok ? k : 0;             // a column that exists; the value is dropped
 #pragma unroll
             for (int r = 0; r < RT; ++r)
 #pragma unroll
                 for (int t = 0; t < NWT; ++t)
-                    wreg[u][t][r] = (k_ok && w_ok[r]) ? (NT ? ldg16_stream(wp[t][r] + k) : ldg16(wp[t][r] + k)) : zero;
+                    wreg[u][t][r] = keep_if(k_ok && w_ok[r], NT ? ldg16_stream(wp[t][r] + ks) : ldg16(wp[t][r] + ks));
 #pragma unroll
-            for (int i = 0; i < MT; ++i) areg[u][i] = (k_ok && a_ok[i]) ? ldg16(ap[i] + k) : zero;
+            for (int i = 0; i < MT; ++i) areg[u][i] = keep_if(k_ok && a_ok[i], ldg16(ap[i] + ks));
         }
 #pragma unroll
         for (int u = 0; u < U; ++u)

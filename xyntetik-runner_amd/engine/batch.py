@@ -25,7 +25,8 @@ class AttentionPlan:
     """The work list of the MFMA attention kernel for one step, cache group, group size and window.
 
     ``items [n, 8]`` int32 on the device: request, first row of a 32-row block, first key,
-    end key, partial slot (-1: the item covers all keys of its block and writes the output).
+    end key, partial slot (-1: the item covers all keys of its block and writes the output),
+    the request's first row in the step, its number of tokens, its first position.
     ``jobs [m, 4]``: request, first row, first slot, number of slots to merge.
     """
     items: torch.Tensor
@@ -37,14 +38,32 @@ class AttentionPlan:
 
 ATTN_ROWS = 32          # query rows (token x head-in-group) per work item
 ATTN_TILE = 32          # keys per tile; items begin and end on tile edges
-ATTN_TARGET_WAVES = 4096
-ATTN_MIN_TILES = 2
+
+
+def tiles_per_item(total_tiles: int, n_kv_heads: int) -> int:
+    """How many 32-key tiles one work item should cover.
+
+    Short items pay their start-up (query load, page numbers, partial results) too often,
+    long ones leave compute units idle; the best length measured on MI355X grows with the
+    square root of the step's work (2-4 tiles for one decoding request at 2k context, 8 for
+    eight, 16 for sixty-four).
+    """
+    want = (max(1, total_tiles) * n_kv_heads / 64.0) ** 0.5
+    t = 2
+    while t * 2 <= want and t < 32:
+        t *= 2
+    return t
+
 
 
 def plan_attention(starts, q_lens, group_size: int, window: Optional[int], n_kv_heads: int):
     """Host side of ``AttentionPlan``: lists of items and merge jobs (plain Python ints)."""
     blocks = []
     total_tiles = 0
+    q0s, acc = [], 0
+    for n in q_lens:
+        q0s.append(acc)
+        acc += n
     for b, (s, n) in enumerate(zip(starts, q_lens)):
         rows = n * group_size
         for row0 in range(0, rows, ATTN_ROWS):
@@ -57,20 +76,20 @@ def plan_attention(starts, q_lens, group_size: int, window: Optional[int], n_kv_
             blocks.append((b, row0, lo, hi, tiles))
             total_tiles += tiles
     chunk = 1 << 30
-    if blocks and len(blocks) * n_kv_heads < ATTN_TARGET_WAVES:
-        chunk = max(ATTN_MIN_TILES, -(-total_tiles * n_kv_heads // ATTN_TARGET_WAVES))
+    if blocks and len(blocks) * n_kv_heads < 2048:         # too few row blocks to fill the chip
+        chunk = tiles_per_item(total_tiles, n_kv_heads)
     items, jobs, slot = [], [], 0
     for b, row0, lo, hi, tiles in blocks:
         parts = -(-tiles // chunk)
         if parts <= 1:
-            items.append((b, row0, lo, hi, -1, 0, 0, 0))
+            items.append((b, row0, lo, hi, -1, q0s[b], q_lens[b], starts[b]))
             continue
         per = -(-tiles // parts)
         first = slot
         k = lo
         while k < hi:
             e = min(hi, k + per * ATTN_TILE)
-            items.append((b, row0, k, e, slot, 0, 0, 0))
+            items.append((b, row0, k, e, slot, q0s[b], q_lens[b], starts[b]))
             slot += 1
             k = e
         jobs.append((b, row0, first, slot - first))

@@ -21,11 +21,10 @@ import numpy as np
 import torch
 
 from ..cache import NULL_PAGE
-from .batch import ATTN_TILE, AttentionPlan, StepEntry
+from .batch import ATTN_TILE, AttentionPlan, StepEntry, tiles_per_item
 
 BUCKETS = (1, 2, 4, 8, 16, 32, 64, 128, 256, 512)
 SPLITS = (1, 2, 4, 8, 16, 32)
-TARGET_WAVES = 4096
 
 
 def bucket_for(n: int) -> Optional[int]:
@@ -36,8 +35,8 @@ def bucket_for(n: int) -> Optional[int]:
 
 
 def splits_for(batch_cap: int, max_tiles: int, n_kv_heads: int) -> int:
-    """Key ranges per request: enough waves to fill the chip, at least two tiles each."""
-    want = min(max(1, max_tiles // 2), max(1, TARGET_WAVES // max(1, batch_cap * n_kv_heads)))
+    """Key ranges per request, so that a range has about ``tiles_per_item`` tiles."""
+    want = max(1, round(max_tiles / tiles_per_item(batch_cap * max_tiles, n_kv_heads)))
     best = 1
     for s in SPLITS:
         if s <= want:
@@ -169,7 +168,9 @@ class StaticDecodeContext:
         items[:, :, 2] = kb
         items[:, :, 3] = ke
         items[:, :, 4] = (np.arange(B)[:, None] * S + s_idx) if S > 1 else -1
-        items[:, :, 5:] = 0
+        items[:, :, 5] = np.arange(B)[:, None]
+        items[:, :, 6] = 1
+        items[:, :, 7] = starts[:, None]
         jobs[:, 0] = np.arange(B)
         jobs[:, 1] = 0
         jobs[:, 2] = np.arange(B) * S
