@@ -161,3 +161,60 @@ def test_out_of_pages_is_an_error_that_changes_nothing(models):
     mx, mean = logit_error(got, want["r3"][40:64])
     assert mx <= TOL["float32"][0]
     runner.manager.check()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_long_decoding(models, tmp_path, dtype):
+    """A short prompt and 250 tokens decoded one by one through the captured decode step:
+    pages fill and new ones are taken, the attention's key ranges change, and every
+    position still matches the plain implementation."""
+    d, cfg, reqs, plens, want = models["A"]
+    toks = prompt_ids(258, cfg["vocab_size"], 77)
+    full = P.forward(cfg, *[P.load_folder(d)[1]], toks)
+    steps = [{"step": 0, "entries": [{"id": "x", "tokens": toks[:8], "want": list(range(8))}], "end": []}]
+    for i in range(8, len(toks)):
+        steps.append({"step": i - 7, "entries": [{"id": "x", "tokens": [toks[i]], "want": [0]}],
+                      "end": ["x"] if i == len(toks) - 1 else []})
+    out, runner = run_replay(d, dtype, steps, tmp_path, page_size=16)
+    assert runner.graphs.replays >= 200 and runner.graphs.captures >= 2
+    check(traces.collect(steps, out, cfg["vocab_size"]), {"x": full}, dtype, "long decoding")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_first_tokens(models, tmp_path, dtype):
+    """Positions 0, 1, 2, ... of fresh requests: one token at a time, and two requests side by side."""
+    d, cfg, reqs, plens, want = models["B"]
+    w = P.load_folder(d)[1]
+    a, b = prompt_ids(5, cfg["vocab_size"], 1), prompt_ids(5, cfg["vocab_size"], 2)
+    steps = [{"step": i, "entries": [{"id": "a", "tokens": [a[i]], "want": [0]}, {"id": "b", "tokens": [b[i]], "want": [0]}],
+              "end": ["a", "b"] if i == 4 else []} for i in range(5)]
+    out, runner = run_replay(d, dtype, steps, tmp_path, page_size=64)
+    check(traces.collect(steps, out, cfg["vocab_size"]), {"a": P.forward(cfg, w, a), "b": P.forward(cfg, w, b)}, dtype, "first tokens")
+
+
+@pytest.mark.parametrize("dtype,tol", [("float32", 2e-6), ("bfloat16", 3e-3)])
+def test_graph_and_eager_decode_agree(models, dtype, tol):
+    """The captured decode step against the same step run kernel by kernel, replayed several
+    times with other work between the replays.  The two split the keys of a request into
+    ranges differently, so they agree to rounding, not bit for bit."""
+    import torch
+    from xyntetik_runner_amd.engine.batch import StepEntry
+    from xyntetik_runner_amd.engine.runner import ModelRunner
+    d, cfg, reqs, plens, want = models["A"]
+    toks = reqs["r4"]
+    outs = {}
+    for use in (True, False):
+        r = ModelRunner.from_folder(d, dtype="bfloat16", max_tokens=512, page_size=16, max_requests=4, use_graphs=use)
+        r.step([StepEntry("p", toks[:40], []), StepEntry("q", toks[:17], [])])
+        rows = []
+        for i in range(40, 70):
+            o = r.step([StepEntry("p", [toks[i]], [0]), StepEntry("q", [toks[i - 23]], [0])])
+            rows.append(o.cpu().numpy())
+            if i % 7 == 0:          # eager work between replays: a prompt portion of a third request
+                r.step([StepEntry("z", toks[:9], [8])])
+                r.finish("z")
+        outs[use] = np.concatenate(rows)
+        if use:
+            assert r.graphs.replays >= 25
+    mx, mean = logit_error(outs[True], outs[False])
+    assert mx <= tol and np.abs(outs[True]).max() > 0, (mx, mean)

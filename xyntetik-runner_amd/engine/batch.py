@@ -173,6 +173,7 @@ class StepContext:
         self.want_rows = dev[offs[7]:offs[8]]
         self._tables = [dev[offs[8 + g]:offs[9 + g]].view(B, self.table_width[g]) for g in range(n_groups)]
         self.fresh_slots_host = [rc.slot for rc in request_caches if rc.fresh]
+        self.slots_host = [rc.slot for rc in request_caches]
         self._plans = {}
 
     def attention_plan(self, group: int, group_size: int, window: Optional[int], n_kv_heads: int) -> AttentionPlan:
