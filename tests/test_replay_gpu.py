@@ -204,7 +204,7 @@ def test_graph_and_eager_decode_agree(models, dtype, tol):
     toks = reqs["r4"]
     outs = {}
     for use in (True, False):
-        r = ModelRunner.from_folder(d, dtype="bfloat16", max_tokens=512, page_size=16, max_requests=4, use_graphs=use)
+        r = ModelRunner.from_folder(d, dtype=dtype, max_tokens=512, page_size=16, max_requests=4, use_graphs=use)
         r.step([StepEntry("p", toks[:40], []), StepEntry("q", toks[:17], [])])
         rows = []
         for i in range(40, 70):

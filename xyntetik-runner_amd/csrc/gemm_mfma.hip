@@ -33,6 +33,7 @@ struct GemmArgs {
     int M, N, K, lda, ldo;
     int out_bf16;      // storage of out
     int epi;
+    int m_fast;        // tile order of the asynchronous kernel: 1 = consecutive workgroups share a weight tile
 };
 
 __device__ inline uint4 ldg16(const bf16_t* p) { return *reinterpret_cast<const uint4*>(p); }
@@ -225,6 +226,179 @@ __global__ __launch_bounds__(64 * WARPS_M * WARPS_N) void k_gemm_tile(GemmArgs g
         }
 }
 
+// ------------------------------------------------------------------------------ tile kernel, asynchronous
+// The same tiling with the operands copied from memory straight into LDS
+// (global_load_lds_dwordx4: every lane names a 16-byte source, the wave's 64 pieces land
+// side by side in LDS) and STAGES K-slices in flight: while the matrix cores work on slice
+// kt, slices kt+1 .. kt+STAGES-1 are on their way, with no registers and no LDS-write
+// instructions spent on them.  A lane whose piece lies outside the matrices reads from a
+// block of zeros instead, so every slice issues the same number of loads and one counter
+// wait (vmcnt) tells when a slice has landed.
+__device__ uint4 xr_zero_chunk[4];      // zero-initialised
+
+template <int N> struct WaitVm {        // s_waitcnt vmcnt(N) only
+    static constexpr int imm = (N & 0xF) | ((N >> 4) << 14) | (0x7 << 4) | (0xF << 8);
+};
+
+// The copies are written as inline assembly: the compiler then does not count them, so it
+// neither makes every LDS read wait for all of them nor drains them at each barrier; the
+// kernel waits for exactly the slice it is about to use (s_waitcnt vmcnt) and meets the
+// other waves at a bare s_barrier.
+__device__ inline void lds_dma16(const void* src, uint32_t lds_byte_addr) {
+    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
+                 :: "v"(src), "s"(lds_byte_addr) : "memory");
+}
+template <int N> __device__ inline void wait_vmcnt() {
+    asm volatile("s_waitcnt vmcnt(%0)" :: "n"(N) : "memory");
+}
+
+template <int BM, int BN, int WARPS_M, int WARPS_N, int STAGES>
+__global__ __launch_bounds__(64 * WARPS_M * WARPS_N) void k_gemm_tile_async(GemmArgs g) {
+    constexpr int WAVES = WARPS_M * WARPS_N;
+    constexpr int BK = 64, CH = BK / 8;
+    constexpr int WM = BM / WARPS_M, WN = BN / WARPS_N;
+    constexpr int TM = WM / 32, TN = WN / 32;
+    constexpr int ROWS = BM + BN;                       // rows of one stage: activations, then weights
+    constexpr int LOADS = ROWS / 8 / WAVES;             // load instructions per wave and stage (8 rows each)
+    static_assert(ROWS % (8 * WAVES) == 0, "stage does not divide among waves");
+    static_assert(LOADS * (STAGES - 2) < 64, "too many loads in flight for the counter");
+    constexpr int BUF = ROWS * CH;                      // chunks per stage
+    extern __shared__ uint4 lds[];                      // [STAGES][BUF]
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm0 = (wave / WARPS_N) * WM, wn0 = (wave % WARPS_N) * WN;
+    // Workgroups are numbered along M first (m_fast) or along N first.  Consecutive
+    // workgroups go to different XCDs, so with 8 row tiles each XCD keeps one activation tile
+    // in its L2 while the weight tile of the moment is fetched once from memory for all.
+    const int tiles_m = (g.M + BM - 1) / BM;
+    const int tiles_n = (g.N + (g.epi == EPI_SWIGLU ? BN / 2 : BN) - 1) / (g.epi == EPI_SWIGLU ? BN / 2 : BN);
+    const int bm_ = g.m_fast ? (int)(blockIdx.x % tiles_m) : (int)(blockIdx.x / tiles_n);
+    const int bx = g.m_fast ? (int)(blockIdx.x / tiles_m) : (int)(blockIdx.x % tiles_n);
+    const int m0 = bm_ * BM;
+    const int n_rows = g.epi == EPI_SWIGLU ? 2 * g.N : g.N;
+    const bf16_t* zero_src = reinterpret_cast<const bf16_t*>(xr_zero_chunk);
+
+    // the pieces this lane fetches for every stage: row of the stage and column chunk
+    const bf16_t* src[LOADS];
+    int src_c[LOADS];
+#pragma unroll
+    for (int i = 0; i < LOADS; ++i) {
+        const int row = (i * WAVES + wave) * 8 + (lane >> 3);     // row of the stage
+        const int slot = lane & 7;
+        const int c = slot ^ (row & 7);                           // the chunk that belongs in this LDS place
+        src_c[i] = c * 8;
+        if (row < BM) {
+            const int m = m0 + row;
+            src[i] = m < g.M ? g.a + (size_t)m * g.lda + c * 8 : nullptr;
+        } else {
+            int oc;
+            const int n = w_row_of<BN, WN>(row - BM, bx, g.N, g.epi, oc);
+            src[i] = (oc < g.N && n < n_rows) ? g.w + (size_t)n * g.K + c * 8 : nullptr;
+        }
+    }
+    const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) void*)lds;
+#define ASYNC_ISSUE(KT)                                                                              \
+    {                                                                                                \
+        const int k0_ = (KT) * BK;                                                                   \
+        const uint32_t dst_ = lds_base + (uint32_t)((((KT) % STAGES) * BUF + wave * 64) * 16);       \
+        _Pragma("unroll") for (int i = 0; i < LOADS; ++i) {                                          \
+            const bf16_t* p_ = (src[i] && k0_ + src_c[i] < g.K) ? src[i] + k0_ : zero_src;           \
+            lds_dma16(p_, __builtin_amdgcn_readfirstlane(dst_ + i * WAVES * 64 * 16));               \
+        }                                                                                            \
+    }
+
+    f32x16 acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+
+    const int nk = (g.K + BK - 1) / BK;
+#pragma unroll
+    for (int st = 0; st < STAGES - 1; ++st) ASYNC_ISSUE(st)
+    const int lr = lane & 31, lg = lane >> 5;
+    for (int kt = 0; kt < nk; ++kt) {
+        // slice kt has landed when at most the STAGES-2 younger slices are still in flight
+        wait_vmcnt<LOADS * (STAGES - 2)>();
+        __builtin_amdgcn_s_barrier();                    // for every wave; and slice kt-1 is no longer read
+        ASYNC_ISSUE(kt + STAGES - 1)                     // into the buffer slice kt-1 used (zeros past the end)
+        const uint4* A = lds + (kt % STAGES) * BUF;
+        const uint4* W = A + BM * CH;
+#pragma unroll
+        for (int ks = 0; ks < BK / 16; ++ks) {
+            bf16x8 af[TM], wf[TN];
+            const int c = ks * 2 + lg;
+#pragma unroll
+            for (int i = 0; i < TM; ++i) {
+                const int r = wm0 + i * 32 + lr;
+                af[i] = as_bf16x8(A[r * CH + (c ^ (r & 7))]);
+            }
+#pragma unroll
+            for (int j = 0; j < TN; ++j) {
+                const int r = wn0 + j * 32 + lr;
+                wf[j] = as_bf16x8(W[r * CH + (c ^ (r & 7))]);
+            }
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int j = 0; j < TN; ++j)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[i], wf[j], acc[i][j], 0, 0, 0);
+        }
+    }
+#undef ASYNC_ISSUE
+    wait_vmcnt<0>();                                     // the trailing loads of zeros
+
+    if (g.epi == EPI_SWIGLU) {
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j + 1 < TN; j += 2) {
+                int oc;
+                w_row_of<BN, WN>(wn0 + j * 32 + lr, bx, g.N, g.epi, oc);
+                if (oc >= g.N) continue;
+                float bg = g.bias ? g.bias[oc] : 0.f, bu = g.bias ? g.bias[g.N + oc] : 0.f;
+#pragma unroll
+                for (int e = 0; e < 16; ++e) {
+                    int m = m0 + wm0 + i * 32 + (e / 4) * 8 + lg * 4 + (e % 4);
+                    if (m < g.M) store_out(g, m, oc, silu_f(acc[i][j][e] + bg) * (acc[i][j + 1][e] + bu));
+                }
+            }
+        return;
+    }
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+            int n = bx * BN + wn0 + j * 32 + lr;
+            if (n >= g.N) continue;
+            float b = g.bias ? g.bias[n] : 0.f;
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+                int m = m0 + wm0 + i * 32 + (e / 4) * 8 + lg * 4 + (e % 4);
+                if (m < g.M) store_out(g, m, n, acc[i][j][e] + b);
+            }
+        }
+}
+
+template <int BM, int BN, int WM_, int WN_, int ST>
+static int launch_tile_async(const GemmArgs& g, hipStream_t stream) {
+    size_t smem = (size_t)ST * (BM + BN) * 8 * 16;
+    static bool attr_set = false;
+    if (!attr_set) {
+        hipError_t e = hipFuncSetAttribute((const void*)k_gemm_tile_async<BM, BN, WM_, WN_, ST>,
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+        if (e != hipSuccess) { xr_set_error("gemm: cannot reserve %zu bytes of LDS: %s", smem, hipGetErrorString(e)); return XR_LAUNCH; }
+        attr_set = true;
+    }
+    int n_out_tile = g.epi == EPI_SWIGLU ? BN / 2 : BN;
+    unsigned grid = (unsigned)(((g.N + n_out_tile - 1) / n_out_tile) * ((g.M + BM - 1) / BM));
+    k_gemm_tile_async<BM, BN, WM_, WN_, ST><<<grid, 64 * WM_ * WN_, smem, stream>>>(g);
+    XR_CHECK_LAUNCH("gemm_tile_async");
+    return XR_OK;
+}
+
 // ------------------------------------------------------------------------------ skinny kernel
 // MT: 16-token groups (M <= 16*MT).  RT: groups of 16 weight rows per wave.  KSW: waves per
 // workgroup; they split K into contiguous slices, so a workgroup owns 16*RT output columns
@@ -385,8 +559,20 @@ extern "C" int xr_gemm_bf16(void* out, const void* a, const void* w, const float
     GemmArgs g;
     g.a = (const bf16_t*)a; g.w = (const bf16_t*)w; g.bias = bias; g.out = out;
     g.M = M; g.N = N; g.K = K; g.lda = lda; g.ldo = ldo; g.out_bf16 = out_dtype == XR_BF16; g.epi = epi;
+    g.m_fast = 0;
+    if (variant >= 1000) { g.m_fast = 1; variant -= 1000; }
     const bool sw = epi == EPI_SWIGLU;
-    if (variant == 0) variant = M <= 64 ? 1 : 2;
+    if (variant == 0) {
+        if (M <= 64) {
+            variant = 1;
+        } else {
+            // the largest tile that still gives every compute unit a workgroup
+            const int n_out = N;
+            auto count = [&](int bm, int bn) { return ((M + bm - 1) / bm) * ((n_out + (sw ? bn / 2 : bn) - 1) / (sw ? bn / 2 : bn)); };
+            variant = count(256, 256) >= 180 ? 14 : (count(256, 128) >= 180 ? 12 : 17);
+            g.m_fast = 1;
+        }
+    }
     if (variant == 1) {
         XR_REQUIRE(M <= 64, "gemm: the skinny kernel takes at most 64 rows, got %d", M);
         if (M <= 16) return sw ? launch_skinny<1, 1, 16, 8, true>(g, stream) : launch_skinny<1, 1, 16, 8, false>(g, stream);
@@ -406,6 +592,22 @@ extern "C" int xr_gemm_bf16(void* out, const void* a, const void* w, const float
 #endif
     if (variant == 2) return launch_tile<128, 128, 2, 2>(g, stream);
     if (variant == 3) return launch_tile<256, 128, 4, 2>(g, stream);
+    if (variant == 4) return launch_tile<256, 128, 2, 2>(g, stream);
+    if (variant == 5) return launch_tile<256, 256, 2, 2>(g, stream);
+    if (variant == 6) return launch_tile<128, 256, 2, 2>(g, stream);
+    if (variant == 7) return launch_tile<256, 256, 2, 4>(g, stream);
+    if (variant == 8) return launch_tile<256, 256, 4, 2>(g, stream);
+    if (variant == 10) return launch_tile_async<128, 128, 2, 2, 3>(g, stream);
+    if (variant == 11) return launch_tile_async<128, 128, 2, 2, 4>(g, stream);
+    if (variant == 12) return launch_tile_async<256, 128, 4, 2, 3>(g, stream);
+    if (variant == 13) return launch_tile_async<256, 256, 2, 4, 2>(g, stream);
+    if (variant == 14) return launch_tile_async<256, 256, 4, 2, 2>(g, stream);
+    if (variant == 15) return launch_tile_async<256, 128, 2, 2, 3>(g, stream);
+    if (variant == 16) return launch_tile_async<128, 256, 2, 4, 3>(g, stream);
+    if (variant == 17) return launch_tile_async<128, 128, 2, 2, 2>(g, stream);
+    if (variant == 18) return launch_tile_async<256, 256, 2, 2, 2>(g, stream);
+    if (variant == 19) return launch_tile_async<256, 128, 2, 2, 2>(g, stream);
+    if (variant == 20) return launch_tile_async<128, 256, 2, 2, 2>(g, stream);
     xr_set_error("gemm: unknown variant %d", variant);
     return XR_BAD_ARG;
 }
