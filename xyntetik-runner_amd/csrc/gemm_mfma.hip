@@ -464,6 +464,7 @@ __global__ __launch_bounds__(64 * KSW) void k_gemm_skinny(GemmArgs g) {
 #pragma unroll
             for (int i = 0; i < MT; ++i) areg[u][i] = keep_if(k_ok && a_ok[i], ldg16(ap[i] + ks));
         }
+        __builtin_amdgcn_sched_barrier(0);      // every load of the batch is issued before the first use
 #pragma unroll
         for (int u = 0; u < U; ++u)
 #pragma unroll
@@ -575,7 +576,13 @@ extern "C" int xr_gemm_bf16(void* out, const void* a, const void* w, const float
     }
     if (variant == 1) {
         XR_REQUIRE(M <= 64, "gemm: the skinny kernel takes at most 64 rows, got %d", M);
-        if (M <= 16) return sw ? launch_skinny<1, 1, 16, 8, true>(g, stream) : launch_skinny<1, 1, 16, 8, false>(g, stream);
+        if (M <= 16) {
+            // measured on MI355X at M = 1 and 8 (waves per workgroup, loads per batch):
+            if (sw) return launch_skinny<1, 1, 8, 8, true>(g, stream);
+            if (N >= 65536 || (N > 4096 && K <= 8192)) return launch_skinny<1, 2, 4, 8, false>(g, stream);
+            if (K > 8192) return launch_skinny<1, 1, 4, 8, false>(g, stream);
+            return launch_skinny<1, 1, 4, 16, false>(g, stream);
+        }
         if (M <= 32) return sw ? launch_skinny<2, 1, 16, 8, true>(g, stream) : launch_skinny<2, 1, 16, 8, false>(g, stream);
         return sw ? launch_skinny<4, 2, 8, 4, true>(g, stream) : launch_skinny<4, 2, 8, 4, false>(g, stream);
     }
