@@ -135,6 +135,28 @@ __global__ __launch_bounds__(256) void k_attn_mfma(AttnArgs a) {
         }                                                                                                \
     }
 
+    // The same loads for a tile that lies wholly inside the request (every page exists): no
+    // select touches the loaded words, so nothing waits for them until the tile is used.
+#define ATTN_LOAD_K_FAST(KT, KF)                                                                         \
+    {                                                                                                    \
+        const int key_ = (KT) + key_off;                                                                 \
+        const int pg_ = __shfl(my_page, (key_ >> a.page_shift) - pages_base, 64);                        \
+        const bf16_t* kp_ = kc + (((size_t)pg_ * a.Hk + kvh) * a.page_size + (key_ & a.page_mask)) * HD + lg * 8; \
+        _Pragma("unroll") for (int kd = 0; kd < KD; ++kd) KF[kd] = ldg16(kp_ + kd * 16);                 \
+    }
+#define ATTN_LOAD_V_FAST(KT, VF)                                                                         \
+    {                                                                                                    \
+        _Pragma("unroll") for (int j = 0; j < 2; ++j) {                                                  \
+            const int k8_ = (KT) + 16 * j + 8 * lg;                                                      \
+            const int pg_ = __shfl(my_page, (k8_ >> a.page_shift) - pages_base, 64);                     \
+            const bf16_t* vp_ = vc + (((size_t)pg_ * a.Hk + kvh) * HD + lr) * a.page_size + (k8_ & a.page_mask); \
+            _Pragma("unroll") for (int d = 0; d < DB; ++d) {                                             \
+                if (HD % 32 == 0 || d * 32 + lr < HD) VF[j][d] = ldg16(vp_ + (size_t)d * 32 * a.page_size); \
+                else VF[j][d] = make_uint4(0, 0, 0, 0);                                                  \
+            }                                                                                            \
+        }                                                                                                \
+    }
+
     f32x16 o[DB];
 #pragma unroll
     for (int d = 0; d < DB; ++d)
@@ -167,8 +189,13 @@ __global__ __launch_bounds__(256) void k_attn_mfma(AttnArgs a) {
                 my_page = bt[in ? pi : 0];
                 my_page = in ? my_page : -1;
             }
-            ATTN_LOAD_K(nx, kn)
-            ATTN_LOAD_V(nx, vn)
+            if (nx + 32 <= seq_len) {
+                ATTN_LOAD_K_FAST(nx, kn)
+                ATTN_LOAD_V_FAST(nx, vn)
+            } else {
+                ATTN_LOAD_K(nx, kn)
+                ATTN_LOAD_V(nx, vn)
+            }
         }
         if (kt + 32 > seq_len) {               // the request's last tile: slots past its end hold old data
 #pragma unroll
