@@ -34,6 +34,9 @@ struct GemmArgs {
     int out_bf16;      // storage of out
     int epi;
     int m_fast;        // tile order of the asynchronous kernel: 1 = consecutive workgroups share a weight tile
+    int splits;        // > 1: K is cut into this many ranges, each workgroup writes raw sums to `partial`
+    int k_per_split;   // columns per range (a multiple of 64)
+    float* partial;    // [splits][M][rows of w]
 };
 
 __device__ inline uint4 ldg16(const bf16_t* p) { return *reinterpret_cast<const uint4*>(p); }
@@ -272,8 +275,11 @@ __global__ __launch_bounds__(64 * WARPS_M * WARPS_N) void k_gemm_tile_async(Gemm
     // in its L2 while the weight tile of the moment is fetched once from memory for all.
     const int tiles_m = (g.M + BM - 1) / BM;
     const int tiles_n = (g.N + (g.epi == EPI_SWIGLU ? BN / 2 : BN) - 1) / (g.epi == EPI_SWIGLU ? BN / 2 : BN);
-    const int bm_ = g.m_fast ? (int)(blockIdx.x % tiles_m) : (int)(blockIdx.x / tiles_n);
-    const int bx = g.m_fast ? (int)(blockIdx.x / tiles_m) : (int)(blockIdx.x % tiles_n);
+    const int tile_ = (int)(blockIdx.x / g.splits), split_ = (int)(blockIdx.x % g.splits);
+    const int bm_ = g.m_fast ? tile_ % tiles_m : tile_ / tiles_n;
+    const int bx = g.m_fast ? tile_ / tiles_m : tile_ % tiles_n;
+    const int k_begin = split_ * g.k_per_split;
+    const int k_end = (k_begin + g.k_per_split) < g.K ? (k_begin + g.k_per_split) : g.K;
     const int m0 = bm_ * BM;
     const int n_rows = g.epi == EPI_SWIGLU ? 2 * g.N : g.N;
     const bf16_t* zero_src = reinterpret_cast<const bf16_t*>(xr_zero_chunk);
@@ -299,10 +305,10 @@ __global__ __launch_bounds__(64 * WARPS_M * WARPS_N) void k_gemm_tile_async(Gemm
     const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) void*)lds;
 #define ASYNC_ISSUE(KT)                                                                              \
     {                                                                                                \
-        const int k0_ = (KT) * BK;                                                                   \
+        const int k0_ = k_begin + (KT) * BK;                                                         \
         const uint32_t dst_ = lds_base + (uint32_t)((((KT) % STAGES) * BUF + wave * 64) * 16);       \
         _Pragma("unroll") for (int i = 0; i < LOADS; ++i) {                                          \
-            const bf16_t* p_ = (src[i] && k0_ + src_c[i] < g.K) ? src[i] + k0_ : zero_src;           \
+            const bf16_t* p_ = (src[i] && k0_ + src_c[i] < k_end) ? src[i] + k0_ : zero_src;         \
             lds_dma16(p_, __builtin_amdgcn_readfirstlane(dst_ + i * WAVES * 64 * 16));               \
         }                                                                                            \
     }
@@ -315,7 +321,7 @@ __global__ __launch_bounds__(64 * WARPS_M * WARPS_N) void k_gemm_tile_async(Gemm
 #pragma unroll
             for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
 
-    const int nk = (g.K + BK - 1) / BK;
+    const int nk = (k_end - k_begin + BK - 1) / BK;
 #pragma unroll
     for (int st = 0; st < STAGES - 1; ++st) ASYNC_ISSUE(st)
     const int lr = lane & 31, lg = lane >> 5;
@@ -350,6 +356,25 @@ __global__ __launch_bounds__(64 * WARPS_M * WARPS_N) void k_gemm_tile_async(Gemm
 #undef ASYNC_ISSUE
     wait_vmcnt<0>();                                     // the trailing loads of zeros
 
+    if (g.splits > 1) {
+        // raw sums of this K range, by weight row: the epilogue belongs to k_gemm_finish
+        const int ldp = g.epi == EPI_SWIGLU ? 2 * g.N : g.N;
+        float* part = g.partial + (size_t)split_ * g.M * ldp;
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j) {
+                int oc;
+                const int n = w_row_of<BN, WN>(wn0 + j * 32 + lr, bx, g.N, g.epi, oc);
+                if (oc >= g.N || n >= ldp) continue;
+#pragma unroll
+                for (int e = 0; e < 16; ++e) {
+                    int m = m0 + wm0 + i * 32 + (e / 4) * 8 + lg * 4 + (e % 4);
+                    if (m < g.M) part[(size_t)m * ldp + n] = acc[i][j][e];
+                }
+            }
+        return;
+    }
     if (g.epi == EPI_SWIGLU) {
 #pragma unroll
         for (int i = 0; i < TM; ++i)
@@ -382,8 +407,27 @@ __global__ __launch_bounds__(64 * WARPS_M * WARPS_N) void k_gemm_tile_async(Gemm
         }
 }
 
+// Sums the K ranges of a split product in a fixed order and applies the epilogue.
+__global__ __launch_bounds__(256) void k_gemm_finish(GemmArgs g) {
+    const int ldp = g.epi == EPI_SWIGLU ? 2 * g.N : g.N;
+    const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= (size_t)g.M * g.N) return;
+    const int m = (int)(idx / g.N), n = (int)(idx % g.N);
+    const size_t step = (size_t)g.M * ldp;
+    const float* p = g.partial + (size_t)m * ldp + n;
+    float v = 0.f, u = 0.f;
+    for (int s = 0; s < g.splits; ++s) v += p[s * step];
+    if (g.epi == EPI_SWIGLU) {
+        for (int s = 0; s < g.splits; ++s) u += p[s * step + g.N];
+        const float bg = g.bias ? g.bias[n] : 0.f, bu = g.bias ? g.bias[g.N + n] : 0.f;
+        store_out(g, m, n, silu_f(v + bg) * (u + bu));
+    } else {
+        store_out(g, m, n, v + (g.bias ? g.bias[n] : 0.f));
+    }
+}
+
 template <int BM, int BN, int WM_, int WN_, int ST>
-static int launch_tile_async(const GemmArgs& g, hipStream_t stream) {
+static int launch_tile_async(GemmArgs g, hipStream_t stream) {
     size_t smem = (size_t)ST * (BM + BN) * 8 * 16;
     static bool attr_set = false;
     if (!attr_set) {
@@ -393,9 +437,22 @@ static int launch_tile_async(const GemmArgs& g, hipStream_t stream) {
         attr_set = true;
     }
     int n_out_tile = g.epi == EPI_SWIGLU ? BN / 2 : BN;
-    unsigned grid = (unsigned)(((g.N + n_out_tile - 1) / n_out_tile) * ((g.M + BM - 1) / BM));
-    k_gemm_tile_async<BM, BN, WM_, WN_, ST><<<grid, 64 * WM_ * WN_, smem, stream>>>(g);
+    unsigned tiles = (unsigned)(((g.N + n_out_tile - 1) / n_out_tile) * ((g.M + BM - 1) / BM));
+    if (g.splits < 1 || !g.partial) g.splits = 1;
+    if (g.splits > 1) {
+        int slices = (g.K + 63) / 64;
+        int per = (slices + g.splits - 1) / g.splits;
+        g.k_per_split = per * 64;
+        g.splits = (slices + per - 1) / per;            // no empty range
+    }
+    if (g.splits == 1) g.k_per_split = ((g.K + 63) / 64) * 64;
+    k_gemm_tile_async<BM, BN, WM_, WN_, ST><<<tiles * g.splits, 64 * WM_ * WN_, smem, stream>>>(g);
     XR_CHECK_LAUNCH("gemm_tile_async");
+    if (g.splits > 1) {
+        size_t n = (size_t)g.M * g.N;
+        k_gemm_finish<<<(unsigned)((n + 255) / 256), 256, 0, stream>>>(g);
+        XR_CHECK_LAUNCH("gemm_finish");
+    }
     return XR_OK;
 }
 
@@ -547,8 +604,10 @@ static int launch_tile(const GemmArgs& g, hipStream_t stream) {
 
 // epi: 0 store, 1 add into float out, 2 SwiGLU (w has 2N rows: gate rows then up rows).
 // variant: 0 = choose by M; 1 = skinny; 2 = tile 128x128; 3 = tile 256x128.
+// workspace (may be null): room for split products, workspace_bytes long; without it K is not split.
 extern "C" int xr_gemm_bf16(void* out, const void* a, const void* w, const float* bias, int M, int N, int K,
-                            int lda, int ldo, int out_dtype, int epi, int variant, hipStream_t stream) {
+                            int lda, int ldo, int out_dtype, int epi, int variant, float* workspace,
+                            size_t workspace_bytes, hipStream_t stream) {
     XR_REQUIRE(M >= 0 && N > 0 && K > 0, "gemm: bad sizes M=%d N=%d K=%d", M, N, K);
     XR_REQUIRE(lda >= K && ldo >= N, "gemm: row strides lda=%d ldo=%d are shorter than K=%d N=%d", lda, ldo, K, N);
     XR_REQUIRE(K % 8 == 0 && lda % 8 == 0, "gemm: the MFMA kernels need K (%d) and the row stride (%d) to be multiples of 8", K, lda);
@@ -560,18 +619,31 @@ extern "C" int xr_gemm_bf16(void* out, const void* a, const void* w, const float
     GemmArgs g;
     g.a = (const bf16_t*)a; g.w = (const bf16_t*)w; g.bias = bias; g.out = out;
     g.M = M; g.N = N; g.K = K; g.lda = lda; g.ldo = ldo; g.out_bf16 = out_dtype == XR_BF16; g.epi = epi;
-    g.m_fast = 0;
+    g.m_fast = 0; g.splits = 1; g.k_per_split = 0; g.partial = workspace;
     if (variant >= 1000) { g.m_fast = 1; variant -= 1000; }
     const bool sw = epi == EPI_SWIGLU;
+    const int w_rows = epi == EPI_SWIGLU ? 2 * N : N;
+    // K ranges so that about 320 workgroups run, if the workspace has room for their sums
+    auto pick_splits = [&](int tiles) {
+        int s = (320 + tiles - 1) / tiles;
+        int max_s = K / 256 > 0 ? K / 256 : 1;
+        s = s < 1 ? 1 : (s > max_s ? max_s : s);
+        while (s > 1 && (size_t)s * M * w_rows * 4 > workspace_bytes) --s;
+        return workspace ? s : 1;
+    };
     if (variant == 0) {
-        if (M <= 64) {
+        if (M <= 16) {
             variant = 1;
+        } else if (M <= 64) {
+            variant = 31;
         } else {
-            // the largest tile that still gives every compute unit a workgroup
+            // the largest tile that still gives every compute unit a workgroup; if even the
+            // smallest does not, K is split as well
             const int n_out = N;
             auto count = [&](int bm, int bn) { return ((M + bm - 1) / bm) * ((n_out + (sw ? bn / 2 : bn) - 1) / (sw ? bn / 2 : bn)); };
             variant = count(256, 256) >= 180 ? 14 : (count(256, 128) >= 180 ? 12 : 17);
             g.m_fast = 1;
+            if (variant == 17 && count(128, 128) < 160) g.splits = pick_splits(count(128, 128));
         }
     }
     if (variant == 1) {
@@ -615,6 +687,12 @@ extern "C" int xr_gemm_bf16(void* out, const void* a, const void* w, const float
     if (variant == 18) return launch_tile_async<256, 256, 2, 2, 2>(g, stream);
     if (variant == 19) return launch_tile_async<256, 128, 2, 2, 2>(g, stream);
     if (variant == 20) return launch_tile_async<128, 256, 2, 2, 2>(g, stream);
+    if (variant == 30 || variant == 31) {       // few rows: 32 or 64 of them against 128 weight rows, K split
+        const int bn_out = sw ? 64 : 128;
+        g.splits = pick_splits((N + bn_out - 1) / bn_out);
+        if (variant == 30) return launch_tile_async<32, 128, 1, 2, 3>(g, stream);
+        return launch_tile_async<64, 128, 2, 2, 3>(g, stream);
+    }
     xr_set_error("gemm: unknown variant %d", variant);
     return XR_BAD_ARG;
 }

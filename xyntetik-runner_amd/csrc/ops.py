@@ -42,7 +42,7 @@ _PROTOS = {
     "xr_fill_rows": [_p, _p, _i, _sz, _u32, _p],
     "xr_convert": [_p, _p, _sz, _i, _i, _p],
     "xr_gemm_ref": [_p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _p],
-    "xr_gemm_bf16": [_p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _p],
+    "xr_gemm_bf16": [_p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _p, _sz, _p],
     "xr_attention_ref": [_p, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _f, _i, _i, _p],
     "xr_sample": [_p, _p, _i, _i, _i, _p, _p, _p, _p, _p, _p, _p, _p, _i, _p, _i, _p],
 }
@@ -160,6 +160,17 @@ class Ops:
         return out
 
     # -- matrix product ---------------------------------------------------------
+    GEMM_WORKSPACE_BYTES = 32 << 20
+
+    def _gemm_workspace(self, device):
+        """Room for the sums of K ranges when a product with few rows is split (one buffer per process;
+        products on one stream use it one after another)."""
+        ws = getattr(self, "_gemm_ws", None)
+        if ws is None or ws.device != device:
+            ws = torch.empty((self.GEMM_WORKSPACE_BYTES // 4,), dtype=torch.float32, device=device)
+            self._gemm_ws = ws
+        return ws.data_ptr(), self.GEMM_WORKSPACE_BYTES
+
     def _mfma_ok(self, a: torch.Tensor, w: torch.Tensor) -> bool:
         return (self.use_mfma and a.dtype == torch.bfloat16 and a.shape[1] % 8 == 0 and a.stride(0) % 8 == 0
                 and a.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0)
@@ -193,7 +204,8 @@ class Ops:
         if self._mfma_ok(a, w):
             self.lib.check(self.lib.xr_gemm_bf16(out.data_ptr(), a.data_ptr(), w.data_ptr(), _ptr(bias), M, N, K,
                                                  a.stride(0), out.stride(0), dtype_code(out.dtype),
-                                                 1 if accumulate else 0, variant, _stream()))
+                                                 1 if accumulate else 0, variant, *self._gemm_workspace(a.device),
+                                                 _stream()))
             return out
         self.lib.check(self.lib.xr_gemm_ref(out.data_ptr(), a.data_ptr(), w.data_ptr(), _ptr(bias), M, N, K,
                                             a.stride(0), out.stride(0), dtype_code(a.dtype),
@@ -216,7 +228,8 @@ class Ops:
                 raise KernelError("linear_swiglu: bias must be float32 [2F]")
             out = torch.empty((M, F), dtype=a.dtype, device=a.device)
             self.lib.check(self.lib.xr_gemm_bf16(out.data_ptr(), a.data_ptr(), w.data_ptr(), _ptr(bias), M, F, K,
-                                                 a.stride(0), F, dtype_code(out.dtype), 2, variant, _stream()))
+                                                 a.stride(0), F, dtype_code(out.dtype), 2, variant,
+                                                 *self._gemm_workspace(a.device), _stream()))
             return out
         return self.silu_mul(self.linear(a, w, bias=bias))
 
