@@ -24,6 +24,7 @@ WORKLOAD = {
     "A": ([5, 17, 33, 64, 150], 16),
     "B": ([1, 9, 40, 64, 100], 24),
     "C": ([3, 31, 70], 40),
+    "D": ([200, 70, 330], 34),
 }
 
 
@@ -69,11 +70,11 @@ def check(got, want, dtype, what):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("which", ["A", "B", "C"])
+@pytest.mark.parametrize("which", ["A", "B", "C", "D"])
 @pytest.mark.parametrize("schedule", ["whole", "tail", "portions", "mixed"])
 def test_schedules_match_plain(models, tmp_path, which, dtype, schedule):
     d, cfg, reqs, plens, want = models[which]
-    page_size = {"A": 16, "B": 64, "C": 4}[which]
+    page_size = {"A": 16, "B": 64, "C": 4, "D": 64}[which]
     if schedule == "whole":
         steps = traces.whole(reqs)
     elif schedule == "tail":

@@ -34,10 +34,22 @@ TINY_C = {
     "attention_bias": True, "mlp_bias": True, "hidden_act": "silu",
 }
 
+# the benchmark model's head size and grouping at a small width: 128-wide heads, 4 query heads per
+# key/value head, prompts long enough for the large-tile matrix kernels and 64-position pages
+TINY_D = {
+    "architectures": ["LlamaForCausalLM"], "model_type": "llama",
+    "num_hidden_layers": 2, "hidden_size": 256, "num_attention_heads": 8, "num_key_value_heads": 2,
+    "head_dim": 128, "intermediate_size": 544, "vocab_size": 1000, "rope_theta": 500000.0,
+    "rope_scaling": {"rope_type": "llama3", "factor": 8.0, "low_freq_factor": 1.0, "high_freq_factor": 4.0,
+                     "original_max_position_embeddings": 64},
+    "rms_norm_eps": 1e-5, "tie_word_embeddings": False, "max_position_embeddings": 1024, "hidden_act": "silu",
+}
+
 MAKE = {
     "A": dict(config=TINY_A, seed=0, norm_jitter=0.0, dtype="bfloat16", vector_dtype=None),
     "B": dict(config=TINY_B, seed=1, norm_jitter=0.1, dtype="bfloat16", vector_dtype="float32"),
     "C": dict(config=TINY_C, seed=2, norm_jitter=0.1, dtype="bfloat16", vector_dtype="float32"),
+    "D": dict(config=TINY_D, seed=3, norm_jitter=0.05, dtype="bfloat16", vector_dtype=None),
 }
 
 

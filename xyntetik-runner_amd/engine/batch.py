@@ -79,6 +79,9 @@ def plan_attention(starts, q_lens, group_size: int, window: Optional[int], n_kv_
     if blocks and len(blocks) * n_kv_heads < 2048:         # too few row blocks to fill the chip
         chunk = tiles_per_item(total_tiles, n_kv_heads)
     items, jobs, slot = [], [], 0
+    # longest first: workgroups are started in list order, and a long item started last
+    # would run on alone at the end
+    blocks.sort(key=lambda blk: -blk[4])
     for b, row0, lo, hi, tiles in blocks:
         parts = -(-tiles // chunk)
         if parts <= 1:
