@@ -145,9 +145,10 @@ def test_linear_refuses_bad_operands(ops):
 class FakeCtx:
     """The part of a step's context that the attention kernels read."""
 
-    def __init__(self, starts, q_lens, tables, page_size):
+    def __init__(self, starts, q_lens, tables, page_size, cta_tiles=None):
         from xyntetik_runner_amd.engine.batch import plan_attention, AttentionPlan
         self.starts, self.q_lens = list(starts), list(q_lens)
+        self.cta_tiles = cta_tiles
         pos, rot, cu = [], [], [0]
         for b, (s, n) in enumerate(zip(starts, q_lens)):
             pos += list(range(s, s + n)); rot += [b] * n; cu.append(cu[-1] + n)
@@ -163,11 +164,12 @@ class FakeCtx:
     def block_table(self, group):
         return self._table
 
-    def attention_plan(self, group, G, window, Hk):
-        items, jobs, n_slots = self._plan_fn(self.starts, self.q_lens, G, window, Hk)
-        it = torch.tensor([v for i in items for v in i], dtype=torch.int32, device=DEV)
+    def attention_plan(self, group, G, window, Hk, page_size=64):
+        cta, items, jobs, n_slots = self._plan_fn(self.starts, self.q_lens, G, window, Hk, page_size,
+                                                  cta_tiles=self.cta_tiles)
+        it = torch.tensor([v for i in cta + items for v in i], dtype=torch.int32, device=DEV)
         jb = torch.tensor([v for j in jobs for v in j], dtype=torch.int32, device=DEV) if jobs else None
-        return self._Plan(it, len(items), jb, len(jobs), n_slots)
+        return self._Plan(it, len(items), jb, len(jobs), n_slots, len(cta))
 
 
 def scatter_pages(n_req_lens, page_size, seed):
@@ -293,6 +295,43 @@ def test_attention(ops, dt, case):
     assert rel(got, want) < (3e-6 if dt == "float32" else 1.2e-2)
 
 
+ATTN_WORKGROUP_CASES = [
+    # H, Hk, D, page, window, starts, q_lens, most tiles per 128-row item (None: the engine's choice)
+    (8, 2, 128, 64, None, [0], [300], None),
+    (8, 2, 128, 64, None, [0], [300], 2),              # key ranges, merged afterwards
+    (4, 1, 80, 32, None, [37, 0, 500], [130, 64, 1], 3),   # head size no power of two; a decoded token beside
+    (6, 2, 256, 64, 100, [200], [150], None),          # window; the largest head
+    (2, 2, 16, 32, None, [5], [70], 1),
+    (5, 1, 64, 128, 33, [1000, 3], [90, 40], 4),       # five heads a group: rows of a token straddle waves
+    (3, 3, 48, 32, 9, [60], [200], None),              # a window shorter than a tile
+]
+
+
+@pytest.mark.parametrize("case", ATTN_WORKGROUP_CASES)
+def test_attention_long_portions(ops, case):
+    """Portions of 64 rows and more go to the kernel that shares key and value tiles in a workgroup."""
+    H, Hk, D, ps, window, starts, q_lens, cta_tiles = case
+    torch.manual_seed(H * 100 + D)
+    lens = [s + n for s, n in zip(starts, q_lens)]
+    tables, n_pages = scatter_pages(lens, ps, D)
+    ctx = FakeCtx(starts, q_lens, tables, ps, cta_tiles=cta_tiles)
+    plan = ctx.attention_plan(0, H // Hk, window, Hk, ps)
+    assert plan.n_cta_items > 0
+    T = sum(q_lens)
+    q = torch.randn(T, H, D).bfloat16()
+    k_seq = [torch.randn(n, Hk, D).bfloat16() for n in lens]
+    v_seq = [torch.randn(n, Hk, D).bfloat16() for n in lens]
+    kc, vc = fill_cache(k_seq, v_seq, tables, n_pages, ps, torch.bfloat16)
+    scale = 1 / math.sqrt(D)
+    want = ref_attention(q.float(), [k.float() for k in k_seq], [v.float() for v in v_seq], starts, q_lens, scale, window)
+    got = ops.attention(q.to(DEV).reshape(T, H * D).contiguous(), kc, vc, ctx, 0, H, Hk, D, ps, scale, window)
+    got = got.cpu().reshape(T, H, D)
+    assert torch.isfinite(got.float()).all(), "read a slot no request owns"
+    # row by row, so that a wrong row among hundreds shows
+    err = (got.double() - want).abs().amax(dim=(1, 2)) / want.abs().amax()
+    assert err.max() < 1.2e-2, f"token {int(err.argmax())}: {float(err.max())}"
+
+
 @pytest.mark.parametrize("dt", ["float32", "bfloat16"])
 @pytest.mark.parametrize("far", [0, 15, 16, 31, 32, 63, 64, 255, 256, 700, 1023])
 def test_attention_finds_one_far_key(ops, dt, far):
@@ -339,21 +378,32 @@ def test_attention_window_edge(ops, dt):
 
 def test_attention_plan_covers_every_key_once():
     from xyntetik_runner_amd.engine.batch import plan_attention
-    for starts, q_lens, G, window, Hk in [([0, 100, 4000], [70, 1, 1], 4, None, 8), ([5000], [1], 4, None, 8),
-                                          ([0], [2048], 4, None, 8), ([300, 2], [1, 9], 2, 50, 1)]:
-        items, jobs, n_slots = plan_attention(starts, q_lens, G, window, Hk)
-        by_block = {}
-        for b, row0, k0, k1, slot, *_ in items:
-            assert k0 % 32 == 0 and k0 < k1
-            by_block.setdefault((b, row0), []).append((k0, k1, slot))
-        for (b, row0), parts in by_block.items():
-            parts.sort()
-            n = q_lens[b]
-            hi = starts[b] + min(n - 1, (row0 + 31) // G) + 1
-            lo = 0 if not window else max(0, starts[b] + row0 // G - window + 1)
-            assert parts[0][0] <= lo and parts[-1][1] == hi
-            assert all(a[1] == c[0] for a, c in zip(parts, parts[1:]))
-            assert (len(parts) == 1) == (parts[0][2] == -1)
-        slots = sorted(s for it in items if (s := it[4]) >= 0)
-        assert slots == list(range(n_slots))
-        assert sum(j[3] for j in jobs) == n_slots
+    for starts, q_lens, G, window, Hk, cta_tiles in [
+            ([0, 100, 4000], [70, 1, 1], 4, None, 8, None), ([5000], [1], 4, None, 8, None),
+            ([0], [2048], 4, None, 8, None), ([300, 2], [1, 9], 2, 50, 1, None),
+            ([10, 0], [333, 15], 3, 40, 2, 2), ([0], [100], 5, None, 1, 1)]:
+        cta_items, items, jobs, n_slots = plan_attention(starts, q_lens, G, window, Hk, 64, cta_tiles)
+        used = []
+        for rows, waves, some in ((128, 4, cta_items), (32, 1, items)):
+            by_block = {}
+            for b, row0, k0, k1, slot, q0, q_len, start in some:
+                assert k0 % 32 == 0 and k0 < k1
+                assert q0 == sum(q_lens[:b]) and q_len == q_lens[b] and start == starts[b]
+                by_block.setdefault((b, row0), []).append((k0, k1, slot))
+            for (b, row0), parts in by_block.items():
+                parts.sort()
+                n = q_lens[b]
+                hi = starts[b] + min(n - 1, (row0 + rows - 1) // G) + 1
+                lo = 0 if not window else max(0, starts[b] + row0 // G - window + 1)
+                assert parts[0][0] <= lo and parts[-1][1] == hi
+                assert all(a[1] == c[0] for a, c in zip(parts, parts[1:]))
+                assert (len(parts) == 1) == (parts[0][2] == -1)
+                if len(parts) > 1:
+                    for w in range(waves):              # every 32-row block that exists is merged from its slots
+                        if row0 + 32 * w < n * G:
+                            assert (b, row0 + 32 * w, parts[0][2] + w, len(parts), waves) in jobs
+                    used += [p[2] + w for p in parts for w in range(waves)]
+        # a row belongs to one kind of item only
+        assert not {(b, r // 128) for b, r, *_ in cta_items} & {(b, r // 128) for b, r, *_ in items}
+        assert sorted(used) == list(range(n_slots))
+        assert sum(j[3] for j in jobs if j[1] // 32 * 32 == j[1]) <= n_slots

@@ -21,6 +21,7 @@
 // results that k_attn_merge combines (/root/reference/src/kernels.cu:2171-2270 does this
 // with 8 fixed slices for decoding).
 #include "common.h"
+#include "async_copy.h"
 
 #ifndef XR_HEAD_DIM
 #error "compile with -DXR_HEAD_DIM=<head size>"
@@ -36,6 +37,7 @@ static_assert(HD % 16 == 0 && HD >= 16 && HD <= 256, "head size must be a multip
 
 #define ITEM_INTS 8                   // req, row0, k_begin, k_end, slot (-1: final), q0, q_len, start
 #define ROWS 32
+#define JOB_INTS 5                    // req, row0, first slot, slots, distance between slots
 
 struct AttnArgs {
     const bf16_t* q;        // [T, H, HD]
@@ -43,13 +45,14 @@ struct AttnArgs {
     const bf16_t* vc;       // [pages, Hk, HD, page_size]
     bf16_t* out;            // [T, H, HD]
     const int* items;       // [n_items, ITEM_INTS]; q0: the request's first row, start: its first position
+    const int* cta_items;   // [n_cta_items, ITEM_INTS]: the same for 128-row blocks that a whole workgroup takes
     const int* cu_q;        // [B + 1] first row (token) of each request in this step
     const int* starts;      // [B] position of each request's first token of this step
     const int* block_table; // [B, table_stride]
     int table_stride;
     float* part_o;          // [slots, Hk, ROWS, HD]
     float* part_ml;         // [slots, Hk, ROWS, 2]
-    int n_items, H, Hk, page_shift, page_mask, page_size;
+    int n_items, n_cta_items, H, Hk, page_shift, page_mask, page_size;
     float scale;
     int window;
 };
@@ -64,6 +67,90 @@ __device__ inline uint4 keep_if(bool ok, uint4 v) {     // zero unless ok, word 
     return make_uint4(ok ? v.x : 0u, ok ? v.y : 0u, ok ? v.z : 0u, ok ? v.w : 0u);
 }
 __device__ inline uint32_t pack2(float lo, float hi) { return pack_bf16x2(lo, hi); }
+
+// One tile's softmax step for the lane's row: p[] from s[], the running maximum m and sum l,
+// and the rescaling of the output accumulators when the maximum moved.
+#define ATTN_SOFTMAX_STEP(KT, KEND)                                                                  \
+        if ((KT) + 32 <= (KEND) && (KT) + 31 <= pos_min && (KT) >= lo_max) {                             \
+            float mt = fmaxf(fmaxf(s[0], s[1]), fmaxf(s[2], s[3]));                                      \
+_Pragma("unroll")                                                                                        \
+            for (int e = 4; e < 16; e += 4) mt = fmaxf(mt, fmaxf(fmaxf(s[e], s[e + 1]), fmaxf(s[e + 2], s[e + 3]))); \
+            mt = fmaxf(mt, __shfl_xor(mt, 32, 64));                                                      \
+            const float mn = fmaxf(m, mt * c2);                                                          \
+            corr = __builtin_amdgcn_exp2f(m - mn);                                                       \
+            float rs = 0.f;                                                                              \
+_Pragma("unroll")                                                                                        \
+            for (int e = 0; e < 16; ++e) {                                                               \
+                p[e] = __builtin_amdgcn_exp2f(fmaf(s[e], c2, -mn));                                      \
+                rs += p[e];                                                                              \
+            }                                                                                            \
+            rs += __shfl_xor(rs, 32, 64);                                                                \
+            l = fmaf(l, corr, rs);                                                                       \
+            m = mn;                                                                                      \
+        } else {                                                                                         \
+            float mt = -INFINITY;                                                                        \
+_Pragma("unroll")                                                                                        \
+            for (int e = 0; e < 16; ++e) {                                                               \
+                const int key = (KT) + 16 * (e >> 3) + 8 * lg + (e & 7);                                 \
+                const bool ok = row_ok && key <= pos && key >= lo && key < (KEND);                       \
+                p[e] = ok ? s[e] * c2 : -INFINITY;                                                       \
+                mt = fmaxf(mt, p[e]);                                                                    \
+            }                                                                                            \
+            mt = fmaxf(mt, __shfl_xor(mt, 32, 64));                                                      \
+            const float mn = fmaxf(m, mt);                                                               \
+            const float mu = mn == -INFINITY ? 0.f : mn;                                                 \
+            corr = __builtin_amdgcn_exp2f(m - mu);                                                       \
+            float rs = 0.f;                                                                              \
+_Pragma("unroll")                                                                                        \
+            for (int e = 0; e < 16; ++e) {                                                               \
+                p[e] = __builtin_amdgcn_exp2f(p[e] - mu);                                                \
+                rs += p[e];                                                                              \
+            }                                                                                            \
+            rs += __shfl_xor(rs, 32, 64);                                                                \
+            l = fmaf(l, corr, rs);                                                                       \
+            m = mn;                                                                                      \
+        }                                                                                                \
+        if (__any(corr != 1.0f)) {                                                                       \
+_Pragma("unroll")                                                                                        \
+            for (int d = 0; d < DB; ++d)                                                                 \
+_Pragma("unroll")                                                                                        \
+                for (int e = 0; e < 16; ++e) o[d][e] *= corr;                                            \
+        }
+
+// Writing a row's result: the final output, or the partial result of a key range.
+#define ATTN_WRITE_OUT(SLOT)                                                                         \
+    const float inv = l > 0.f ? 1.0f / l : 0.f;                                                          \
+    if (!row_ok) return;                                                                                 \
+    if ((SLOT) < 0) {                                                                                    \
+        bf16_t* op = a.out + ((size_t)t * a.H + h) * HD;                                                 \
+_Pragma("unroll")                                                                                        \
+        for (int d = 0; d < DB; ++d)                                                                     \
+_Pragma("unroll")                                                                                        \
+            for (int e4 = 0; e4 < 4; ++e4) {                                                             \
+                const int dd = d * 32 + e4 * 8 + lg * 4;                                                 \
+                if (dd < HD) {                                                                           \
+                    uint2 w = make_uint2(pack2(o[d][e4 * 4 + 0] * inv, o[d][e4 * 4 + 1] * inv),          \
+                                         pack2(o[d][e4 * 4 + 2] * inv, o[d][e4 * 4 + 3] * inv));         \
+                    *reinterpret_cast<uint2*>(op + dd) = w;                                              \
+                }                                                                                        \
+            }                                                                                            \
+        return;                                                                                          \
+    }                                                                                                    \
+    float* po = a.part_o + (((size_t)(SLOT) * a.Hk + kvh) * ROWS + lr) * HD;                             \
+_Pragma("unroll")                                                                                        \
+    for (int d = 0; d < DB; ++d)                                                                         \
+_Pragma("unroll")                                                                                        \
+        for (int e4 = 0; e4 < 4; ++e4) {                                                                 \
+            const int dd = d * 32 + e4 * 8 + lg * 4;                                                     \
+            if (dd < HD)                                                                                 \
+                *reinterpret_cast<float4*>(po + dd) = make_float4(o[d][e4 * 4 + 0] * inv, o[d][e4 * 4 + 1] * inv, \
+                                                                  o[d][e4 * 4 + 2] * inv, o[d][e4 * 4 + 3] * inv); \
+        }                                                                                                \
+    if (lg == 0) {                                                                                       \
+        float* pm = a.part_ml + (((size_t)(SLOT) * a.Hk + kvh) * ROWS + lr) * 2;                         \
+        pm[0] = m;                                                                                       \
+        pm[1] = l;                                                                                       \
+    }
 
 __global__ __launch_bounds__(256) void k_attn_mfma(AttnArgs a) {
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -218,55 +305,9 @@ __global__ __launch_bounds__(256) void k_attn_mfma(AttnArgs a) {
 #pragma unroll
         for (int kd = 0; kd < KD; ++kd)
             s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16x8(kf[kd]), qf[kd], s, 0, 0, 0);
-        // ---- running maximum and sum, in units of log2: p = 2^(s*c - m), c = scale * log2(e)
         float p[16];
         float corr;
-        if (kt + 32 <= kend && kt + 31 <= pos_min && kt >= lo_max) {
-            // every key of the tile is visible to every row: no mask
-            float mt = fmaxf(fmaxf(s[0], s[1]), fmaxf(s[2], s[3]));
-#pragma unroll
-            for (int e = 4; e < 16; e += 4) mt = fmaxf(mt, fmaxf(fmaxf(s[e], s[e + 1]), fmaxf(s[e + 2], s[e + 3])));
-            mt = fmaxf(mt, __shfl_xor(mt, 32, 64));
-            const float mn = fmaxf(m, mt * c2);
-            corr = __builtin_amdgcn_exp2f(m - mn);
-            float rs = 0.f;
-#pragma unroll
-            for (int e = 0; e < 16; ++e) {
-                p[e] = __builtin_amdgcn_exp2f(fmaf(s[e], c2, -mn));
-                rs += p[e];
-            }
-            rs += __shfl_xor(rs, 32, 64);
-            l = fmaf(l, corr, rs);
-            m = mn;
-        } else {
-            float mt = -INFINITY;
-#pragma unroll
-            for (int e = 0; e < 16; ++e) {
-                const int key = kt + 16 * (e >> 3) + 8 * lg + (e & 7);
-                const bool ok = row_ok && key <= pos && key >= lo && key < kend;
-                p[e] = ok ? s[e] * c2 : -INFINITY;
-                mt = fmaxf(mt, p[e]);
-            }
-            mt = fmaxf(mt, __shfl_xor(mt, 32, 64));
-            const float mn = fmaxf(m, mt);
-            const float mu = mn == -INFINITY ? 0.f : mn;
-            corr = __builtin_amdgcn_exp2f(m - mu);
-            float rs = 0.f;
-#pragma unroll
-            for (int e = 0; e < 16; ++e) {
-                p[e] = __builtin_amdgcn_exp2f(p[e] - mu);
-                rs += p[e];
-            }
-            rs += __shfl_xor(rs, 32, 64);
-            l = fmaf(l, corr, rs);
-            m = mn;
-        }
-        if (__any(corr != 1.0f)) {             // the maximum moved for some row
-#pragma unroll
-            for (int d = 0; d < DB; ++d)
-#pragma unroll
-                for (int e = 0; e < 16; ++e) o[d][e] *= corr;
-        }
+        ATTN_SOFTMAX_STEP(kt, kend)
         // ---- O^T += V^T P^T
 #pragma unroll
         for (int j = 0; j < 2; ++j) {
@@ -287,46 +328,206 @@ __global__ __launch_bounds__(256) void k_attn_mfma(AttnArgs a) {
         }
     }
 
-    // ---- write: lane owns row `rho`; register e of block d is channel d*32 + (e/4)*8 + lg*4 + e%4
-    const float inv = l > 0.f ? 1.0f / l : 0.f;
-    if (!row_ok) return;
-    if (slot < 0) {
-        bf16_t* op = a.out + ((size_t)t * a.H + h) * HD;
+    ATTN_WRITE_OUT(slot)
+}
+
+// ------------------------------------------------------------------------------ workgroup kernel
+// Long prompt portions: a workgroup of 4 waves takes 128 consecutive rows of one request and
+// key/value head (wave w the rows row0 + 32 w ..) and a range of keys.  The K tile
+// [32 keys][HD] and the V^T tile [HD][32 keys] are copied once into LDS for all four waves,
+// by asynchronous copies that run CTA_STAGES - 1 tiles ahead (measured at head size 128: 4 tiles
+// in LDS give 10% over 3, 5 nothing more), instead of once per wave from
+// the caches; each wave then works as above with its fragments read from LDS.  A wave skips
+// the tiles that none of its rows can see, but takes part in every copy and barrier.
+//
+// LDS places are 16-byte chunks.  K: row r (key kt + r) has its chunk c at r * KSTR + c',
+// c' = c ^ (r mod CK) where CK is a power of two, else c with rows one chunk apart more
+// than their length, so that the lanes of a fragment read (32 rows, one column) fall into
+// different banks.  V^T: channel d has the 4 chunks of its 32 keys at d * 4 + (c ^ (d/4 mod 4)).
+constexpr int CK = HD / 8;                                  // chunks of a key row
+constexpr bool CK_POW2 = (CK & (CK - 1)) == 0;
+constexpr int KSTR = CK_POW2 ? CK : CK + 1;                 // chunks between key rows
+constexpr int NKC = 32 * KSTR;                              // chunks of a K tile
+constexpr int NVC = DB * 32 * 4;                            // chunks of a V^T tile
+constexpr int CTA_ROWS = 128;
+constexpr int CTA_LOADS = (NKC + NVC + 255) / 256;          // copies per lane and tile
+constexpr int STAGE_CHUNKS = CTA_LOADS * 256;
+constexpr int CTA_STAGES = STAGE_CHUNKS * 16 * 4 <= 64 * 1024 ? 4 : 3;   // tiles in LDS: two workgroups a compute unit, or one
+static_assert(CTA_LOADS * (CTA_STAGES - 2) < 64, "too many copies in flight for the counter");
+
+__global__ __launch_bounds__(256, 2) void k_attn_cta(AttnArgs a) {
+    extern __shared__ uint4 lds[];                          // [CTA_STAGES][STAGE_CHUNKS]
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int kvh = blockIdx.y;
+    const int* it = a.cta_items + (size_t)blockIdx.x * ITEM_INTS;
+    const int req = it[0], row0 = it[1] + wave * ROWS, kbeg = it[2], kend = it[3];
+    const int slot = it[4] < 0 ? -1 : it[4] + wave;
+    const int q0 = it[5], q_len = it[6], start = it[7];
+    const int G = a.H / a.Hk;
+    const int lr = lane & 31, lg = lane >> 5;
+    const int seq_len = start + q_len;
+    const int* bt = a.block_table + (size_t)req * a.table_stride;
+
+    // this lane's query row
+    const int rho = row0 + lr;
+    const int tok = rho / G, hg = rho - tok * G;
+    const bool row_ok = tok < q_len;
+    const int t = q0 + tok, h = kvh * G + hg;
+    const int pos = start + tok;
+    const int lo = (a.window > 0 && pos - a.window + 1 > 0) ? pos - a.window + 1 : 0;
+
+    bf16x8 qf[KD];
+    {
+        const bf16_t* qp = a.q + ((size_t)(row_ok ? t : q0) * a.H + h) * HD + lg * 8;
 #pragma unroll
-        for (int d = 0; d < DB; ++d)
-#pragma unroll
-            for (int e4 = 0; e4 < 4; ++e4) {
-                const int dd = d * 32 + e4 * 8 + lg * 4;
-                if (dd < HD) {
-                    uint2 w = make_uint2(pack2(o[d][e4 * 4 + 0] * inv, o[d][e4 * 4 + 1] * inv),
-                                         pack2(o[d][e4 * 4 + 2] * inv, o[d][e4 * 4 + 3] * inv));
-                    *reinterpret_cast<uint2*>(op + dd) = w;
-                }
-            }
-        return;
+        for (int kd = 0; kd < KD; ++kd) qf[kd] = as_bf16x8(keep_if(row_ok, ldg16(qp + kd * 16)));
     }
-    float* po = a.part_o + (((size_t)slot * a.Hk + kvh) * ROWS + lr) * HD;
+    const int ra = lr >> 3, rg = (lr >> 2) & 1, rb = lr & 3;
+    const int key_off = 16 * (ra >> 1) + 8 * rg + 4 * (ra & 1) + rb;
+
+    // the pieces this lane copies for every tile
+    int src_off[CTA_LOADS], src_key[CTA_LOADS];
+    bool src_is_k[CTA_LOADS];
+#pragma unroll
+    for (int i = 0; i < CTA_LOADS; ++i) {
+        const int q = i * 256 + tid;
+        src_is_k[i] = q < NKC;
+        if (q < NKC) {
+            const int r = q / KSTR, cs = q - r * KSTR;
+            const int c = CK_POW2 ? (cs ^ (r & (CK - 1))) : cs;
+            src_off[i] = r * HD + c * 8;
+            src_key[i] = cs < CK ? r : (1 << 30);           // the spare chunk of a row stays zero
+        } else {
+            const int v = q - NKC, d = v >> 2, c = (v & 3) ^ ((d >> 2) & 3);
+            src_off[i] = d * a.page_size + c * 8;
+            src_key[i] = (v < NVC && d < HD) ? c * 8 : (1 << 30);
+        }
+    }
+    const bf16_t* __restrict__ kc = a.kc;
+    const bf16_t* __restrict__ vc = a.vc;
+    const bf16_t* zero_src = reinterpret_cast<const bf16_t*>(xr_zero_chunk);
+    const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) void*)lds;
+
+    // page numbers of the item's keys, one per lane, 64 pages at a time
+    int pages_base = kbeg >> a.page_shift;
+    int my_page;
+    {
+        const int pi = pages_base + lane;
+        const bool in = ((long)pi << a.page_shift) < seq_len;
+        my_page = bt[in ? pi : 0];
+        my_page = in ? my_page : -1;
+    }
+    const int nt = (kend - kbeg + 31) >> 5;
+    // a tile lies within one page (pages hold at least 32 positions, tiles begin at multiples of 32)
+#define CTA_ISSUE(TI)                                                                                    \
+    {                                                                                                    \
+        const int ti_ = (TI);                                                                            \
+        const int kt_ = kbeg + ti_ * 32;                                                                 \
+        int pg_ = -1;                                                                                    \
+        if (ti_ < nt) {                                                                                  \
+            if ((kt_ >> a.page_shift) - pages_base >= 64) {                                              \
+                pages_base = kt_ >> a.page_shift;                                                        \
+                const int pi = pages_base + lane;                                                        \
+                const bool in = ((long)pi << a.page_shift) < seq_len;                                    \
+                my_page = bt[in ? pi : 0];                                                               \
+                my_page = in ? my_page : -1;                                                             \
+            }                                                                                            \
+            pg_ = __builtin_amdgcn_readlane(my_page, __builtin_amdgcn_readfirstlane((kt_ >> a.page_shift) - pages_base)); \
+        }                                                                                                \
+        const size_t pb_ = (size_t)(pg_ < 0 ? 0 : pg_) * a.Hk + kvh;                                     \
+        const bf16_t* kb_ = kc + (pb_ * a.page_size + (kt_ & a.page_mask)) * HD;                         \
+        const bf16_t* vb_ = vc + pb_ * HD * a.page_size + (kt_ & a.page_mask);                           \
+        const uint32_t dst_ = lds_base + (uint32_t)(((ti_ % CTA_STAGES) * STAGE_CHUNKS + wave * 64) * 16); \
+        _Pragma("unroll") for (int i = 0; i < CTA_LOADS; ++i) {                                          \
+            const bool ok_ = pg_ >= 0 && kt_ + src_key[i] < seq_len;                                     \
+            const bf16_t* p_ = ok_ ? (src_is_k[i] ? kb_ : vb_) + src_off[i] : zero_src;                  \
+            lds_dma16(p_, __builtin_amdgcn_readfirstlane(dst_ + i * 256 * 16));                          \
+        }                                                                                                \
+    }
+
+    f32x16 o[DB];
 #pragma unroll
     for (int d = 0; d < DB; ++d)
 #pragma unroll
-        for (int e4 = 0; e4 < 4; ++e4) {
-            const int dd = d * 32 + e4 * 8 + lg * 4;
-            if (dd < HD)
-                *reinterpret_cast<float4*>(po + dd) = make_float4(o[d][e4 * 4 + 0] * inv, o[d][e4 * 4 + 1] * inv,
-                                                                  o[d][e4 * 4 + 2] * inv, o[d][e4 * 4 + 3] * inv);
-        }
-    if (lg == 0) {
-        float* pm = a.part_ml + (((size_t)slot * a.Hk + kvh) * ROWS + lr) * 2;
-        pm[0] = m;
-        pm[1] = l;
+        for (int e = 0; e < 16; ++e) o[d][e] = 0.f;
+    float m = -INFINITY, l = 0.f;      // m in units of log2
+    const float c2 = a.scale * 1.44269504088896340736f;
+    // what the rows of this wave can see: keys [lo_min, pos_max]; keys in [lo_max, pos_min] by all
+    int pos_min = row_ok ? pos : 0x7fffffff, lo_max = row_ok ? lo : 0;
+    int pos_max = row_ok ? pos : -1, lo_min = row_ok ? lo : 0x7fffffff;
+#pragma unroll
+    for (int o_ = 32; o_ > 0; o_ >>= 1) {
+        pos_min = min(pos_min, __shfl_xor(pos_min, o_, 64));
+        lo_max = max(lo_max, __shfl_xor(lo_max, o_, 64));
+        pos_max = max(pos_max, __shfl_xor(pos_max, o_, 64));
+        lo_min = min(lo_min, __shfl_xor(lo_min, o_, 64));
     }
+
+#pragma unroll
+    for (int st = 0; st < CTA_STAGES - 1; ++st) CTA_ISSUE(st)
+    for (int ti = 0; ti < nt; ++ti) {
+        // tile ti has landed when at most the CTA_STAGES-2 younger tiles are still on their way
+        wait_vmcnt<CTA_LOADS * (CTA_STAGES - 2)>();
+        __builtin_amdgcn_s_barrier();                    // for every wave; and tile ti-1 is no longer read
+        CTA_ISSUE(ti + CTA_STAGES - 1)                   // into the place of tile ti-1 (zeros past the end)
+        const int kt = kbeg + ti * 32;
+        if (kt > pos_max || kt + 32 <= lo_min) continue; // nothing here for this wave's rows
+        const uint4* Ks = lds + (ti % CTA_STAGES) * STAGE_CHUNKS;
+        const uint4* Vs = Ks + NKC;
+        uint4 kf[KD], vf[2][DB];
+#pragma unroll
+        for (int kd = 0; kd < KD; ++kd) {
+            const int c = 2 * kd + lg;
+            kf[kd] = Ks[key_off * KSTR + (CK_POW2 ? (c ^ (key_off & (CK - 1))) : c)];
+        }
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int d = 0; d < DB; ++d) vf[j][d] = Vs[(d * 32 + lr) * 4 + ((2 * j + lg) ^ ((lr >> 2) & 3))];
+        if (kt + 32 > seq_len) {               // the request's last tile: slots past its end hold old data
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                const int k8 = kt + 16 * j + 8 * lg;
+                uint32_t mk[4];
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                    mk[e] = (k8 + 2 * e < seq_len ? 0x0000FFFFu : 0u) | (k8 + 2 * e + 1 < seq_len ? 0xFFFF0000u : 0u);
+#pragma unroll
+                for (int d = 0; d < DB; ++d) {
+                    vf[j][d].x &= mk[0]; vf[j][d].y &= mk[1]; vf[j][d].z &= mk[2]; vf[j][d].w &= mk[3];
+                }
+            }
+        }
+        f32x16 s;
+#pragma unroll
+        for (int e = 0; e < 16; ++e) s[e] = 0.f;
+#pragma unroll
+        for (int kd = 0; kd < KD; ++kd)
+            s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16x8(kf[kd]), qf[kd], s, 0, 0, 0);
+        float p[16];
+        float corr;
+        ATTN_SOFTMAX_STEP(kt, kend)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            uint4 pk = make_uint4(pack2(p[8 * j + 0], p[8 * j + 1]), pack2(p[8 * j + 2], p[8 * j + 3]),
+                                  pack2(p[8 * j + 4], p[8 * j + 5]), pack2(p[8 * j + 6], p[8 * j + 7]));
+            const bf16x8 pf = as_bf16x8(pk);
+#pragma unroll
+            for (int d = 0; d < DB; ++d)
+                o[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16x8(vf[j][d]), pf, o[d], 0, 0, 0);
+        }
+    }
+#undef CTA_ISSUE
+    wait_vmcnt<0>();                                     // the trailing copies of zeros
+
+    ATTN_WRITE_OUT(slot)
 }
 
-// One merge job: {req, row0, first_slot, n_slots}.  Slot s holds the normalised output of
+// One merge job: {req, row0, first_slot, n_slots, slot_stride}.  Slot s holds the normalised output of
 // its keys with their maximum m_s (in units of log2) and sum l_s; the whole is
 // sum_s w_s O_s / sum_s w_s with w_s = l_s * 2^(m_s - max m).
 struct MergeArgs {
-    const int* jobs;        // [n_jobs, 4]
+    const int* jobs;        // [n_jobs, JOB_INTS]
     const int* cu_q;
     const float* part_o;
     const float* part_ml;
@@ -335,8 +536,8 @@ struct MergeArgs {
 };
 
 __global__ __launch_bounds__(256) void k_attn_merge(MergeArgs a) {
-    const int* job = a.jobs + (size_t)blockIdx.x * 4;
-    const int req = job[0], row0 = job[1], s0 = job[2], ns = job[3];
+    const int* job = a.jobs + (size_t)blockIdx.x * JOB_INTS;
+    const int req = job[0], row0 = job[1], s0 = job[2], ns = job[3], stride = job[4];
     const int kvh = blockIdx.y;
     const int G = a.H / a.Hk;
     const int q0 = a.cu_q[req], q_len = a.cu_q[req + 1] - q0;
@@ -347,7 +548,7 @@ __global__ __launch_bounds__(256) void k_attn_merge(MergeArgs a) {
         const int tok = rho / G, hg = rho - tok * G;
         const float* ml = a.part_ml + (((size_t)s0 * a.Hk + kvh) * ROWS + r) * 2;
         const float* po = a.part_o + (((size_t)s0 * a.Hk + kvh) * ROWS + r) * HD + d4;
-        const size_t ml_step = (size_t)a.Hk * ROWS * 2, po_step = (size_t)a.Hk * ROWS * HD;
+        const size_t ml_step = (size_t)stride * a.Hk * ROWS * 2, po_step = (size_t)stride * a.Hk * ROWS * HD;
         float mx = -INFINITY;
 #pragma unroll 4
         for (int s = 0; s < ns; ++s) mx = fmaxf(mx, ml[s * ml_step]);
@@ -370,7 +571,8 @@ __global__ __launch_bounds__(256) void k_attn_merge(MergeArgs a) {
 extern "C" int xr_attn_head_dim() { return HD; }
 
 extern "C" int xr_attention_mfma(void* out, const void* q, const void* k_cache, const void* v_cache,
-                                 const int* items, int n_items, const int* jobs, int n_jobs, const int* cu_q,
+                                 const int* items, int n_items, int n_cta_items, const int* jobs, int n_jobs,
+                                 const int* cu_q,
                                  const int* starts, const int* block_table, int table_stride, float* part_o,
                                  float* part_ml, int H, int Hk, int D, int page_size, float scale, int window,
                                  hipStream_t stream) {
@@ -379,17 +581,32 @@ extern "C" int xr_attention_mfma(void* out, const void* q, const void* k_cache, 
     int shift = ilog2_exact(page_size);
     XR_REQUIRE(shift >= 4, "attention: the MFMA kernel needs a page size that is a power of two of at least 16, got %d", page_size);
     XR_REQUIRE(window >= 0, "attention: window %d is negative", window);
-    XR_REQUIRE(n_items >= 0 && n_jobs >= 0, "attention: negative work counts");
+    XR_REQUIRE(n_items >= 0 && n_jobs >= 0 && n_cta_items >= 0, "attention: negative work counts");
+    XR_REQUIRE(n_cta_items == 0 || page_size >= 32, "attention: 128-row items need pages of at least 32 positions, got %d", page_size);
     XR_REQUIRE(n_jobs == 0 || (part_o && part_ml && jobs), "attention: split work without partial buffers");
-    if (n_items == 0) return XR_OK;
+    if (n_items + n_cta_items == 0) return XR_OK;
     AttnArgs a;
     a.q = (const bf16_t*)q; a.kc = (const bf16_t*)k_cache; a.vc = (const bf16_t*)v_cache; a.out = (bf16_t*)out;
-    a.items = items; a.cu_q = cu_q; a.starts = starts; a.block_table = block_table; a.table_stride = table_stride;
+    // the list begins with the items of the workgroup kernel
+    a.cta_items = items; a.n_cta_items = n_cta_items; a.items = items + (size_t)n_cta_items * ITEM_INTS; a.cu_q = cu_q; a.starts = starts; a.block_table = block_table; a.table_stride = table_stride;
     a.part_o = part_o; a.part_ml = part_ml; a.n_items = n_items; a.H = H; a.Hk = Hk;
     a.page_shift = shift; a.page_mask = page_size - 1; a.page_size = page_size; a.scale = scale; a.window = window;
-    dim3 grid((n_items + 3) / 4, Hk);
-    k_attn_mfma<<<grid, 256, 0, stream>>>(a);
-    XR_CHECK_LAUNCH("attention_mfma");
+    if (n_cta_items > 0) {
+        constexpr int smem = CTA_STAGES * STAGE_CHUNKS * 16;
+        static bool attr_set = false;
+        if (!attr_set) {
+            hipError_t e = hipFuncSetAttribute((const void*)k_attn_cta, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+            XR_REQUIRE(e == hipSuccess, "attention: %d bytes of LDS refused: %s", smem, hipGetErrorString(e));
+            attr_set = true;
+        }
+        k_attn_cta<<<dim3(n_cta_items, Hk), 256, smem, stream>>>(a);
+        XR_CHECK_LAUNCH("attention_cta");
+    }
+    if (n_items > 0) {
+        dim3 grid((n_items + 3) / 4, Hk);
+        k_attn_mfma<<<grid, 256, 0, stream>>>(a);
+        XR_CHECK_LAUNCH("attention_mfma");
+    }
     if (n_jobs > 0) {
         MergeArgs mg;
         mg.jobs = jobs; mg.cu_q = cu_q; mg.part_o = part_o; mg.part_ml = part_ml; mg.out = (bf16_t*)out;

@@ -16,6 +16,7 @@
 // The reference's float-weight "GEMM" is a multi-column matvec (/root/reference/src/kernels.cu:116-144);
 // its tensor-core kernels (:856) exist for quantised weights only.
 #include "common.h"
+#include "async_copy.h"
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
@@ -237,24 +238,6 @@ __global__ __launch_bounds__(64 * WARPS_M * WARPS_N) void k_gemm_tile(GemmArgs g
 // instructions spent on them.  A lane whose piece lies outside the matrices reads from a
 // block of zeros instead, so every slice issues the same number of loads and one counter
 // wait (vmcnt) tells when a slice has landed.
-__device__ uint4 xr_zero_chunk[4];      // zero-initialised
-
-template <int N> struct WaitVm {        // s_waitcnt vmcnt(N) only
-    static constexpr int imm = (N & 0xF) | ((N >> 4) << 14) | (0x7 << 4) | (0xF << 8);
-};
-
-// The copies are written as inline assembly: the compiler then does not count them, so it
-// neither makes every LDS read wait for all of them nor drains them at each barrier; the
-// kernel waits for exactly the slice it is about to use (s_waitcnt vmcnt) and meets the
-// other waves at a bare s_barrier.
-__device__ inline void lds_dma16(const void* src, uint32_t lds_byte_addr) {
-    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
-                 :: "v"(src), "s"(lds_byte_addr) : "memory");
-}
-template <int N> __device__ inline void wait_vmcnt() {
-    asm volatile("s_waitcnt vmcnt(%0)" :: "n"(N) : "memory");
-}
-
 template <int BM, int BN, int WARPS_M, int WARPS_N, int STAGES>
 __global__ __launch_bounds__(64 * WARPS_M * WARPS_N) void k_gemm_tile_async(GemmArgs g) {
     constexpr int WAVES = WARPS_M * WARPS_N;
@@ -437,7 +420,8 @@ static int launch_tile_async(GemmArgs g, hipStream_t stream) {
         attr_set = true;
     }
     int n_out_tile = g.epi == EPI_SWIGLU ? BN / 2 : BN;
-    unsigned tiles = (unsigned)(((g.N + n_out_tile - 1) / n_out_tile) * ((g.M + BM - 1) / BM));
+    unsigned tiles_n = (unsigned)((g.N + n_out_tile - 1) / n_out_tile), tiles_m = (unsigned)((g.M + BM - 1) / BM);
+    unsigned tiles = tiles_n * tiles_m;
     if (g.splits < 1 || !g.partial) g.splits = 1;
     if (g.splits > 1) {
         int slices = (g.K + 63) / 64;

@@ -277,15 +277,15 @@ class Ops:
         out = torch.empty((T, H * D), dtype=q.dtype, device=q.device)
         if self.use_mfma and q.dtype == torch.bfloat16 and D % 16 == 0 and 16 <= D <= 256 and page_size >= 16:
             lib = self.attention_lib(D)
-            plan = ctx.attention_plan(group, H // Hk, window, Hk)
+            plan = ctx.attention_plan(group, H // Hk, window, Hk, page_size)
             part_o = part_ml = None
             if plan.n_slots:
                 part_o = torch.empty((plan.n_slots, Hk, 32, D), dtype=torch.float32, device=q.device)
                 part_ml = torch.empty((plan.n_slots, Hk, 32, 2), dtype=torch.float32, device=q.device)
             lib.check(lib.xr_attention_mfma(
                 out.data_ptr(), q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), plan.items.data_ptr(),
-                plan.n_items, _ptr(plan.jobs), plan.n_jobs, ctx.cu_q.data_ptr(), ctx.starts_dev.data_ptr(),
-                block_table.data_ptr(), block_table.stride(0), _ptr(part_o), _ptr(part_ml), H, Hk, D, page_size,
+                plan.n_items, plan.n_cta_items, _ptr(plan.jobs), plan.n_jobs, ctx.cu_q.data_ptr(),
+                ctx.starts_dev.data_ptr(), block_table.data_ptr(), block_table.stride(0), _ptr(part_o), _ptr(part_ml), H, Hk, D, page_size,
                 float(scale), int(window or 0), _stream()))
             return out
         self.lib.check(self.lib.xr_attention_ref(
@@ -300,7 +300,7 @@ class Ops:
         if lib is None:
             unit = f"attn_d{D}"
             path = _build.find_built(unit) or _build.build_unit(unit)
-            lib = _Lib(path, {"xr_attention_mfma": [_p, _p, _p, _p, _p, _i, _p, _i, _p, _p, _p, _i, _p, _p,
+            lib = _Lib(path, {"xr_attention_mfma": [_p, _p, _p, _p, _p, _i, _i, _p, _i, _p, _p, _p, _i, _p, _p,
                                                     _i, _i, _i, _i, _f, _i, _p]})
             self._attn_libs[D] = lib
         return lib

@@ -24,20 +24,28 @@ import torch
 class AttentionPlan:
     """The work list of the MFMA attention kernel for one step, cache group, group size and window.
 
-    ``items [n, 8]`` int32 on the device: request, first row of a 32-row block, first key,
+    ``items [c + n, 8]`` int32 on the device: request, first row of a row block, first key,
     end key, partial slot (-1: the item covers all keys of its block and writes the output),
-    the request's first row in the step, its number of tokens, its first position.
-    ``jobs [m, 4]``: request, first row, first slot, number of slots to merge.
+    the request's first row in the step, its number of tokens, its first position.  The first
+    ``n_cta_items`` are blocks of 128 rows that a workgroup takes together (its wave w the rows
+    from ``row0 + 32 w``, with partial slot ``slot + w``), the other ``n_items`` blocks of 32
+    rows, one wave each.
+    ``jobs [m, 5]``: request, first row of 32, first slot, number of slots to merge and the
+    distance between them.
     """
     items: torch.Tensor
     n_items: int
     jobs: Optional[torch.Tensor]
     n_jobs: int
     n_slots: int
+    n_cta_items: int = 0
 
 
 ATTN_ROWS = 32          # query rows (token x head-in-group) per work item
 ATTN_TILE = 32          # keys per tile; items begin and end on tile edges
+ATTN_CTA_ROWS = 128     # rows of an item that a whole workgroup takes
+ATTN_CTA_MIN_ROWS = 64  # a request brings at least this many rows to be served by workgroups
+ATTN_CTA_SLOTS = 768    # parts of that kind wanted in a step before blocks are left whole (measured)
 
 
 def tiles_per_item(total_tiles: int, n_kv_heads: int) -> int:
@@ -56,32 +64,73 @@ def tiles_per_item(total_tiles: int, n_kv_heads: int) -> int:
 
 
 
-def plan_attention(starts, q_lens, group_size: int, window: Optional[int], n_kv_heads: int):
-    """Host side of ``AttentionPlan``: lists of items and merge jobs (plain Python ints)."""
-    blocks = []
+def plan_attention(starts, q_lens, group_size: int, window: Optional[int], n_kv_heads: int,
+                   page_size: int = 64, cta_tiles: Optional[int] = None):
+    """Host side of ``AttentionPlan``: ``(cta_items, items, jobs, n_slots)`` as plain Python ints.
+
+    ``cta_tiles`` fixes the most tiles a 128-row item may cover (for measurements); by
+    default it follows from how many such items the step has.
+    """
+    blocks, cta_blocks = [], []
     total_tiles = 0
     q0s, acc = [], 0
     for n in q_lens:
         q0s.append(acc)
         acc += n
+
+    def key_range(s, n, row0, rows):
+        tok_lo = row0 // group_size
+        tok_hi = min(n - 1, (row0 + rows - 1) // group_size)
+        lo = 0 if not window else max(0, s + tok_lo - window + 1)
+        lo = (lo // ATTN_TILE) * ATTN_TILE
+        hi = s + tok_hi + 1
+        return lo, hi, -(-(hi - lo) // ATTN_TILE)
+
     for b, (s, n) in enumerate(zip(starts, q_lens)):
         rows = n * group_size
+        if rows >= ATTN_CTA_MIN_ROWS and page_size >= ATTN_TILE:
+            for row0 in range(0, rows, ATTN_CTA_ROWS):
+                cta_blocks.append((b, row0) + key_range(s, n, row0, ATTN_CTA_ROWS))
+            continue
         for row0 in range(0, rows, ATTN_ROWS):
-            tok_lo = row0 // group_size
-            tok_hi = min(n - 1, (row0 + ATTN_ROWS - 1) // group_size)
-            lo = 0 if not window else max(0, s + tok_lo - window + 1)
-            lo = (lo // ATTN_TILE) * ATTN_TILE
-            hi = s + tok_hi + 1
-            tiles = -(-(hi - lo) // ATTN_TILE)
-            blocks.append((b, row0, lo, hi, tiles))
-            total_tiles += tiles
+            blk = (b, row0) + key_range(s, n, row0, ATTN_ROWS)
+            blocks.append(blk)
+            total_tiles += blk[4]
+    items, cta_items, jobs, slot = [], [], [], 0
+    # longest first: workgroups are started in list order, and a long item started last
+    # would run on alone at the end
+    cta_blocks.sort(key=lambda blk: -blk[4])
+    blocks.sort(key=lambda blk: -blk[4])
+
+    if cta_blocks:
+        chunk = cta_tiles
+        if chunk is None:
+            # As many parts as fill the chip once; the longest block decides the step's time
+            # otherwise (a prompt's last rows see all of it, its first rows nothing).
+            work = sum(blk[4] for blk in cta_blocks)
+            chunk = max(8, -(-work * n_kv_heads // ATTN_CTA_SLOTS))
+        for b, row0, lo, hi, tiles in cta_blocks:
+            parts = -(-tiles // chunk)
+            if parts <= 1:
+                cta_items.append((b, row0, lo, hi, -1, q0s[b], q_lens[b], starts[b]))
+                continue
+            per = -(-tiles // parts)
+            first = slot
+            k = lo
+            while k < hi:
+                e = min(hi, k + per * ATTN_TILE)
+                cta_items.append((b, row0, k, e, slot, q0s[b], q_lens[b], starts[b]))
+                slot += ATTN_CTA_ROWS // ATTN_ROWS
+                k = e
+            n_parts = (slot - first) // (ATTN_CTA_ROWS // ATTN_ROWS)
+            rows = q_lens[b] * group_size
+            for w in range(ATTN_CTA_ROWS // ATTN_ROWS):
+                if row0 + w * ATTN_ROWS < rows:
+                    jobs.append((b, row0 + w * ATTN_ROWS, first + w, n_parts, ATTN_CTA_ROWS // ATTN_ROWS))
+
     chunk = 1 << 30
     if blocks and len(blocks) * n_kv_heads < 2048:         # too few row blocks to fill the chip
         chunk = tiles_per_item(total_tiles, n_kv_heads)
-    items, jobs, slot = [], [], 0
-    # longest first: workgroups are started in list order, and a long item started last
-    # would run on alone at the end
-    blocks.sort(key=lambda blk: -blk[4])
     for b, row0, lo, hi, tiles in blocks:
         parts = -(-tiles // chunk)
         if parts <= 1:
@@ -95,8 +144,8 @@ def plan_attention(starts, q_lens, group_size: int, window: Optional[int], n_kv_
             items.append((b, row0, k, e, slot, q0s[b], q_lens[b], starts[b]))
             slot += 1
             k = e
-        jobs.append((b, row0, first, slot - first))
-    return items, jobs, slot
+        jobs.append((b, row0, first, slot - first, 1))
+    return cta_items, items, jobs, slot
 
 
 @dataclass
@@ -179,17 +228,20 @@ class StepContext:
         self.slots_host = [rc.slot for rc in request_caches]
         self._plans = {}
 
-    def attention_plan(self, group: int, group_size: int, window: Optional[int], n_kv_heads: int) -> AttentionPlan:
+    def attention_plan(self, group: int, group_size: int, window: Optional[int], n_kv_heads: int,
+                       page_size: int = 64) -> AttentionPlan:
         """The MFMA attention work list, made once per step and shared by all layers that can."""
-        key = (group_size, window, n_kv_heads)
+        key = (group_size, window, n_kv_heads, page_size)
         plan = self._plans.get(key)
         if plan is None:
-            items, jobs, n_slots = plan_attention(self.starts, self.q_lens, group_size, window, n_kv_heads)
-            flat = [v for it in items for v in it] + [v for j in jobs for v in j]
+            cta_items, items, jobs, n_slots = plan_attention(self.starts, self.q_lens, group_size, window,
+                                                             n_kv_heads, page_size)
+            flat = [v for it in cta_items + items for v in it] + [v for j in jobs for v in j]
             host = torch.tensor(flat, dtype=torch.int32).pin_memory()
             dev = host.to(self.device, non_blocking=True)
-            ni, nj = len(items), len(jobs)
-            plan = AttentionPlan(dev[:ni * 8], ni, dev[ni * 8:] if nj else None, nj, n_slots)
+            nc, ni, nj = len(cta_items), len(items), len(jobs)
+            nw = (nc + ni) * 8
+            plan = AttentionPlan(dev[:nw], ni, dev[nw:] if nj else None, nj, n_slots, nc)
             plan._host = host
             self._plans[key] = plan
         return plan

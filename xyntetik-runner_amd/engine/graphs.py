@@ -68,7 +68,7 @@ class StaticDecodeContext:
 
     def _alloc(self) -> None:
         B, S = self.B, self.S
-        n_plan = len(self._plan_keys) * (B * S * 8 + B * 4)
+        n_plan = len(self._plan_keys) * (B * S * 8 + B * 5)
         offs = np.concatenate([[0], np.cumsum(self._sizes)]).astype(np.int64)
         total = int(offs[-1]) + n_plan
         self._offs = offs
@@ -83,15 +83,16 @@ class StaticDecodeContext:
         for k in self._plan_keys:
             self._plan_off[k] = base
             items = d[base:base + B * S * 8]
-            jobs = d[base + B * S * 8:base + B * S * 8 + B * 4]
+            jobs = d[base + B * S * 8:base + B * S * 8 + B * 5]
             self._plans[k] = AttentionPlan(items, B * S, jobs if S > 1 else None, B if S > 1 else 0,
                                            B * S if S > 1 else 0)
-            base += B * S * 8 + B * 4
+            base += B * S * 8 + B * 5
 
     def block_table(self, group: int) -> torch.Tensor:
         return self._tables[group]
 
-    def attention_plan(self, group: int, group_size: int, window: Optional[int], n_kv_heads: int) -> AttentionPlan:
+    def attention_plan(self, group: int, group_size: int, window: Optional[int], n_kv_heads: int,
+                       page_size: int = 64) -> AttentionPlan:
         key = (group_size, window, n_kv_heads)
         if key not in self._plans:
             if torch.cuda.is_current_stream_capturing():
@@ -149,7 +150,7 @@ class StaticDecodeContext:
         group_size, window, _ = key
         B, S = self.B, self.S
         items = h[base:base + B * S * 8].reshape(B, S, 8)
-        jobs = h[base + B * S * 8:base + B * S * 8 + B * 4].reshape(B, 4)
+        jobs = h[base + B * S * 8:base + B * S * 8 + B * 5].reshape(B, 5)
         hi = starts.astype(np.int64) + 1                          # keys [lo, hi)
         lo = np.zeros(B, dtype=np.int64)
         if window:
@@ -175,6 +176,7 @@ class StaticDecodeContext:
         jobs[:, 1] = 0
         jobs[:, 2] = np.arange(B) * S
         jobs[:, 3] = S
+        jobs[:, 4] = 1
 
 
 class DecodeGraphs:
