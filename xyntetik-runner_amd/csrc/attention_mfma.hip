@@ -7,8 +7,11 @@
 // window bound :6326); the arrangement is not.  The query rows that share one key/value
 // head -- (token, head-in-group) pairs of one request -- are packed 32 to a block, so the
 // 4 heads of a decoded token, or 8 tokens x 4 heads of a prompt portion, read each key
-// and value once.  A wave takes one work item: a row block and a range of keys, listed
-// by the host.  For every tile of 32 keys it computes, transposed,
+// and value once.  The host lists the work: row blocks with a range of keys each.  Long
+// portions go to k_attn_cta (128 rows a workgroup, the tiles shared by its waves), all else
+// to k_attn_stream (32 rows a workgroup, the tiles dealt out to its waves); both bring
+// the tiles of K and V^T into LDS by asynchronous copies and have a wave compute, for every
+// tile of 32 keys, transposed,
 //     S^T[key, row] = K[key, :] . Q[row, :]        v_mfma_f32_32x32x16_bf16, A = K tile
 //     O^T[d, row]  += V^T[d, key] * P^T[key, row]  A = V^T tile (values are cached transposed)
 // so that a lane owns one query row throughout: row maxima and sums are sums over the
@@ -19,7 +22,9 @@
 // Scores, maxima, sums and the output accumulate in 32-bit; P is rounded to bfloat16
 // for the second product.  Items that cover part of a row block's keys write partial
 // results that k_attn_merge combines (/root/reference/src/kernels.cu:2171-2270 does this
-// with 8 fixed slices for decoding).
+// with 8 fixed slices for decoding).  Page sizes are powers of two from 16; a key that does
+// not exist (past the request's end, or in a page the window has given back) is copied from
+// a block of zeros, and the words of V^T past the end in the last tile are masked on use.
 #include "common.h"
 #include "async_copy.h"
 
@@ -151,185 +156,6 @@ _Pragma("unroll")                                                               
         pm[0] = m;                                                                                       \
         pm[1] = l;                                                                                       \
     }
-
-__global__ __launch_bounds__(256) void k_attn_mfma(AttnArgs a) {
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int item = blockIdx.x * 4 + wave;
-    if (item >= a.n_items) return;
-    const int kvh = blockIdx.y;
-    const int* it = a.items + (size_t)item * ITEM_INTS;
-    // everything about the item and its request comes with the item: no second lookup
-    const int req = it[0], row0 = it[1], kbeg = it[2], kend = it[3], slot = it[4];
-    const int q0 = it[5], q_len = it[6], start = it[7];
-    const int G = a.H / a.Hk;
-    const int lr = lane & 31, lg = lane >> 5;
-    const int seq_len = start + q_len;
-    const int* bt = a.block_table + (size_t)req * a.table_stride;
-
-    // this lane's query row
-    const int rho = row0 + lr;
-    const int tok = rho / G, hg = rho - tok * G;
-    const bool row_ok = tok < q_len;
-    const int t = q0 + tok, h = kvh * G + hg;
-    const int pos = start + tok;
-    const int lo = (a.window > 0 && pos - a.window + 1 > 0) ? pos - a.window + 1 : 0;
-
-    const uint4 zero = make_uint4(0, 0, 0, 0);
-    bf16x8 qf[KD];
-    {
-        const bf16_t* qp = a.q + ((size_t)(row_ok ? t : q0) * a.H + h) * HD + lg * 8;
-#pragma unroll
-        for (int kd = 0; kd < KD; ++kd) qf[kd] = as_bf16x8(keep_if(row_ok, ldg16(qp + kd * 16)));
-    }
-    // the key this lane's tile row stands for: r = 8a + 4g + b  ->  16(a/2) + 8g + 4(a%2) + b
-    const int ra = lr >> 3, rg = (lr >> 2) & 1, rb = lr & 3;
-    const int key_off = 16 * (ra >> 1) + 8 * rg + 4 * (ra & 1) + rb;
-
-    // Page numbers of the item's keys, one per lane, fetched once per 64 pages: inside the
-    // loop a page number comes from another lane's register, not from memory.
-    const bf16_t* __restrict__ kc = a.kc;
-    const bf16_t* __restrict__ vc = a.vc;
-    const int page0 = kbeg >> a.page_shift;
-    int pages_base = page0;
-    int my_page;
-    {
-        const int pi = page0 + lane;
-        const bool in = ((long)pi << a.page_shift) < seq_len;
-        my_page = bt[in ? pi : 0];
-        my_page = in ? my_page : -1;
-    }
-    // Loads are never predicated: a key that does not exist is read from the null page and
-    // its words are replaced by zeros, so whole 16-byte loads stay in flight.
-#define ATTN_LOAD_K(KT, KF)                                                                              \
-    {                                                                                                    \
-        const int key_ = (KT) + key_off;                                                                 \
-        const int pg_ = __shfl(my_page, ((key_ < seq_len ? key_ : (KT)) >> a.page_shift) - pages_base, 64); \
-        const bool ok_ = key_ < seq_len && pg_ >= 0;                                                     \
-        const bf16_t* kp_ = kc + (((size_t)(ok_ ? pg_ : 0) * a.Hk + kvh) * a.page_size + (key_ & a.page_mask)) * HD + lg * 8; \
-        _Pragma("unroll") for (int kd = 0; kd < KD; ++kd) KF[kd] = keep_if(ok_, ldg16(kp_ + kd * 16));   \
-    }
-#define ATTN_LOAD_V(KT, VF)                                                                              \
-    {                                                                                                    \
-        _Pragma("unroll") for (int j = 0; j < 2; ++j) {                                                  \
-            const int k8_ = (KT) + 16 * j + 8 * lg;                                                      \
-            const int pg_ = __shfl(my_page, ((k8_ < seq_len ? k8_ : (KT)) >> a.page_shift) - pages_base, 64); \
-            const bool ok_ = k8_ < seq_len && pg_ >= 0;                                                  \
-            _Pragma("unroll") for (int d = 0; d < DB; ++d) {                                             \
-                const int dd_ = d * 32 + lr;                                                             \
-                const bool okd_ = ok_ && dd_ < HD;                                                       \
-                VF[j][d] = keep_if(okd_, ldg16(vc + (((size_t)(okd_ ? pg_ : 0) * a.Hk + kvh) * HD + (okd_ ? dd_ : 0)) * a.page_size + (k8_ & a.page_mask))); \
-            }                                                                                            \
-        }                                                                                                \
-    }
-
-    // The same loads for a tile that lies wholly inside the request (every page exists): no
-    // select touches the loaded words, so nothing waits for them until the tile is used.
-#define ATTN_LOAD_K_FAST(KT, KF)                                                                         \
-    {                                                                                                    \
-        const int key_ = (KT) + key_off;                                                                 \
-        const int pg_ = __shfl(my_page, (key_ >> a.page_shift) - pages_base, 64);                        \
-        const bf16_t* kp_ = kc + (((size_t)pg_ * a.Hk + kvh) * a.page_size + (key_ & a.page_mask)) * HD + lg * 8; \
-        _Pragma("unroll") for (int kd = 0; kd < KD; ++kd) KF[kd] = ldg16(kp_ + kd * 16);                 \
-    }
-#define ATTN_LOAD_V_FAST(KT, VF)                                                                         \
-    {                                                                                                    \
-        _Pragma("unroll") for (int j = 0; j < 2; ++j) {                                                  \
-            const int k8_ = (KT) + 16 * j + 8 * lg;                                                      \
-            const int pg_ = __shfl(my_page, (k8_ >> a.page_shift) - pages_base, 64);                     \
-            const bf16_t* vp_ = vc + (((size_t)pg_ * a.Hk + kvh) * HD + lr) * a.page_size + (k8_ & a.page_mask); \
-            _Pragma("unroll") for (int d = 0; d < DB; ++d) {                                             \
-                if (HD % 32 == 0 || d * 32 + lr < HD) VF[j][d] = ldg16(vp_ + (size_t)d * 32 * a.page_size); \
-                else VF[j][d] = make_uint4(0, 0, 0, 0);                                                  \
-            }                                                                                            \
-        }                                                                                                \
-    }
-
-    f32x16 o[DB];
-#pragma unroll
-    for (int d = 0; d < DB; ++d)
-#pragma unroll
-        for (int e = 0; e < 16; ++e) o[d][e] = 0.f;
-    float m = -INFINITY, l = 0.f;      // m in units of log2
-    const float c2 = a.scale * 1.44269504088896340736f;
-    // a tile whose keys lie in [lo_max, pos_min] is visible to every row that exists
-    int pos_min = row_ok ? pos : 0x7fffffff, lo_max = row_ok ? lo : 0;
-#pragma unroll
-    for (int o_ = 32; o_ > 0; o_ >>= 1) {
-        pos_min = min(pos_min, __shfl_xor(pos_min, o_, 64));
-        lo_max = max(lo_max, __shfl_xor(lo_max, o_, 64));
-    }
-
-    // Loads run one tile ahead of their use.
-    uint4 kf[KD], vf[2][DB];
-    if (kbeg < kend) {
-        ATTN_LOAD_K(kbeg, kf)
-        ATTN_LOAD_V(kbeg, vf)
-    }
-    for (int kt = kbeg; kt < kend; kt += 32) {
-        uint4 kn[KD], vn[2][DB];
-        const int nx = kt + 32;
-        if (nx < kend) {
-            if (((nx >> a.page_shift) - pages_base) >= 64) {
-                pages_base = nx >> a.page_shift;
-                const int pi = pages_base + lane;
-                const bool in = ((long)pi << a.page_shift) < seq_len;
-                my_page = bt[in ? pi : 0];
-                my_page = in ? my_page : -1;
-            }
-            if (nx + 32 <= seq_len) {
-                ATTN_LOAD_K_FAST(nx, kn)
-                ATTN_LOAD_V_FAST(nx, vn)
-            } else {
-                ATTN_LOAD_K(nx, kn)
-                ATTN_LOAD_V(nx, vn)
-            }
-        }
-        if (kt + 32 > seq_len) {               // the request's last tile: slots past its end hold old data
-#pragma unroll
-            for (int j = 0; j < 2; ++j) {
-                const int k8 = kt + 16 * j + 8 * lg;
-                uint32_t mk[4];
-#pragma unroll
-                for (int e = 0; e < 4; ++e)
-                    mk[e] = (k8 + 2 * e < seq_len ? 0x0000FFFFu : 0u) | (k8 + 2 * e + 1 < seq_len ? 0xFFFF0000u : 0u);
-#pragma unroll
-                for (int d = 0; d < DB; ++d) {
-                    vf[j][d].x &= mk[0]; vf[j][d].y &= mk[1]; vf[j][d].z &= mk[2]; vf[j][d].w &= mk[3];
-                }
-            }
-        }
-        // ---- S^T = K Q^T
-        f32x16 s;
-#pragma unroll
-        for (int e = 0; e < 16; ++e) s[e] = 0.f;
-#pragma unroll
-        for (int kd = 0; kd < KD; ++kd)
-            s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16x8(kf[kd]), qf[kd], s, 0, 0, 0);
-        float p[16];
-        float corr;
-        ATTN_SOFTMAX_STEP(kt, kend)
-        // ---- O^T += V^T P^T
-#pragma unroll
-        for (int j = 0; j < 2; ++j) {
-            uint4 pk = make_uint4(pack2(p[8 * j + 0], p[8 * j + 1]), pack2(p[8 * j + 2], p[8 * j + 3]),
-                                  pack2(p[8 * j + 4], p[8 * j + 5]), pack2(p[8 * j + 6], p[8 * j + 7]));
-            const bf16x8 pf = as_bf16x8(pk);
-#pragma unroll
-            for (int d = 0; d < DB; ++d)
-                o[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16x8(vf[j][d]), pf, o[d], 0, 0, 0);
-        }
-        if (nx < kend) {
-#pragma unroll
-            for (int kd = 0; kd < KD; ++kd) kf[kd] = kn[kd];
-#pragma unroll
-            for (int j = 0; j < 2; ++j)
-#pragma unroll
-                for (int d = 0; d < DB; ++d) vf[j][d] = vn[j][d];
-        }
-    }
-
-    ATTN_WRITE_OUT(slot)
-}
 
 // ------------------------------------------------------------------------------ workgroup kernel
 // Long prompt portions: a workgroup of 4 waves takes 128 consecutive rows of one request and
@@ -523,6 +349,254 @@ __global__ __launch_bounds__(256, 2) void k_attn_cta(AttnArgs a) {
     ATTN_WRITE_OUT(slot)
 }
 
+// ------------------------------------------------------------------------------ streaming kernel
+// Decoded tokens and short portions: few rows, many keys, bound by how fast the keys and
+// values arrive.  A workgroup takes one item (a 32-row block and a range of keys); its waves
+// share the rows and take the item's tiles in turn, wave w the tiles w, w + STREAM_WAVES, ..
+// Every wave copies its own tiles into a ring of its own in LDS (whole key rows and runs of
+// 64 bytes of V^T per lane group, instead of 32 bytes from 32 places per load instruction)
+// and reads its fragments from there, so the main loop has no barrier at all.  At the end
+// the waves' results are combined through LDS and written as the output or as one partial.
+constexpr int STREAM_WAVES = HD <= 128 ? 4 : 2;
+constexpr int W_LOADS = (NKC + NVC + 63) / 64;              // copies per lane and tile
+constexpr int W_STAGE = W_LOADS * 64;                       // chunks of a wave's tile
+constexpr int STREAM_STAGES = W_STAGE * 16 * STREAM_WAVES * 3 <= 96 * 1024 ? 3 : 2;
+constexpr int MERGE_STRIDE = HD + 4;                        // floats between rows of the combining buffer
+constexpr int STREAM_RING_BYTES = STREAM_WAVES * STREAM_STAGES * W_STAGE * 16;
+constexpr int STREAM_MERGE_BYTES = STREAM_WAVES * ROWS * (MERGE_STRIDE + 2) * 4;
+constexpr int STREAM_LDS_BYTES = STREAM_RING_BYTES > STREAM_MERGE_BYTES ? STREAM_RING_BYTES : STREAM_MERGE_BYTES;
+static_assert(W_LOADS * (STREAM_STAGES - 1) < 64, "too many copies in flight for the counter");
+static_assert(STREAM_LDS_BYTES <= 160 * 1024, "the rings do not fit into LDS");
+
+__global__ __launch_bounds__(64 * STREAM_WAVES) void k_attn_stream(AttnArgs a) {
+    extern __shared__ uint4 lds[];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int kvh = blockIdx.y;
+    const int* it = a.items + (size_t)blockIdx.x * ITEM_INTS;
+    const int req = it[0], row0 = it[1], kbeg = it[2], kend = it[3], slot = it[4];
+    const int q0 = it[5], q_len = it[6], start = it[7];
+    const int G = a.H / a.Hk;
+    const int lr = lane & 31, lg = lane >> 5;
+    const int seq_len = start + q_len;
+    const int* bt = a.block_table + (size_t)req * a.table_stride;
+
+    const int rho = row0 + lr;
+    const int tok = rho / G, hg = rho - tok * G;
+    const bool row_ok = tok < q_len;
+    const int t = q0 + tok, h = kvh * G + hg;
+    const int pos = start + tok;
+    const int lo = (a.window > 0 && pos - a.window + 1 > 0) ? pos - a.window + 1 : 0;
+
+    bf16x8 qf[KD];
+    {
+        const bf16_t* qp = a.q + ((size_t)(row_ok ? t : q0) * a.H + h) * HD + lg * 8;
+#pragma unroll
+        for (int kd = 0; kd < KD; ++kd) qf[kd] = as_bf16x8(keep_if(row_ok, ldg16(qp + kd * 16)));
+    }
+    const int ra = lr >> 3, rg = (lr >> 2) & 1, rb = lr & 3;
+    const int key_off = 16 * (ra >> 1) + 8 * rg + 4 * (ra & 1) + rb;
+
+    // the pieces this lane copies for every tile: a key (K: its row, V^T: the first of 8) and
+    // an offset from that key's place in its page
+    int src_off[W_LOADS], src_key[W_LOADS];
+    bool src_is_k[W_LOADS];
+#pragma unroll
+    for (int i = 0; i < W_LOADS; ++i) {
+        const int q = i * 64 + lane;
+        src_is_k[i] = q < NKC;
+        if (q < NKC) {
+            const int r = q / KSTR, cs = q - r * KSTR;
+            const int c = CK_POW2 ? (cs ^ (r & (CK - 1))) : cs;
+            src_off[i] = c * 8;
+            src_key[i] = cs < CK ? r : (1 << 30);           // the spare chunk of a row stays zero
+        } else {
+            const int v = q - NKC, d = v >> 2, c = (v & 3) ^ ((d >> 2) & 3);
+            src_off[i] = d * a.page_size;
+            src_key[i] = (v < NVC && d < HD) ? c * 8 : (1 << 30);
+        }
+    }
+    const bf16_t* __restrict__ kc = a.kc;
+    const bf16_t* __restrict__ vc = a.vc;
+    const bf16_t* zero_src = reinterpret_cast<const bf16_t*>(xr_zero_chunk);
+    const uint32_t ring_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) void*)lds +
+                               (uint32_t)(wave * STREAM_STAGES * W_STAGE * 16);
+    const uint4* ring = lds + wave * STREAM_STAGES * W_STAGE;
+
+    int pages_base = kbeg >> a.page_shift;
+    int my_page;
+    {
+        const int pi = pages_base + lane;
+        const bool in = ((long)pi << a.page_shift) < seq_len;
+        my_page = bt[in ? pi : 0];
+        my_page = in ? my_page : -1;
+    }
+    const int nt = (kend - kbeg + 31) >> 5;
+    const int n_mine = nt > wave ? (nt - wave + STREAM_WAVES - 1) / STREAM_WAVES : 0;
+    // Copy of this wave's j-th tile (zeros past its last one).  With pages of 32 positions and
+    // more a tile lies in one page; with smaller ones every lane looks its own page up.
+#define STREAM_ISSUE(J)                                                                                  \
+    {                                                                                                    \
+        const int j_ = (J);                                                                              \
+        const int kt_ = kbeg + (wave + j_ * STREAM_WAVES) * 32;                                          \
+        const bool live_ = j_ < n_mine;                                                                  \
+        if (live_ && ((kt_ + 31) >> a.page_shift) - pages_base >= 64) {                                  \
+            pages_base = kt_ >> a.page_shift;                                                            \
+            const int pi = pages_base + lane;                                                            \
+            const bool in = ((long)pi << a.page_shift) < seq_len;                                        \
+            my_page = bt[in ? pi : 0];                                                                   \
+            my_page = in ? my_page : -1;                                                                 \
+        }                                                                                                \
+        const uint32_t dst_ = ring_base + (uint32_t)((j_ % STREAM_STAGES) * W_STAGE * 16);               \
+        if (a.page_size >= 32) {                                                                         \
+            int pg_ = -1;                                                                                \
+            if (live_) pg_ = __builtin_amdgcn_readlane(my_page, __builtin_amdgcn_readfirstlane((kt_ >> a.page_shift) - pages_base)); \
+            const size_t pb_ = (size_t)(pg_ < 0 ? 0 : pg_) * a.Hk + kvh;                                 \
+            const int ko_ = kt_ & a.page_mask;                                                           \
+            const bf16_t* kb_ = kc + (pb_ * a.page_size + ko_) * HD;                                     \
+            const bf16_t* vb_ = vc + pb_ * HD * a.page_size + ko_;                                       \
+            _Pragma("unroll") for (int i = 0; i < W_LOADS; ++i) {                                        \
+                const bool ok_ = pg_ >= 0 && kt_ + src_key[i] < seq_len;                                 \
+                const bf16_t* p_ = ok_ ? (src_is_k[i] ? kb_ + src_key[i] * HD : vb_ + src_key[i]) + src_off[i] : zero_src; \
+                lds_dma16(p_, __builtin_amdgcn_readfirstlane(dst_ + i * 64 * 16));                       \
+            }                                                                                            \
+        } else {                                                                                         \
+            _Pragma("unroll") for (int i = 0; i < W_LOADS; ++i) {                                        \
+                const int key_ = kt_ + src_key[i];                                                       \
+                const bool in_ = live_ && key_ < seq_len;                                                \
+                const int pg_ = __shfl(my_page, in_ ? (key_ >> a.page_shift) - pages_base : 0, 64);      \
+                const bool ok_ = in_ && pg_ >= 0;                                                        \
+                const size_t pb_ = (size_t)(ok_ ? pg_ : 0) * a.Hk + kvh;                                 \
+                const int ko_ = key_ & a.page_mask;                                                      \
+                const bf16_t* p_ = src_is_k[i] ? kc + (pb_ * a.page_size + ko_) * HD + src_off[i]        \
+                                               : vc + pb_ * HD * a.page_size + src_off[i] + ko_;         \
+                lds_dma16(ok_ ? p_ : zero_src, __builtin_amdgcn_readfirstlane(dst_ + i * 64 * 16));      \
+            }                                                                                            \
+        }                                                                                                \
+    }
+
+    f32x16 o[DB];
+#pragma unroll
+    for (int d = 0; d < DB; ++d)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) o[d][e] = 0.f;
+    float m = -INFINITY, l = 0.f;      // m in units of log2
+    const float c2 = a.scale * 1.44269504088896340736f;
+    int pos_min = row_ok ? pos : 0x7fffffff, lo_max = row_ok ? lo : 0;
+#pragma unroll
+    for (int o_ = 32; o_ > 0; o_ >>= 1) {
+        pos_min = min(pos_min, __shfl_xor(pos_min, o_, 64));
+        lo_max = max(lo_max, __shfl_xor(lo_max, o_, 64));
+    }
+
+#pragma unroll
+    for (int st = 0; st < STREAM_STAGES - 1; ++st) STREAM_ISSUE(st)
+    for (int j = 0; j < n_mine; ++j) {
+        wait_vmcnt<W_LOADS * (STREAM_STAGES - 2)>();     // tile j is there
+        STREAM_ISSUE(j + STREAM_STAGES - 1)              // into the place of tile j-1, whose fragments are in registers
+        const int kt = kbeg + (wave + j * STREAM_WAVES) * 32;
+        const uint4* Ks = ring + (j % STREAM_STAGES) * W_STAGE;
+        const uint4* Vs = Ks + NKC;
+        uint4 kf[KD], vf[2][DB];
+#pragma unroll
+        for (int kd = 0; kd < KD; ++kd) {
+            const int c = 2 * kd + lg;
+            kf[kd] = Ks[key_off * KSTR + (CK_POW2 ? (c ^ (key_off & (CK - 1))) : c)];
+        }
+#pragma unroll
+        for (int jj = 0; jj < 2; ++jj)
+#pragma unroll
+            for (int d = 0; d < DB; ++d) vf[jj][d] = Vs[(d * 32 + lr) * 4 + ((2 * jj + lg) ^ ((lr >> 2) & 3))];
+        if (kt + 32 > seq_len) {               // the request's last tile: slots past its end hold old data
+#pragma unroll
+            for (int jj = 0; jj < 2; ++jj) {
+                const int k8 = kt + 16 * jj + 8 * lg;
+                uint32_t mk[4];
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                    mk[e] = (k8 + 2 * e < seq_len ? 0x0000FFFFu : 0u) | (k8 + 2 * e + 1 < seq_len ? 0xFFFF0000u : 0u);
+#pragma unroll
+                for (int d = 0; d < DB; ++d) {
+                    vf[jj][d].x &= mk[0]; vf[jj][d].y &= mk[1]; vf[jj][d].z &= mk[2]; vf[jj][d].w &= mk[3];
+                }
+            }
+        }
+        f32x16 s;
+#pragma unroll
+        for (int e = 0; e < 16; ++e) s[e] = 0.f;
+#pragma unroll
+        for (int kd = 0; kd < KD; ++kd)
+            s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16x8(kf[kd]), qf[kd], s, 0, 0, 0);
+        float p[16];
+        float corr;
+        ATTN_SOFTMAX_STEP(kt, kend)
+#pragma unroll
+        for (int jj = 0; jj < 2; ++jj) {
+            uint4 pk = make_uint4(pack2(p[8 * jj + 0], p[8 * jj + 1]), pack2(p[8 * jj + 2], p[8 * jj + 3]),
+                                  pack2(p[8 * jj + 4], p[8 * jj + 5]), pack2(p[8 * jj + 6], p[8 * jj + 7]));
+            const bf16x8 pf = as_bf16x8(pk);
+#pragma unroll
+            for (int d = 0; d < DB; ++d)
+                o[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16x8(vf[jj][d]), pf, o[d], 0, 0, 0);
+        }
+    }
+#undef STREAM_ISSUE
+    wait_vmcnt<0>();                                     // the trailing copies of zeros
+    __syncthreads();                                     // the rings are free
+
+    // ---- combine the waves: sum_w 2^(m_w - max) O_w over sum_w 2^(m_w - max) l_w
+    float* mo = reinterpret_cast<float*>(lds);           // [waves][ROWS][MERGE_STRIDE] unnormalised outputs
+    float* mml = mo + STREAM_WAVES * ROWS * MERGE_STRIDE; // [waves][ROWS][2]
+    if (row_ok) {
+        float* dst = mo + (wave * ROWS + lr) * MERGE_STRIDE;
+#pragma unroll
+        for (int d = 0; d < DB; ++d)
+#pragma unroll
+            for (int e4 = 0; e4 < 4; ++e4) {
+                const int dd = d * 32 + e4 * 8 + lg * 4;
+                if (dd < HD)
+                    *reinterpret_cast<float4*>(dst + dd) = make_float4(o[d][e4 * 4 + 0], o[d][e4 * 4 + 1],
+                                                                       o[d][e4 * 4 + 2], o[d][e4 * 4 + 3]);
+            }
+        if (lg == 0) {
+            mml[(wave * ROWS + lr) * 2] = m;
+            mml[(wave * ROWS + lr) * 2 + 1] = l;
+        }
+    }
+    __syncthreads();
+    const int rows_left = q_len * G - row0;
+    const int n_rows = rows_left < ROWS ? rows_left : ROWS;
+    for (int idx = tid; idx < n_rows * (HD / 4); idx += 64 * STREAM_WAVES) {
+        const int r = idx / (HD / 4), d4 = (idx - r * (HD / 4)) * 4;
+        float mx = -INFINITY;
+#pragma unroll
+        for (int w = 0; w < STREAM_WAVES; ++w) mx = fmaxf(mx, mml[(w * ROWS + r) * 2]);
+        float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+        float lsum = 0.f;
+#pragma unroll
+        for (int w = 0; w < STREAM_WAVES; ++w) {
+            const float mw = mml[(w * ROWS + r) * 2], lw = mml[(w * ROWS + r) * 2 + 1];
+            const float f = lw > 0.f ? __builtin_amdgcn_exp2f(mw - mx) : 0.f;
+            const float4 v = *reinterpret_cast<const float4*>(mo + (w * ROWS + r) * MERGE_STRIDE + d4);
+            acc.x += f * v.x; acc.y += f * v.y; acc.z += f * v.z; acc.w += f * v.w;
+            lsum += f * lw;
+        }
+        const float inv = lsum > 0.f ? 1.0f / lsum : 0.f;
+        const int rr = row0 + r, tk = rr / G, hh = kvh * G + (rr - tk * G);
+        if (slot < 0) {
+            bf16_t* op = a.out + ((size_t)(q0 + tk) * a.H + hh) * HD + d4;
+            *reinterpret_cast<uint2*>(op) = make_uint2(pack2(acc.x * inv, acc.y * inv), pack2(acc.z * inv, acc.w * inv));
+        } else {
+            float* po = a.part_o + (((size_t)slot * a.Hk + kvh) * ROWS + r) * HD + d4;
+            *reinterpret_cast<float4*>(po) = make_float4(acc.x * inv, acc.y * inv, acc.z * inv, acc.w * inv);
+            if (d4 == 0) {
+                float* pm = a.part_ml + (((size_t)slot * a.Hk + kvh) * ROWS + r) * 2;
+                pm[0] = mx;
+                pm[1] = lsum;
+            }
+        }
+    }
+}
+
 // One merge job: {req, row0, first_slot, n_slots, slot_stride}.  Slot s holds the normalised output of
 // its keys with their maximum m_s (in units of log2) and sum l_s; the whole is
 // sum_s w_s O_s / sum_s w_s with w_s = l_s * 2^(m_s - max m).
@@ -603,9 +677,15 @@ extern "C" int xr_attention_mfma(void* out, const void* q, const void* k_cache, 
         XR_CHECK_LAUNCH("attention_cta");
     }
     if (n_items > 0) {
-        dim3 grid((n_items + 3) / 4, Hk);
-        k_attn_mfma<<<grid, 256, 0, stream>>>(a);
-        XR_CHECK_LAUNCH("attention_mfma");
+        static bool attr_set = false;
+        if (!attr_set) {
+            hipError_t e = hipFuncSetAttribute((const void*)k_attn_stream, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                               STREAM_LDS_BYTES);
+            XR_REQUIRE(e == hipSuccess, "attention: %d bytes of LDS refused: %s", STREAM_LDS_BYTES, hipGetErrorString(e));
+            attr_set = true;
+        }
+        k_attn_stream<<<dim3(n_items, Hk), 64 * STREAM_WAVES, STREAM_LDS_BYTES, stream>>>(a);
+        XR_CHECK_LAUNCH("attention_stream");
     }
     if (n_jobs > 0) {
         MergeArgs mg;

@@ -45,23 +45,20 @@ ATTN_ROWS = 32          # query rows (token x head-in-group) per work item
 ATTN_TILE = 32          # keys per tile; items begin and end on tile edges
 ATTN_CTA_ROWS = 128     # rows of an item that a whole workgroup takes
 ATTN_CTA_MIN_ROWS = 64  # a request brings at least this many rows to be served by workgroups
+ATTN_STREAM_SLOTS = 256 # workgroups of the streaming kernel that run at a time (one a compute unit)
+ATTN_MIN_RANGE = 4      # tiles: the shortest key range worth a workgroup
 ATTN_CTA_SLOTS = 768    # parts of that kind wanted in a step before blocks are left whole (measured)
 
 
-def tiles_per_item(total_tiles: int, n_kv_heads: int) -> int:
-    """How many 32-key tiles one work item should cover.
+def key_ranges(tiles: int, share: float) -> int:
+    """Into how many key ranges a 32-row block of ``tiles`` tiles is cut, given its share of
+    the workgroups that run at a time.
 
-    Short items pay their start-up (query load, page numbers, partial results) too often,
-    long ones leave compute units idle; the best length measured on MI355X grows with the
-    square root of the step's work (2-4 tiles for one decoding request at 2k context, 8 for
-    eight, 16 for sixty-four).
+    Measured on MI355X (batch 1-64, 2k and 8k context): the streaming kernel is fastest with
+    one round of workgroups and ranges as long as that allows; a range under 4 tiles costs more
+    to start and to merge than to run.
     """
-    want = (max(1, total_tiles) * n_kv_heads / 64.0) ** 0.5
-    t = 2
-    while t * 2 <= want and t < 32:
-        t *= 2
-    return t
-
+    return max(1, min(int(share), tiles // ATTN_MIN_RANGE))
 
 
 def plan_attention(starts, q_lens, group_size: int, window: Optional[int], n_kv_heads: int,
@@ -128,11 +125,9 @@ def plan_attention(starts, q_lens, group_size: int, window: Optional[int], n_kv_
                 if row0 + w * ATTN_ROWS < rows:
                     jobs.append((b, row0 + w * ATTN_ROWS, first + w, n_parts, ATTN_CTA_ROWS // ATTN_ROWS))
 
-    chunk = 1 << 30
-    if blocks and len(blocks) * n_kv_heads < 2048:         # too few row blocks to fill the chip
-        chunk = tiles_per_item(total_tiles, n_kv_heads)
+    budget = max(1, ATTN_STREAM_SLOTS // n_kv_heads)       # items that run at a time
     for b, row0, lo, hi, tiles in blocks:
-        parts = -(-tiles // chunk)
+        parts = 1 if len(blocks) >= budget else key_ranges(tiles, budget * tiles / total_tiles)
         if parts <= 1:
             items.append((b, row0, lo, hi, -1, q0s[b], q_lens[b], starts[b]))
             continue

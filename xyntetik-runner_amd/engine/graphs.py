@@ -21,7 +21,7 @@ import numpy as np
 import torch
 
 from ..cache import NULL_PAGE
-from .batch import ATTN_TILE, AttentionPlan, StepEntry, tiles_per_item
+from .batch import ATTN_MIN_RANGE, ATTN_STREAM_SLOTS, ATTN_TILE, AttentionPlan, StepEntry
 
 BUCKETS = (1, 2, 4, 8, 16, 32, 64, 128, 256, 512)
 SPLITS = (1, 2, 4, 8, 16, 32)
@@ -35,8 +35,8 @@ def bucket_for(n: int) -> Optional[int]:
 
 
 def splits_for(batch_cap: int, max_tiles: int, n_kv_heads: int) -> int:
-    """Key ranges per request, so that a range has about ``tiles_per_item`` tiles."""
-    want = max(1, round(max_tiles / tiles_per_item(batch_cap * max_tiles, n_kv_heads)))
+    """Key ranges per request: one round of workgroups, and no range shorter than it pays."""
+    want = max(1, min(ATTN_STREAM_SLOTS // (batch_cap * n_kv_heads), max_tiles // ATTN_MIN_RANGE))
     best = 1
     for s in SPLITS:
         if s <= want:
