@@ -1,15 +1,15 @@
 // bfloat16 matrix products on the gfx950 matrix cores, 32-bit accumulation:
 //   out[M,N] = a[M,K] * w[N,K]^T (+ bias)        (weights [n_out][n_in], row-major)
 // Two kernels share the epilogues:
-//   * k_gemm_tile:   large M (prompt portions).  A workgroup computes a BM x BN tile; both
-//     operands are staged through LDS in 64-wide K slices (16-byte chunks, XOR-swizzled
-//     so that fragment reads do not collide), double-buffered, and fed to
-//     v_mfma_f32_32x32x16_bf16.
-//   * k_gemm_skinny: M <= 64 (decoding).  The product is bound by reading the weights
+//   * k_gemm_tile_async: more than 16 rows (prompt portions, large batches).  A workgroup
+//     computes a BM x BN tile; both operands are copied from memory straight into LDS in
+//     64-wide K slices (16-byte chunks, XOR-swizzled so that fragment reads do not collide),
+//     several slices ahead, and fed to v_mfma_f32_32x32x16_bf16.  With few tiles K is split
+//     over workgroups and k_gemm_finish adds the parts in a fixed order.
+//   * k_gemm_skinny: M <= 16 (decoding).  The product is bound by reading the weights
 //     once, so each wave streams 16 weight rows straight from memory into MFMA fragments
 //     (v_mfma_f32_16x16x32_bf16, weights as the A operand, tokens as the B operand) with
-//     many loads in flight, the few activation rows come through LDS, and the waves of a
-//     workgroup split K among themselves.
+//     many loads in flight, and the waves of a workgroup split K among themselves.
 // Epilogues: store (float or bfloat16), add into a float output (the residual stream),
 // and SwiGLU: with w = [gate rows; up rows] the kernel writes silu(gate) * up, so the
 // [M, 2F] intermediate never reaches memory (/root/reference/src/model.c:6399-6404).
@@ -86,167 +86,32 @@ __device__ inline int w_row_of(int r, int bx, int N, int epi, int& out_col) {
     return (t & 1) ? N + out_col : out_col;
 }
 
-template <int BM, int BN, int WARPS_M, int WARPS_N>
-__global__ __launch_bounds__(64 * WARPS_M * WARPS_N) void k_gemm_tile(GemmArgs g) {
-    constexpr int THREADS = 64 * WARPS_M * WARPS_N;
-    constexpr int BK = 64, CH = BK / 8;                 // 8 chunks of 16 bytes per row
-    constexpr int WM = BM / WARPS_M, WN = BN / WARPS_N;
-    constexpr int TM = WM / 32, TN = WN / 32;
-    constexpr int A_CHUNKS = BM * CH / THREADS, W_CHUNKS = BN * CH / THREADS;
-    static_assert(BM * CH % THREADS == 0 && BN * CH % THREADS == 0, "tile does not divide among threads");
-    extern __shared__ uint4 lds[];                      // [2][(BM + BN) * CH]
-    constexpr int BUF = (BM + BN) * CH;                 // chunks per buffer; weights follow activations
-
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int wm0 = (wave / WARPS_N) * WM, wn0 = (wave % WARPS_N) * WN;
-    const int m0 = blockIdx.y * BM;
-    const int bx = blockIdx.x;
-    const int n_rows = g.epi == EPI_SWIGLU ? 2 * g.N : g.N;
-
-    // Which chunks this thread stages.  Loads are never predicated: a chunk outside the
-    // matrix is read from a row and column that exist and then replaced by zeros, so the
-    // compiler keeps whole 16-byte global loads in flight.
-    int a_row[A_CHUNKS], a_c[A_CHUNKS];
-    size_t a_off[A_CHUNKS];
-    bool a_ok[A_CHUNKS];
-#pragma unroll
-    for (int i = 0; i < A_CHUNKS; ++i) {
-        int q = tid + i * THREADS;
-        a_row[i] = q / CH; a_c[i] = q % CH;
-        int m = m0 + a_row[i];
-        a_ok[i] = m < g.M;
-        a_off[i] = (size_t)(a_ok[i] ? m : 0) * g.lda + a_c[i] * 8;
-    }
-    int w_row[W_CHUNKS], w_c[W_CHUNKS];
-    size_t w_off[W_CHUNKS];
-    bool w_ok[W_CHUNKS];
-#pragma unroll
-    for (int i = 0; i < W_CHUNKS; ++i) {
-        int q = tid + i * THREADS;
-        w_row[i] = q / CH; w_c[i] = q % CH;
-        int oc;
-        int n = w_row_of<BN, WN>(w_row[i], bx, g.N, g.epi, oc);
-        w_ok[i] = oc < g.N && n < n_rows;
-        w_off[i] = (size_t)(w_ok[i] ? n : 0) * g.K + w_c[i] * 8;
-    }
-    const bf16_t* __restrict__ gA = g.a;
-    const bf16_t* __restrict__ gW = g.w;
-
-    f32x16 acc[TM][TN];
-#pragma unroll
-    for (int i = 0; i < TM; ++i)
-#pragma unroll
-        for (int j = 0; j < TN; ++j)
-#pragma unroll
-            for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
-
-    uint4 ra[A_CHUNKS], rw[W_CHUNKS];
-    const uint4 zero = make_uint4(0, 0, 0, 0);
-#define TILE_LOAD_GLOBAL(K0)                                                                     \
-    {                                                                                            \
-        _Pragma("unroll") for (int i = 0; i < A_CHUNKS; ++i) {                                   \
-            const bool in_k = (K0) + a_c[i] * 8 < g.K;                                           \
-            const uint4 v = ldg16(gA + a_off[i] + (in_k ? (K0) : 0));                            \
-            ra[i] = keep_if(a_ok[i] && in_k, v);                                                 \
-        }                                                                                        \
-        _Pragma("unroll") for (int i = 0; i < W_CHUNKS; ++i) {                                   \
-            const bool in_k = (K0) + w_c[i] * 8 < g.K;                                           \
-            const uint4 v = ldg16(gW + w_off[i] + (in_k ? (K0) : 0));                            \
-            rw[i] = keep_if(w_ok[i] && in_k, v);                                                 \
-        }                                                                                        \
-    }
-#define TILE_STORE_LDS(BUFI)                                                                     \
-    {                                                                                            \
-        _Pragma("unroll") for (int i = 0; i < A_CHUNKS; ++i)                                     \
-            lds[(BUFI) * BUF + a_row[i] * CH + (a_c[i] ^ (a_row[i] & 7))] = ra[i];               \
-        _Pragma("unroll") for (int i = 0; i < W_CHUNKS; ++i)                                     \
-            lds[(BUFI) * BUF + BM * CH + w_row[i] * CH + (w_c[i] ^ (w_row[i] & 7))] = rw[i];     \
-    }
-
-    const int nk = (g.K + BK - 1) / BK;
-    TILE_LOAD_GLOBAL(0)
-    TILE_STORE_LDS(0)
-    __syncthreads();
-    const int lr = lane & 31, lg = lane >> 5;
-    for (int kt = 0; kt < nk; ++kt) {
-        const int buf = kt & 1;
-        if (kt + 1 < nk) TILE_LOAD_GLOBAL((kt + 1) * BK)
-#pragma unroll
-        for (int ks = 0; ks < BK / 16; ++ks) {
-            bf16x8 af[TM], wf[TN];
-            const int c = ks * 2 + lg;
-#pragma unroll
-            for (int i = 0; i < TM; ++i) {
-                int r = wm0 + i * 32 + lr;
-                af[i] = as_bf16x8(lds[buf * BUF + r * CH + (c ^ (r & 7))]);
-            }
-#pragma unroll
-            for (int j = 0; j < TN; ++j) {
-                int r = wn0 + j * 32 + lr;
-                wf[j] = as_bf16x8(lds[buf * BUF + BM * CH + r * CH + (c ^ (r & 7))]);
-            }
-#pragma unroll
-            for (int i = 0; i < TM; ++i)
-#pragma unroll
-                for (int j = 0; j < TN; ++j)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[i], wf[j], acc[i][j], 0, 0, 0);
-        }
-        if (kt + 1 < nk) TILE_STORE_LDS(buf ^ 1)
-        __syncthreads();
-    }
-#undef TILE_LOAD_GLOBAL
-#undef TILE_STORE_LDS
-
-    // epilogue: lane holds column (lane % 32), rows (e/4)*8 + (lane/32)*4 + e%4 of each 32x32 tile
-    if (g.epi == EPI_SWIGLU) {
-#pragma unroll
-        for (int i = 0; i < TM; ++i)
-#pragma unroll
-            for (int j = 0; j + 1 < TN; j += 2) {
-                int oc;
-                w_row_of<BN, WN>(wn0 + j * 32 + lr, bx, g.N, g.epi, oc);
-                if (oc >= g.N) continue;
-                float bg = g.bias ? g.bias[oc] : 0.f, bu = g.bias ? g.bias[g.N + oc] : 0.f;
-#pragma unroll
-                for (int e = 0; e < 16; ++e) {
-                    int m = m0 + wm0 + i * 32 + (e / 4) * 8 + lg * 4 + (e % 4);
-                    if (m < g.M) store_out(g, m, oc, silu_f(acc[i][j][e] + bg) * (acc[i][j + 1][e] + bu));
-                }
-            }
-        return;
-    }
-#pragma unroll
-    for (int i = 0; i < TM; ++i)
-#pragma unroll
-        for (int j = 0; j < TN; ++j) {
-            int n = bx * BN + wn0 + j * 32 + lr;
-            if (n >= g.N) continue;
-            float b = g.bias ? g.bias[n] : 0.f;
-#pragma unroll
-            for (int e = 0; e < 16; ++e) {
-                int m = m0 + wm0 + i * 32 + (e / 4) * 8 + lg * 4 + (e % 4);
-                if (m < g.M) store_out(g, m, n, acc[i][j][e] + b);
-            }
-        }
-}
-
-// ------------------------------------------------------------------------------ tile kernel, asynchronous
-// The same tiling with the operands copied from memory straight into LDS
+// WARPS_M x WARPS_N waves share a BM x BN tile; a wave owns (BM/WARPS_M) x (BN/WARPS_N) of it
+// as 32x32 MFMA tiles.  The operands are copied from memory straight into LDS
 // (global_load_lds_dwordx4: every lane names a 16-byte source, the wave's 64 pieces land
-// side by side in LDS) and STAGES K-slices in flight: while the matrix cores work on slice
+// side by side in LDS) with STAGES K-slices in flight: while the matrix cores work on slice
 // kt, slices kt+1 .. kt+STAGES-1 are on their way, with no registers and no LDS-write
 // instructions spent on them.  A lane whose piece lies outside the matrices reads from a
 // block of zeros instead, so every slice issues the same number of loads and one counter
-// wait (vmcnt) tells when a slice has landed.
+// wait (vmcnt) tells when a slice has landed.  Measured on MI355X: what bounds the kernel is
+// the rate at which a compute unit's L1 delivers the slices (about 20 bytes a cycle), so
+// the tile with the most products per byte that still fills the chip is chosen.
+// Where chunk c of row r lies within the row in LDS: at c ^ swz(r).  A fragment read takes
+// one column of 32 rows; LDS serves 16 lanes of 16 bytes a cycle from 64 banks of 4 bytes, so
+// 16 consecutive rows must fall into 16 different 16-byte bank groups.  Two rows of 128 bytes
+// (8 chunks) fill the banks, so the shift counts pairs of rows.  (The counter of LDS bank
+// conflicts reads zero with this, and half the active cycles with a shift by the row number.)
+template <int CH> __device__ inline int swz(int r) { static_assert(CH == 8, "rows of 8 chunks"); return (r >> 1) & 7; }
+
 template <int BM, int BN, int WARPS_M, int WARPS_N, int STAGES>
 __global__ __launch_bounds__(64 * WARPS_M * WARPS_N) void k_gemm_tile_async(GemmArgs g) {
     constexpr int WAVES = WARPS_M * WARPS_N;
-    constexpr int BK = 64, CH = BK / 8;
+    constexpr int BK = 64, CH = BK / 8, RPL = 64 / CH;  // chunks of a row; rows that one load instruction covers
     constexpr int WM = BM / WARPS_M, WN = BN / WARPS_N;
     constexpr int TM = WM / 32, TN = WN / 32;
     constexpr int ROWS = BM + BN;                       // rows of one stage: activations, then weights
-    constexpr int LOADS = ROWS / 8 / WAVES;             // load instructions per wave and stage (8 rows each)
-    static_assert(ROWS % (8 * WAVES) == 0, "stage does not divide among waves");
+    constexpr int LOADS = ROWS / RPL / WAVES;           // load instructions per wave and stage
+    static_assert(ROWS % (RPL * WAVES) == 0, "stage does not divide among waves");
     static_assert(LOADS * (STAGES - 2) < 64, "too many loads in flight for the counter");
     constexpr int BUF = ROWS * CH;                      // chunks per stage
     extern __shared__ uint4 lds[];                      // [STAGES][BUF]
@@ -272,9 +137,9 @@ __global__ __launch_bounds__(64 * WARPS_M * WARPS_N) void k_gemm_tile_async(Gemm
     int src_c[LOADS];
 #pragma unroll
     for (int i = 0; i < LOADS; ++i) {
-        const int row = (i * WAVES + wave) * 8 + (lane >> 3);     // row of the stage
-        const int slot = lane & 7;
-        const int c = slot ^ (row & 7);                           // the chunk that belongs in this LDS place
+        const int row = (i * WAVES + wave) * RPL + lane / CH;     // row of the stage
+        const int slot = lane % CH;
+        const int c = slot ^ swz<CH>(row);                        // the chunk that belongs in this LDS place
         src_c[i] = c * 8;
         if (row < BM) {
             const int m = m0 + row;
@@ -286,15 +151,18 @@ __global__ __launch_bounds__(64 * WARPS_M * WARPS_N) void k_gemm_tile_async(Gemm
         }
     }
     const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) void*)lds;
-#define ASYNC_ISSUE(KT)                                                                              \
+// the copies PART, PART + PARTS, .. of slice KT: spread over the k-steps of the slice before, so
+// that no wave has to push a whole slice into the memory pipeline at once
+#define ASYNC_ISSUE_PART(KT, PART, PARTS)                                                            \
     {                                                                                                \
         const int k0_ = k_begin + (KT) * BK;                                                         \
         const uint32_t dst_ = lds_base + (uint32_t)((((KT) % STAGES) * BUF + wave * 64) * 16);       \
-        _Pragma("unroll") for (int i = 0; i < LOADS; ++i) {                                          \
+        _Pragma("unroll") for (int i = (PART); i < LOADS; i += (PARTS)) {                            \
             const bf16_t* p_ = (src[i] && k0_ + src_c[i] < k_end) ? src[i] + k0_ : zero_src;         \
             lds_dma16(p_, __builtin_amdgcn_readfirstlane(dst_ + i * WAVES * 64 * 16));               \
         }                                                                                            \
     }
+#define ASYNC_ISSUE(KT) ASYNC_ISSUE_PART(KT, 0, 1)
 
     f32x16 acc[TM][TN];
 #pragma unroll
@@ -312,31 +180,47 @@ __global__ __launch_bounds__(64 * WARPS_M * WARPS_N) void k_gemm_tile_async(Gemm
         // slice kt has landed when at most the STAGES-2 younger slices are still in flight
         wait_vmcnt<LOADS * (STAGES - 2)>();
         __builtin_amdgcn_s_barrier();                    // for every wave; and slice kt-1 is no longer read
-        ASYNC_ISSUE(kt + STAGES - 1)                     // into the buffer slice kt-1 used (zeros past the end)
         const uint4* A = lds + (kt % STAGES) * BUF;
         const uint4* W = A + BM * CH;
+        // fragments of k-step ks+1 are read from LDS while the matrix cores work on k-step ks
+        bf16x8 af[2][TM], wf[2][TN];
+#define READ_FRAGS(KS, B)                                                                            \
+    {                                                                                                \
+        const int c_ = (KS) * 2 + lg;                                                                \
+        _Pragma("unroll") for (int i = 0; i < TM; ++i) {                                             \
+            const int r = wm0 + i * 32 + lr;                                                         \
+            af[B][i] = as_bf16x8(A[r * CH + (c_ ^ swz<CH>(r))]);                                        \
+        }                                                                                            \
+        _Pragma("unroll") for (int j = 0; j < TN; ++j) {                                             \
+            const int r = wn0 + j * 32 + lr;                                                         \
+            wf[B][j] = as_bf16x8(W[r * CH + (c_ ^ swz<CH>(r))]);                                        \
+        }                                                                                            \
+    }
+        READ_FRAGS(0, 0)
 #pragma unroll
         for (int ks = 0; ks < BK / 16; ++ks) {
-            bf16x8 af[TM], wf[TN];
-            const int c = ks * 2 + lg;
-#pragma unroll
-            for (int i = 0; i < TM; ++i) {
-                const int r = wm0 + i * 32 + lr;
-                af[i] = as_bf16x8(A[r * CH + (c ^ (r & 7))]);
-            }
-#pragma unroll
-            for (int j = 0; j < TN; ++j) {
-                const int r = wn0 + j * 32 + lr;
-                wf[j] = as_bf16x8(W[r * CH + (c ^ (r & 7))]);
-            }
+            // a quarter of the copies of slice kt+STAGES-1, into the buffer that slice kt-1 used
+            // (zeros past the end)
+            ASYNC_ISSUE_PART(kt + STAGES - 1, ks, BK / 16)
+            if (ks + 1 < BK / 16) READ_FRAGS(ks + 1, (ks + 1) & 1)
 #pragma unroll
             for (int i = 0; i < TM; ++i)
 #pragma unroll
                 for (int j = 0; j < TN; ++j)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[i], wf[j], acc[i][j], 0, 0, 0);
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[ks & 1][i], wf[ks & 1][j], acc[i][j], 0, 0, 0);
+            // the order wanted of the scheduler: a fragment read, then its share of the products
+            if (ks + 1 < BK / 16) {
+#pragma unroll
+                for (int r = 0; r < TM + TN; ++r) {
+                    __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+                    __builtin_amdgcn_sched_group_barrier(0x008, (TM * TN) / (TM + TN) > 0 ? (TM * TN) / (TM + TN) : 1, 0);
+                }
+            }
         }
+#undef READ_FRAGS
     }
 #undef ASYNC_ISSUE
+#undef ASYNC_ISSUE_PART
     wait_vmcnt<0>();                                     // the trailing loads of zeros
 
     if (g.splits > 1) {
@@ -569,25 +453,9 @@ static int launch_skinny(const GemmArgs& g, hipStream_t stream) {
     return XR_OK;
 }
 
-template <int BM, int BN, int WM_, int WN_>
-static int launch_tile(const GemmArgs& g, hipStream_t stream) {
-    size_t smem = (size_t)2 * (BM + BN) * 8 * 16;
-    static bool attr_set = false;
-    if (!attr_set) {
-        hipError_t e = hipFuncSetAttribute((const void*)k_gemm_tile<BM, BN, WM_, WN_>,
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
-        if (e != hipSuccess) { xr_set_error("gemm: cannot reserve %zu bytes of LDS: %s", smem, hipGetErrorString(e)); return XR_LAUNCH; }
-        attr_set = true;
-    }
-    int n_out_tile = g.epi == EPI_SWIGLU ? BN / 2 : BN;
-    dim3 grid((g.N + n_out_tile - 1) / n_out_tile, (g.M + BM - 1) / BM);
-    k_gemm_tile<BM, BN, WM_, WN_><<<grid, 64 * WM_ * WN_, smem, stream>>>(g);
-    XR_CHECK_LAUNCH("gemm_tile");
-    return XR_OK;
-}
-
 // epi: 0 store, 1 add into float out, 2 SwiGLU (w has 2N rows: gate rows then up rows).
-// variant: 0 = choose by M; 1 = skinny; 2 = tile 128x128; 3 = tile 256x128.
+// variant: 0 = choose by shape; 1 = skinny; 10..20 = tile shapes; 30, 31 = few rows with K split;
+//          +1000 = row tiles of one weight tile follow each other.
 // workspace (may be null): room for split products, workspace_bytes long; without it K is not split.
 extern "C" int xr_gemm_bf16(void* out, const void* a, const void* w, const float* bias, int M, int N, int K,
                             int lda, int ldo, int out_dtype, int epi, int variant, float* workspace,
@@ -653,13 +521,6 @@ extern "C" int xr_gemm_bf16(void* out, const void* a, const void* w, const float
     SK(148, 4, 4, 4, 4, false) SK(149, 4, 4, 8, 2, false)
 #undef SK
 #endif
-    if (variant == 2) return launch_tile<128, 128, 2, 2>(g, stream);
-    if (variant == 3) return launch_tile<256, 128, 4, 2>(g, stream);
-    if (variant == 4) return launch_tile<256, 128, 2, 2>(g, stream);
-    if (variant == 5) return launch_tile<256, 256, 2, 2>(g, stream);
-    if (variant == 6) return launch_tile<128, 256, 2, 2>(g, stream);
-    if (variant == 7) return launch_tile<256, 256, 2, 4>(g, stream);
-    if (variant == 8) return launch_tile<256, 256, 4, 2>(g, stream);
     if (variant == 10) return launch_tile_async<128, 128, 2, 2, 3>(g, stream);
     if (variant == 11) return launch_tile_async<128, 128, 2, 2, 4>(g, stream);
     if (variant == 12) return launch_tile_async<256, 128, 4, 2, 3>(g, stream);
