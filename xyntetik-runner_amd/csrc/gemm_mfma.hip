@@ -182,42 +182,29 @@ __global__ __launch_bounds__(64 * WARPS_M * WARPS_N) void k_gemm_tile_async(Gemm
         __builtin_amdgcn_s_barrier();                    // for every wave; and slice kt-1 is no longer read
         const uint4* A = lds + (kt % STAGES) * BUF;
         const uint4* W = A + BM * CH;
-        // fragments of k-step ks+1 are read from LDS while the matrix cores work on k-step ks
-        bf16x8 af[2][TM], wf[2][TN];
-#define READ_FRAGS(KS, B)                                                                            \
-    {                                                                                                \
-        const int c_ = (KS) * 2 + lg;                                                                \
-        _Pragma("unroll") for (int i = 0; i < TM; ++i) {                                             \
-            const int r = wm0 + i * 32 + lr;                                                         \
-            af[B][i] = as_bf16x8(A[r * CH + (c_ ^ swz<CH>(r))]);                                        \
-        }                                                                                            \
-        _Pragma("unroll") for (int j = 0; j < TN; ++j) {                                             \
-            const int r = wn0 + j * 32 + lr;                                                         \
-            wf[B][j] = as_bf16x8(W[r * CH + (c_ ^ swz<CH>(r))]);                                        \
-        }                                                                                            \
-    }
-        READ_FRAGS(0, 0)
 #pragma unroll
         for (int ks = 0; ks < BK / 16; ++ks) {
             // a quarter of the copies of slice kt+STAGES-1, into the buffer that slice kt-1 used
             // (zeros past the end)
             ASYNC_ISSUE_PART(kt + STAGES - 1, ks, BK / 16)
-            if (ks + 1 < BK / 16) READ_FRAGS(ks + 1, (ks + 1) & 1)
+            bf16x8 af[TM], wf[TN];
+            const int c = ks * 2 + lg;
+#pragma unroll
+            for (int i = 0; i < TM; ++i) {
+                const int r = wm0 + i * 32 + lr;
+                af[i] = as_bf16x8(A[r * CH + (c ^ swz<CH>(r))]);
+            }
+#pragma unroll
+            for (int j = 0; j < TN; ++j) {
+                const int r = wn0 + j * 32 + lr;
+                wf[j] = as_bf16x8(W[r * CH + (c ^ swz<CH>(r))]);
+            }
 #pragma unroll
             for (int i = 0; i < TM; ++i)
 #pragma unroll
                 for (int j = 0; j < TN; ++j)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[ks & 1][i], wf[ks & 1][j], acc[i][j], 0, 0, 0);
-            // the order wanted of the scheduler: a fragment read, then its share of the products
-            if (ks + 1 < BK / 16) {
-#pragma unroll
-                for (int r = 0; r < TM + TN; ++r) {
-                    __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-                    __builtin_amdgcn_sched_group_barrier(0x008, (TM * TN) / (TM + TN) > 0 ? (TM * TN) / (TM + TN) : 1, 0);
-                }
-            }
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[i], wf[j], acc[i][j], 0, 0, 0);
         }
-#undef READ_FRAGS
     }
 #undef ASYNC_ISSUE
 #undef ASYNC_ISSUE_PART
