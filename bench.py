@@ -82,7 +82,9 @@ def measure_decode(runner, cfg, batch, prompt_len, steps, warmup, seed):
     eng = Engine(runner, max_batched_tokens=max(2048, prompt_len), max_running=batch,
                  max_model_len=cfg["max_position_embeddings"], stop_ids=[])
     rng = np.random.default_rng(seed)
-    sp = SamplingParams(temperature=0.0, max_new_tokens=warmup + steps + 8, ignore_eos=True)
+    # a request admitted first decodes while the others' prompts are still computed (up to
+    # `batch` steps): nobody may finish before the last timed step
+    sp = SamplingParams(temperature=0.0, max_new_tokens=batch + warmup + steps + 8, ignore_eos=True)
     ids = [eng.add_request([int(t) for t in rng.integers(0, cfg["vocab_size"], size=prompt_len)], sp) for _ in range(batch)]
     while any(eng.requests[i].n_computed < prompt_len for i in ids):
         eng.step()
@@ -95,7 +97,11 @@ def measure_decode(runner, cfg, batch, prompt_len, steps, warmup, seed):
         eng.step()
     torch.cuda.synchronize()
     dt = time.perf_counter() - t0
+    if len(eng.scheduler.running) != batch or any(i not in eng.requests for i in ids):
+        raise RuntimeError(f"decode batch {batch}: a request ended or waited during the timed steps")
     ctx1 = sum(eng.requests[i].n_tokens for i in ids)
+    if ctx1 - ctx0 != batch * steps:
+        raise RuntimeError(f"decode batch {batch}: {ctx1 - ctx0} tokens decoded in {steps} steps")
     for i in ids:
         eng.scheduler.abort(eng.requests.pop(i))
     if runner.graphs is not None:
@@ -141,7 +147,7 @@ def main():
     layers = args.layers or layers_full
     cfg["num_hidden_layers"] = layers
     P, B = args.prompt_len, args.batch
-    span = P + args.warmup + args.steps + 80
+    span = P + args.warmup + args.steps + 80 + max(64, B)
     spec, runner = build_runner(cfg, args.dtype, max_tokens=max(64, B) * (-(-span // 64) * 64) + 4096, max_requests=64)
 
     pre_s = measure_prefill(runner, cfg, 2048, repeats=3, seed=1)

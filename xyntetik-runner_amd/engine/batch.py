@@ -47,7 +47,7 @@ ATTN_CTA_ROWS = 128     # rows of an item that a whole workgroup takes
 ATTN_CTA_MIN_ROWS = 64  # a request brings at least this many rows to be served by workgroups
 ATTN_STREAM_SLOTS = 256 # workgroups of the streaming kernel that run at a time (one a compute unit)
 ATTN_MIN_RANGE = 4      # tiles: the shortest key range worth a workgroup
-ATTN_CTA_SLOTS = 768    # parts of that kind wanted in a step before blocks are left whole (measured)
+ATTN_CTA_FILL = 256     # 128-row items (times key/value heads) that give every compute unit one
 
 
 def key_ranges(tiles: int, share: float) -> int:
@@ -102,10 +102,15 @@ def plan_attention(starts, q_lens, group_size: int, window: Optional[int], n_kv_
     if cta_blocks:
         chunk = cta_tiles
         if chunk is None:
-            # As many parts as fill the chip once; the longest block decides the step's time
-            # otherwise (a prompt's last rows see all of it, its first rows nothing).
-            work = sum(blk[4] for blk in cta_blocks)
-            chunk = max(8, -(-work * n_kv_heads // ATTN_CTA_SLOTS))
+            # Whole blocks when there is one for every compute unit: the merge of split blocks
+            # costs more than the idle end of a step whose last rows see the most keys
+            # (2048 tokens, 8 key/value heads: 102 us whole, 96 us + 19 us of merging split).
+            # Fewer blocks are cut into about as many parts as fill the chip once.
+            if len(cta_blocks) * n_kv_heads >= ATTN_CTA_FILL:
+                chunk = 1 << 30
+            else:
+                work = sum(blk[4] for blk in cta_blocks)
+                chunk = max(8, -(-work * n_kv_heads // (2 * ATTN_CTA_FILL)))
         for b, row0, lo, hi, tiles in cta_blocks:
             parts = -(-tiles // chunk)
             if parts <= 1:
