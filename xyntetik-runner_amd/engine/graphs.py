@@ -187,7 +187,8 @@ class DecodeGraphs:
         self.graphs: Dict[Tuple[int, int, int], Tuple[StaticDecodeContext, torch.cuda.CUDAGraph, torch.Tensor]] = {}
         self.pool = None
         kv, st, _ = runner.model.cache_needs()
-        self.usable = not any(s is not None for s in st)          # state slots are served eagerly
+        # state slots are served eagerly, and so are parts that look at their data on the host
+        self.usable = not any(s is not None for s in st) and runner.model.capturable()
         self.kv_heads = max((k.num_kv_heads for k in kv if k is not None), default=1)
         self.replays = 0
         self.captures = 0

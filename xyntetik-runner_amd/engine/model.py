@@ -40,6 +40,10 @@ class Model:
         yield self.spec.final_norm.prefix, self.final_norm
         yield self.spec.head.prefix, self.head
 
+    def capturable(self) -> bool:
+        """Whether a step's launches are the same for any data (every part says so)."""
+        return all(part.capturable for _, part in self._named_parts())
+
     def expected(self) -> Dict[str, ParamSpec]:
         out: Dict[str, ParamSpec] = {}
         for prefix, part in self._named_parts():

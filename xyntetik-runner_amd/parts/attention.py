@@ -64,6 +64,10 @@ class PagedAttention(Mixer):
             specs[f"{o}.bias"] = ParamSpec((E,), role="vector", init="normal")
         return specs
 
+    @property
+    def capturable(self) -> bool:
+        return self.position is None or self.position.capturable
+
     def bind(self, tensors, rt) -> None:
         self.rt = rt
         q, k, v, o = self.names

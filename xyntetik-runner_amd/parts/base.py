@@ -68,6 +68,10 @@ class StateSpec:
 class Part:
     """Common base: parameters by relative name."""
 
+    #: False if ``forward`` reads device data on the host (which kernels it launches then
+    #: depends on the data): steps of a model with such a part are never recorded as HIP graphs.
+    capturable = True
+
     def param_specs(self) -> Dict[str, ParamSpec]:
         return {}
 
