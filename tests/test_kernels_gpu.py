@@ -104,6 +104,56 @@ def test_linear_bf16_mfma(ops, M, N, K):
                        a.double() @ w.double().T + b.double()) < 1e-5
 
 
+@pytest.mark.parametrize("M", [1, 8, 16, 17, 64, 65, 300])
+@pytest.mark.parametrize("N,K", [(48, 64), (100, 72), (333, 264), (1000, 1032), (16, 8)])
+def test_linear_packed_weights_give_the_same(ops, M, N, K):
+    """Weights in the kernels' own order (1 KB blocks, zero padding) against the same weights
+    row-major: the same sums in the same order, so the same bits; and against float64."""
+    from xyntetik_runner_amd.csrc.ops import PackedWeight
+    a = (torch.randn(M, K, device=DEV) * 0.5).bfloat16()
+    w = (torch.randn(N, K, device=DEV) * 0.1).bfloat16()
+    b = torch.randn(N, device=DEV) * 0.1
+    pw = ops.pack_weight(w)
+    assert isinstance(pw, PackedWeight) and pw.shape == (N, K)
+    blocks = pw.data.cpu()
+    n, k = 16 * (N // 16) + min(N % 16, 3) - (1 if N % 16 == 0 else 0), 8 * (K // 8 - 1)   # some row and chunk that exist
+    assert torch.equal(blocks[n // 16, k // 32, (k % 32) // 8, n % 16], w[n, k:k + 8].cpu())
+    if N % 16:
+        assert (blocks[-1, :, :, N % 16:] == 0).all()                   # rows that do not exist
+    if K % 32:
+        assert (blocks[:, -1, (K % 32) // 8:] == 0).all()               # nor columns
+    want = a.double() @ w.double().T + b.double()
+    got = ops.linear(a, pw, bias=b, out_dtype=torch.float32)
+    assert rel(got, want) < 1e-5
+    assert torch.equal(got, ops.linear(a, w, bias=b, out_dtype=torch.float32))
+    base = torch.randn(M, N, device=DEV)
+    o1, o2 = base.clone(), base.clone()
+    ops.linear(a, pw, out=o1, accumulate=True)
+    ops.linear(a, w, out=o2, accumulate=True)
+    assert torch.equal(o1, o2) and rel(o1, base.double() + a.double() @ w.double().T) < 1e-5
+    F = 16 * max(1, N // 16)                                            # gate and up rows: heights in steps of 16
+    w2 = (torch.randn(2 * F, K, device=DEV) * 0.1).bfloat16()
+    b2 = torch.randn(2 * F, device=DEV) * 0.1
+    pw2 = ops.pack_weight(w2, gated=True)
+    assert isinstance(pw2, PackedWeight)
+    r = a.double() @ w2.double().T + b2.double()
+    got = ops.linear_swiglu(a, pw2, bias=b2)
+    assert rel(got, r[:, :F] / (1 + torch.exp(-r[:, :F])) * r[:, F:]) < 6e-3
+    assert torch.equal(got, ops.linear_swiglu(a, w2, bias=b2))
+
+
+def test_pack_weight_leaves_what_the_mfma_kernels_do_not_take(ops):
+    w = torch.randn(40, 20, device=DEV).bfloat16()                      # width no multiple of 8
+    assert ops.pack_weight(w) is w
+    w = torch.randn(40, 24, device=DEV)                                 # 32-bit
+    assert ops.pack_weight(w) is w
+    w = torch.randn(2 * 24, 16, device=DEV).bfloat16()                  # gate and up rows of 24: not in steps of 16
+    assert ops.pack_weight(w, gated=True) is w and not isinstance(ops.pack_weight(w), torch.Tensor)
+    from xyntetik_runner_amd.csrc.ops import KernelError
+    with pytest.raises(KernelError):                                    # a packed weight has no 32-bit kernel to fall back to
+        ops.linear(torch.randn(3, 16, device=DEV), ops.pack_weight(w))
+
+
 @pytest.mark.parametrize("M,N,K", [(1, 7, 5), (9, 100, 77), (70, 65, 130)])
 @pytest.mark.parametrize("dt", ["float32", "bfloat16"])
 def test_linear_plain_kernel(ops, M, N, K, dt):

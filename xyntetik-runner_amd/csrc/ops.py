@@ -42,7 +42,8 @@ _PROTOS = {
     "xr_fill_rows": [_p, _p, _i, _sz, _u32, _p],
     "xr_convert": [_p, _p, _sz, _i, _i, _p],
     "xr_gemm_ref": [_p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _p],
-    "xr_gemm_bf16": [_p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _p, _sz, _p],
+    "xr_gemm_bf16": [_p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _i, _p, _sz, _p],
+    "xr_pack_weight": [_p, _p, _i, _i, _p],
     "xr_attention_ref": [_p, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _f, _i, _i, _p],
     "xr_sample": [_p, _p, _i, _i, _i, _p, _p, _p, _p, _p, _p, _p, _p, _i, _p, _i, _p],
 }
@@ -54,6 +55,28 @@ def _ptr(t: Optional[torch.Tensor]) -> Optional[int]:
 
 def _stream() -> int:
     return torch.cuda.current_stream().cuda_stream
+
+
+class PackedWeight:
+    """A bfloat16 weight matrix ``[rows, cols]`` in the order the MFMA kernels read it: blocks of
+    16 rows x 32 columns, 1 KB each (``data[row group, column block, chunk, row, 8 columns]``),
+    rows and columns padded with zeros.  Made by
+    ``Ops.pack_weight``; ``Ops.linear`` and ``Ops.linear_swiglu`` take it in place of the matrix."""
+
+    def __init__(self, data: torch.Tensor, rows: int, cols: int):
+        self.data, self.rows, self.cols = data, rows, cols
+
+    @property
+    def shape(self):
+        return (self.rows, self.cols)
+
+    @property
+    def dtype(self):
+        return self.data.dtype
+
+    @property
+    def device(self):
+        return self.data.device
 
 
 class _Lib:
@@ -175,22 +198,40 @@ class Ops:
         return (self.use_mfma and a.dtype == torch.bfloat16 and a.shape[1] % 8 == 0 and a.stride(0) % 8 == 0
                 and a.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0)
 
-    def linear(self, a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None,
+    def pack_weight(self, w: torch.Tensor, gated: bool = False):
+        """``w`` for use as the weight of ``linear`` (``gated``: of ``linear_swiglu``): packed for
+        the MFMA kernels where they will serve it (bfloat16, a width that is a multiple of 8, for
+        gate and up rows a height that is a multiple of 32), else ``w`` itself."""
+        if not (self.use_mfma and w.dtype == torch.bfloat16 and w.dim() == 2 and w.shape[1] % 8 == 0):
+            return w
+        N, K = w.shape
+        if gated and N % 32:
+            return w
+        self._dev(w)
+        self._contig(w, "pack_weight input")
+        data = torch.empty((-(-N // 16), -(-K // 32), 4, 16, 8), dtype=torch.bfloat16, device=w.device)
+        self.lib.check(self.lib.xr_pack_weight(data.data_ptr(), w.data_ptr(), N, K, _stream()))
+        return PackedWeight(data, N, K)
+
+    def linear(self, a: torch.Tensor, w, bias: Optional[torch.Tensor] = None,
                out_dtype: Optional[torch.dtype] = None, out: Optional[torch.Tensor] = None,
                accumulate: bool = False, variant: int = 0) -> torch.Tensor:
         """``a [M, K] @ w [N, K]^T (+ bias)``; with ``accumulate`` added into 32-bit ``out``.
 
         bfloat16 operands run on the matrix cores (32-bit accumulation); float32 operands, and
-        shapes the MFMA kernels do not take, run the plain 32-bit FMA kernel.
+        shapes the MFMA kernels do not take, run the plain 32-bit FMA kernel.  ``w`` is a matrix
+        or a ``PackedWeight``.
         """
-        self._dev(a, w, bias, out)
-        if a.dim() != 2 or w.dim() != 2 or a.shape[1] != w.shape[1]:
+        packed = isinstance(w, PackedWeight)
+        wt = w.data if packed else w
+        self._dev(a, wt, bias, out)
+        if a.dim() != 2 or len(w.shape) != 2 or a.shape[1] != w.shape[1]:
             raise KernelError(f"linear: shapes {tuple(a.shape)} x {tuple(w.shape)}^T do not fit")
         if a.dtype != w.dtype:
             raise KernelError(f"linear: input is {a.dtype}, weight is {w.dtype}")
         if a.stride(1) != 1:
             raise KernelError("linear: input must have unit column stride")
-        self._contig(w, "linear weight")
+        self._contig(wt, "linear weight")
         M, K = a.shape
         N = w.shape[0]
         if out is None:
@@ -201,36 +242,43 @@ class Ops:
             raise KernelError(f"linear: output is {tuple(out.shape)}, product is {(M, N)}")
         if bias is not None and (bias.dtype != torch.float32 or bias.numel() != N):
             raise KernelError("linear: bias must be float32 [N]")
-        if self._mfma_ok(a, w):
-            self.lib.check(self.lib.xr_gemm_bf16(out.data_ptr(), a.data_ptr(), w.data_ptr(), _ptr(bias), M, N, K,
+        if self._mfma_ok(a, wt):
+            self.lib.check(self.lib.xr_gemm_bf16(out.data_ptr(), a.data_ptr(), wt.data_ptr(), _ptr(bias), M, N, K,
                                                  a.stride(0), out.stride(0), dtype_code(out.dtype),
-                                                 1 if accumulate else 0, variant, *self._gemm_workspace(a.device),
-                                                 _stream()))
+                                                 1 if accumulate else 0, variant, 1 if packed else 0,
+                                                 *self._gemm_workspace(a.device), _stream()))
             return out
+        if packed:
+            raise KernelError("linear: a packed weight needs bfloat16 rows that are 16-byte aligned")
         self.lib.check(self.lib.xr_gemm_ref(out.data_ptr(), a.data_ptr(), w.data_ptr(), _ptr(bias), M, N, K,
                                             a.stride(0), out.stride(0), dtype_code(a.dtype),
                                             dtype_code(out.dtype), 1 if accumulate else 0, _stream()))
         return out
 
-    def linear_swiglu(self, a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None,
+    def linear_swiglu(self, a: torch.Tensor, w, bias: Optional[torch.Tensor] = None,
                       variant: int = 0) -> torch.Tensor:
-        """``silu(a @ w[:F]^T) * (a @ w[F:]^T)`` for ``w [2F, K]`` = gate rows then up rows."""
+        """``silu(a @ w[:F]^T) * (a @ w[F:]^T)`` for ``w [2F, K]`` = gate rows then up rows
+        (a matrix, or a ``PackedWeight`` made with ``gated=True``)."""
+        packed = isinstance(w, PackedWeight)
+        wt = w.data if packed else w
         F = w.shape[0] // 2
         if w.shape[0] % 2:
             raise KernelError("linear_swiglu: the weight must have an even number of rows")
-        if self._mfma_ok(a, w):
-            self._dev(a, w, bias)
-            self._contig(w, "linear_swiglu weight")
+        if self._mfma_ok(a, wt):
+            self._dev(a, wt, bias)
+            self._contig(wt, "linear_swiglu weight")
             M, K = a.shape
             if K != w.shape[1] or a.stride(1) != 1:
                 raise KernelError(f"linear_swiglu: shapes {tuple(a.shape)} x {tuple(w.shape)}^T do not fit")
             if bias is not None and (bias.dtype != torch.float32 or bias.numel() != 2 * F):
                 raise KernelError("linear_swiglu: bias must be float32 [2F]")
             out = torch.empty((M, F), dtype=a.dtype, device=a.device)
-            self.lib.check(self.lib.xr_gemm_bf16(out.data_ptr(), a.data_ptr(), w.data_ptr(), _ptr(bias), M, F, K,
+            self.lib.check(self.lib.xr_gemm_bf16(out.data_ptr(), a.data_ptr(), wt.data_ptr(), _ptr(bias), M, F, K,
                                                  a.stride(0), F, dtype_code(out.dtype), 2, variant,
-                                                 *self._gemm_workspace(a.device), _stream()))
+                                                 1 if packed else 0, *self._gemm_workspace(a.device), _stream()))
             return out
+        if packed:
+            raise KernelError("linear_swiglu: a packed weight needs bfloat16 rows that are 16-byte aligned")
         return self.silu_mul(self.linear(a, w, bias=bias))
 
     # -- attention --------------------------------------------------------------

@@ -15,6 +15,7 @@ No memset is recorded: the step's kernels write every byte they later read.
 """
 from __future__ import annotations
 
+import gc
 from typing import Dict, List, Optional, Tuple
 
 import numpy as np
@@ -222,9 +223,19 @@ class DecodeGraphs:
         out = r.model.logits(ctx, x, ctx.want_rows)
         torch.cuda.synchronize()
         graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(graph, pool=self.pool):
-            gx = r.model.forward(ctx, r.storage.layers)
-            glogits = r.model.logits(ctx, gx, ctx.want_rows)
+        # No garbage collection while the stream records: an earlier step's context that a
+        # collection frees gives back pinned memory, which is no operation a recording allows
+        # (the process aborts).  Cycles are collected before, and again afterwards as usual.
+        gc.collect()
+        gc_was_on = gc.isenabled()
+        gc.disable()
+        try:
+            with torch.cuda.graph(graph, pool=self.pool):
+                gx = r.model.forward(ctx, r.storage.layers)
+                glogits = r.model.logits(ctx, gx, ctx.want_rows)
+        finally:
+            if gc_was_on:
+                gc.enable()
         if self.pool is None:
             self.pool = graph.pool()
         self.graphs[key] = (ctx, graph, glogits)

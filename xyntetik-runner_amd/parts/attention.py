@@ -74,8 +74,8 @@ class PagedAttention(Mixer):
         mats = [tensors[f"{q}.weight"]]
         if not self.kv_shared:
             mats += [tensors[f"{k}.weight"], tensors[f"{v}.weight"]]
-        self.w_in = torch.cat(mats, dim=0).contiguous() if len(mats) > 1 else mats[0]
-        self.w_out = tensors[f"{o}.weight"]
+        self.w_in = rt.ops.pack_weight(torch.cat(mats, dim=0).contiguous() if len(mats) > 1 else mats[0])
+        self.w_out = rt.ops.pack_weight(tensors[f"{o}.weight"])
         if self.bias:
             bs = [tensors[f"{q}.bias"]]
             if not self.kv_shared:

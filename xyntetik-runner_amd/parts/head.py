@@ -23,9 +23,12 @@ class LinearHead(Part):
 
     def bind(self, tensors, rt, tied_to=None) -> None:
         self.rt = rt
-        self.weight = tied_to if self.tied else tensors[self.weight_name]
-        if self.weight is None:
+        weight = tied_to if self.tied else tensors[self.weight_name]
+        if weight is None:
             raise ValueError("a tied head needs the embedding table")
+        # in the kernels' own order where they have one (a tied head then keeps a copy of its own:
+        # the embedding gathers rows from the table as it is stored)
+        self.weight = rt.ops.pack_weight(weight)
 
     def forward(self, ctx, h):
         return self.rt.ops.linear(h, self.weight, out_dtype=torch.float32)

@@ -38,8 +38,10 @@ class GatedMLP(FeedForward):
     def bind(self, tensors, rt) -> None:
         self.rt = rt
         g, u, d = self.names
-        self.w_gate_up = torch.cat([tensors[f"{g}.weight"], tensors[f"{u}.weight"]], dim=0).contiguous()
-        self.w_down = tensors[f"{d}.weight"]
+        # gate rows then up rows, so that one product makes both; in the kernels' own order
+        self.w_gate_up = rt.ops.pack_weight(
+            torch.cat([tensors[f"{g}.weight"], tensors[f"{u}.weight"]], dim=0).contiguous(), gated=True)
+        self.w_down = rt.ops.pack_weight(tensors[f"{d}.weight"])
         if self.bias:
             self.b_gate_up = torch.cat([tensors[f"{g}.bias"], tensors[f"{u}.bias"]]).float().contiguous()
             self.b_down = tensors[f"{d}.bias"].float().contiguous()
