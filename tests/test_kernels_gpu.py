@@ -117,11 +117,11 @@ def test_linear_packed_weights_give_the_same(ops, M, N, K):
     assert isinstance(pw, PackedWeight) and pw.shape == (N, K)
     blocks = pw.data.cpu()
     n, k = 16 * (N // 16) + min(N % 16, 3) - (1 if N % 16 == 0 else 0), 8 * (K // 8 - 1)   # some row and chunk that exist
-    assert torch.equal(blocks[n // 16, k // 32, (k % 32) // 8, n % 16], w[n, k:k + 8].cpu())
+    assert torch.equal(blocks[n // 16, k // 32, n % 16, k % 32:k % 32 + 8], w[n, k:k + 8].cpu())
     if N % 16:
-        assert (blocks[-1, :, :, N % 16:] == 0).all()                   # rows that do not exist
+        assert (blocks[-1, :, N % 16:, :] == 0).all()                   # rows that do not exist
     if K % 32:
-        assert (blocks[:, -1, (K % 32) // 8:] == 0).all()               # nor columns
+        assert (blocks[:, -1, :, K % 32:] == 0).all()                   # nor columns
     want = a.double() @ w.double().T + b.double()
     got = ops.linear(a, pw, bias=b, out_dtype=torch.float32)
     assert rel(got, want) < 1e-5

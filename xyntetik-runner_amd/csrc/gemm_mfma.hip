@@ -158,8 +158,9 @@ __global__ __launch_bounds__(64 * WARPS_M * WARPS_N) void k_gemm_tile_async(Gemm
             const bool ok = oc < g.N && n < n_rows;
             if (g.w_packed) {
                 // row n % 16 of group n / 16; the slice's 64 columns are 2 blocks, chunk c the
-                // (c % 4)-th of its row in block c / 4; a slice further on is 2 blocks = 1024 elements on
-                src[i] = ok ? g.w + (size_t)(n >> 4) * kblocks * 512 + (c >> 2) * 512 + ((c & 3) * 16 + (n & 15)) * 8 : nullptr;
+                // (c % 4)-th of its row in block c / 4; a slice further on is 2 blocks = 1024 elements on,
+                // so one copy instruction of a wave (8 rows) reads two runs of 512 bytes
+                src[i] = ok ? g.w + (size_t)(n >> 4) * kblocks * 512 + (c >> 2) * 512 + (n & 15) * 32 + (c & 3) * 8 : nullptr;
                 src_kmul[i] = 16;
             } else {
                 src[i] = ok ? g.w + (size_t)n * g.K + c * 8 : nullptr;
@@ -355,8 +356,8 @@ __global__ __launch_bounds__(64 * KSW) void k_gemm_skinny(GemmArgs g) {
     // the wave reads the k-step's block of its group, the lane its 16 bytes of it.
     const size_t kblocks = (size_t)((g.K + 31) / 32);
     const int step_stride = g.w_packed ? 512 : 32;
-    const int lane_off = g.w_packed ? lane * 8 : lq * 8;
-    const int dead_off = g.w_packed ? lane * 8 : 0;      // where a lane whose column does not exist reads
+    const int lane_off = g.w_packed ? (l16 * 4 + lq) * 8 : lq * 8;
+    const int dead_off = g.w_packed ? (l16 * 4 + lq) * 8 : 0;      // where a lane whose column does not exist reads
     const bf16_t* wp[NWT][RT];
     bool w_ok[RT];
 #pragma unroll
@@ -472,15 +473,16 @@ static int launch_skinny(const GemmArgs& g, hipStream_t stream) {
 }
 
 // ------------------------------------------------------------------------------ packing
-// dst [ceil(N/16)][ceil(K/32)][4 chunks][16 rows][8 columns] from src [N, K] row-major (K a
-// multiple of 8): within a block of 16 rows x 32 columns the 16-byte chunk of row r and columns
-// 8c .. 8c+7 is the (16 c + r)-th, which is the one lane 16 c + r of a wave feeds to
-// v_mfma_f32_16x16x32_bf16.  Rows and columns that do not exist are zeros.  A thread moves one chunk.
+// dst [ceil(N/16)][ceil(K/32)][16 rows][32 columns] from src [N, K] row-major (K a multiple
+// of 8): a block is what one v_mfma_f32_16x16x32_bf16 takes as its weight operand, 1 KB that a
+// wave reads with one load (lane 16 c + r the 16 bytes of row r, columns 8c .. 8c+7).  Rows
+// and columns that do not exist are zeros.  A thread moves one 16-byte chunk.  (Measured: rows
+// within a block rather than chunks within a block serve both kernels best.)
 __global__ __launch_bounds__(256) void k_pack_weight(bf16_t* dst, const bf16_t* src, int N, int K, size_t chunks) {
     const size_t q = (size_t)blockIdx.x * 256 + threadIdx.x;
     if (q >= chunks) return;
     const size_t kblocks = (size_t)((K + 31) / 32);
-    const int r = (int)(q & 15), c = (int)((q >> 4) & 3);
+    const int c = (int)(q & 3), r = (int)((q >> 2) & 15);
     const size_t blk = q >> 6, grp = blk / kblocks, kb = blk - grp * kblocks;
     const size_t n = grp * 16 + r, k = kb * 32 + c * 8;
     uint4 v = make_uint4(0, 0, 0, 0);

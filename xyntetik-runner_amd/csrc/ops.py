@@ -59,8 +59,8 @@ def _stream() -> int:
 
 class PackedWeight:
     """A bfloat16 weight matrix ``[rows, cols]`` in the order the MFMA kernels read it: blocks of
-    16 rows x 32 columns, 1 KB each (``data[row group, column block, chunk, row, 8 columns]``),
-    rows and columns padded with zeros.  Made by
+    16 rows x 32 columns, 1 KB each (``data[row group, column block, row, column]``), rows and
+    columns padded with zeros.  Made by
     ``Ops.pack_weight``; ``Ops.linear`` and ``Ops.linear_swiglu`` take it in place of the matrix."""
 
     def __init__(self, data: torch.Tensor, rows: int, cols: int):
@@ -209,7 +209,7 @@ class Ops:
             return w
         self._dev(w)
         self._contig(w, "pack_weight input")
-        data = torch.empty((-(-N // 16), -(-K // 32), 4, 16, 8), dtype=torch.bfloat16, device=w.device)
+        data = torch.empty((-(-N // 16), -(-K // 32), 16, 32), dtype=torch.bfloat16, device=w.device)
         self.lib.check(self.lib.xr_pack_weight(data.data_ptr(), w.data_ptr(), N, K, _stream()))
         return PackedWeight(data, N, K)
 
