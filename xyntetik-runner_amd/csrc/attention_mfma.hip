@@ -670,6 +670,7 @@ extern "C" int xr_attention_mfma(void* out, const void* q, const void* k_cache, 
         static bool attr_set = false;
         if (!attr_set) {
             hipError_t e = hipFuncSetAttribute((const void*)k_attn_cta, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+            if (e != hipSuccess) (void)hipGetLastError();     // or the next launch's check would report this refusal
             XR_REQUIRE(e == hipSuccess, "attention: %d bytes of LDS refused: %s", smem, hipGetErrorString(e));
             attr_set = true;
         }
@@ -681,6 +682,7 @@ extern "C" int xr_attention_mfma(void* out, const void* q, const void* k_cache, 
         if (!attr_set) {
             hipError_t e = hipFuncSetAttribute((const void*)k_attn_stream, hipFuncAttributeMaxDynamicSharedMemorySize,
                                                STREAM_LDS_BYTES);
+            if (e != hipSuccess) (void)hipGetLastError();
             XR_REQUIRE(e == hipSuccess, "attention: %d bytes of LDS refused: %s", STREAM_LDS_BYTES, hipGetErrorString(e));
             attr_set = true;
         }

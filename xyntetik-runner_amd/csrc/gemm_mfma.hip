@@ -305,7 +305,11 @@ static int launch_tile_async(GemmArgs g, hipStream_t stream) {
     if (!attr_set) {
         hipError_t e = hipFuncSetAttribute((const void*)k_gemm_tile_async<BM, BN, WM_, WN_, ST>,
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
-        if (e != hipSuccess) { xr_set_error("gemm: cannot reserve %zu bytes of LDS: %s", smem, hipGetErrorString(e)); return XR_LAUNCH; }
+        if (e != hipSuccess) {
+            (void)hipGetLastError();             // or the next launch's check would report this refusal
+            xr_set_error("gemm: cannot reserve %zu bytes of LDS: %s", smem, hipGetErrorString(e));
+            return XR_LAUNCH;
+        }
         attr_set = true;
     }
     int n_out_tile = g.epi == EPI_SWIGLU ? BN / 2 : BN;
@@ -463,7 +467,11 @@ static int launch_skinny(const GemmArgs& g, hipStream_t stream) {
     if (!attr_set) {
         hipError_t e = hipFuncSetAttribute((const void*)k_gemm_skinny<MT, RT, KSW, U, SW, NT>,
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
-        if (e != hipSuccess) { xr_set_error("gemm: cannot reserve %zu bytes of LDS: %s", smem, hipGetErrorString(e)); return XR_LAUNCH; }
+        if (e != hipSuccess) {
+            (void)hipGetLastError();             // or the next launch's check would report this refusal
+            xr_set_error("gemm: cannot reserve %zu bytes of LDS: %s", smem, hipGetErrorString(e));
+            return XR_LAUNCH;
+        }
         attr_set = true;
     }
     unsigned blocks = (unsigned)((g.N + 16 * RT - 1) / (16 * RT));
@@ -549,11 +557,12 @@ extern "C" int xr_gemm_bf16(void* out, const void* a, const void* w, const float
     if (variant == 1) {
         XR_REQUIRE(M <= 64, "gemm: the skinny kernel takes at most 64 rows, got %d", M);
         if (M <= 16) {
-            // measured on MI355X at M = 1 and 8 (waves per workgroup, loads per batch):
+            // measured on MI355X with packed weights at M = 1, 8 and 16 (waves per workgroup, loads
+            // per batch): the output head, q/k/v, the down product, the output product
             if (sw) return launch_skinny<1, 1, 8, 8, true>(g, stream);
-            if (N >= 65536 || (N > 4096 && K <= 8192)) return launch_skinny<1, 2, 4, 8, false>(g, stream);
-            if (K > 8192) return launch_skinny<1, 1, 4, 8, false>(g, stream);
-            return launch_skinny<1, 1, 4, 16, false>(g, stream);
+            if (N >= 65536) return M <= 8 ? launch_skinny<1, 1, 8, 8, false>(g, stream) : launch_skinny<1, 2, 4, 8, false>(g, stream);
+            if (N > 4096 && K <= 8192) return M <= 8 ? launch_skinny<1, 1, 4, 8, false>(g, stream) : launch_skinny<1, 2, 4, 8, false>(g, stream);
+            return launch_skinny<1, 1, 8, 4, false>(g, stream);
         }
         if (M <= 32) return sw ? launch_skinny<2, 1, 16, 8, true>(g, stream) : launch_skinny<2, 1, 16, 8, false>(g, stream);
         return sw ? launch_skinny<4, 2, 8, 4, true>(g, stream) : launch_skinny<4, 2, 8, 4, false>(g, stream);
@@ -567,6 +576,9 @@ extern "C" int xr_gemm_bf16(void* out, const void* a, const void* w, const float
     SK(140, 4, 2, 8, 4, false) SK(141, 4, 1, 8, 4, false) SK(142, 4, 1, 16, 4, false) SK(143, 4, 2, 4, 4, false)
     SK(144, 4, 4, 4, 2, false) SK(145, 4, 2, 8, 4, true) SK(146, 4, 1, 8, 8, false) SK(147, 4, 2, 8, 2, false)
     SK(148, 4, 4, 4, 4, false) SK(149, 4, 4, 8, 2, false)
+    SK(116, 1, 1, 4, 32, false) SK(117, 1, 1, 8, 4, false) SK(118, 1, 2, 8, 4, false) SK(119, 1, 2, 4, 16, false)
+    SK(120, 1, 1, 2, 32, false) SK(121, 1, 4, 4, 8, false) SK(122, 1, 2, 2, 16, false) SK(123, 1, 1, 16, 16, false)
+    SK(124, 1, 4, 8, 4, false) SK(125, 1, 2, 16, 8, false) SK(126, 1, 4, 2, 8, false)
 #undef SK
 #endif
     if (variant == 10) return launch_tile_async<128, 128, 2, 2, 3>(g, stream);
