@@ -131,6 +131,34 @@ def test_sampling_kernel_distribution_and_many_rows():
     assert np.all(got2[0::2] == 5) and np.array_equal(got2[1::2], got[1::2])
 
 
+def test_greedy_pick_over_a_long_row_split_in_ranges():
+    """Long rows are read by several workgroups: the first index of the maximum must still win,
+    wherever the ties fall, and rows with temperature beside them are left to the sampler."""
+    import torch
+    from xyntetik_runner_amd.csrc.ops import load_ops
+    ops = load_ops()
+    dev = torch.device("cuda:0")
+    V = 50001                                             # no multiple of the 32 ranges, nor of 4
+    rng = np.random.default_rng(3)
+    rows = rng.normal(size=(7, V)).astype(np.float32)
+    chunk = ((V + 31) // 32 + 3) & ~3
+    rows[0, [chunk - 1, chunk, 3 * chunk + 5, V - 1]] = 9.0   # ties on both sides of a range's edge and at the end
+    rows[1, V - 1] = 9.0                                   # the last element alone
+    rows[2, :] = -np.inf                                   # nothing is larger than anything: index 0
+    rows[3, :] = np.nan
+    rows[3, 40000] = -5.0                                  # the only number
+    rows[4, 0] = 9.0
+    rows[5, [17, 30000]] = [8.0, 9.0]
+    t = torch.tensor(rows, device=dev)
+    temp = torch.zeros(7, device=dev)
+    temp[6] = 1.0
+    rows[6, :] = -30.0
+    rows[6, 123] = 30.0                                    # a sampled row with one token that has all the mass
+    t[6] = torch.tensor(rows[6], device=dev)
+    got = ops.sample(t, temp, torch.full((7,), 0.5, device=dev)).cpu().tolist()
+    assert got == [chunk - 1, V - 1, 0, 40000, 0, 30000, 123]
+
+
 def test_preemption_gives_the_same_tokens(folders):
     """A pool too small for all requests at once: some are preempted and recomputed, and
     every request still gets the tokens it gets when it has the cache to itself."""

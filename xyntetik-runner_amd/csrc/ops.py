@@ -45,7 +45,7 @@ _PROTOS = {
     "xr_gemm_bf16": [_p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _i, _p, _sz, _p],
     "xr_pack_weight": [_p, _p, _i, _i, _p],
     "xr_attention_ref": [_p, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _f, _i, _i, _p],
-    "xr_sample": [_p, _p, _i, _i, _i, _p, _p, _p, _p, _p, _p, _p, _p, _i, _p, _i, _p],
+    "xr_sample": [_p, _p, _i, _i, _i, _p, _p, _p, _p, _p, _p, _p, _p, _i, _p, _i, _p, _p],
 }
 
 
@@ -362,11 +362,13 @@ class Ops:
             raise KernelError("sample: logits must be float32 [rows, vocab]")
         W, V = logits.shape
         out = torch.empty((W,), dtype=torch.int32, device=logits.device)
+        # room for the greedy rows' first pass (32 ranges a row) when a row is long enough to need one
+        greedy_ws = torch.empty((W, 32, 2), dtype=torch.float32, device=logits.device) if V >= 8192 else None
         self.lib.check(self.lib.xr_sample(
             out.data_ptr(), logits.data_ptr(), W, V, logits.stride(0), temp.data_ptr(), _ptr(top_k),
             _ptr(top_p), _ptr(min_p), _ptr(repeat_penalty), draw.data_ptr(), _ptr(recent), _ptr(n_recent),
             recent.shape[1] if recent is not None else 0, _ptr(exempt),
-            exempt.numel() if exempt is not None else 0, _stream()))
+            exempt.numel() if exempt is not None else 0, _ptr(greedy_ws), _stream()))
         return out
 
 

@@ -34,7 +34,44 @@ struct SampleArgs {
     int recent_cap;
     const int* exempt;
     int n_exempt;
+    const float* greedy_part;   // [W, GREEDY_SPLITS, 2] (value, index bits) from k_greedy_partial, or null
 };
+
+#define GREEDY_SPLITS 32
+
+// The greedy pick's first pass for rows without temperature: a row's logits are read by
+// GREEDY_SPLITS workgroups instead of one (one workgroup reads 128k logits in 60 us, bound by
+// its loads' latency), each leaving the maximum of its range and the first index that has it.
+__global__ __launch_bounds__(256) void k_greedy_partial(const float* logits, int ld, int V, const float* temp, float* part) {
+    const int r = blockIdx.x, sp = blockIdx.y;
+    if (temp[r] > 0.f) return;
+    const int chunk = ((V + GREEDY_SPLITS - 1) / GREEDY_SPLITS + 3) & ~3;
+    const int lo = sp * chunk, hi = lo + chunk < V ? lo + chunk : V;
+    const float* row = logits + (size_t)r * ld;
+    float best = -INFINITY;
+    int bi = 0x7fffffff;
+    for (int i = lo + threadIdx.x; i < hi; i += 256) {
+        float v = row[i];
+        if (v > best || (v == best && i < bi)) { best = v; bi = i; }
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+        float ob = __shfl_xor(best, o, 64);
+        int oi = __shfl_xor(bi, o, 64);
+        if (ob > best || (ob == best && oi < bi)) { best = ob; bi = oi; }
+    }
+    __shared__ float sb[4];
+    __shared__ int si[4];
+    if ((threadIdx.x & 63) == 0) { sb[threadIdx.x >> 6] = best; si[threadIdx.x >> 6] = bi; }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        for (int w = 1; w < 4; ++w)
+            if (sb[w] > best || (sb[w] == best && si[w] < bi)) { best = sb[w]; bi = si[w]; }
+        float* p = part + ((size_t)r * GREEDY_SPLITS + sp) * 2;
+        p[0] = best;
+        p[1] = __int_as_float(bi);
+    }
+}
 
 __device__ inline uint32_t order_key32(float z) {
     if (z != z) return 0xFFFFFFFFu;          // NaN sorts last
@@ -147,12 +184,20 @@ __global__ __launch_bounds__(SM_THREADS) void k_sample(SampleArgs a) {
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
 
     if (!(temp > 0.f)) {
-        // greedy: first index of the maximum
+        // greedy: first index of the maximum, over the logits or over the ranges' results
         float best = -INFINITY;
         int bi = 0x7fffffff;
-        for (int i = threadIdx.x; i < V; i += SM_THREADS) {
-            float v = row[i];
-            if (v > best || (v == best && i < bi)) { best = v; bi = i; }
+        if (a.greedy_part) {
+            if (threadIdx.x < GREEDY_SPLITS) {
+                const float* p = a.greedy_part + ((size_t)r * GREEDY_SPLITS + threadIdx.x) * 2;
+                best = p[0];
+                bi = __float_as_int(p[1]);
+            }
+        } else {
+            for (int i = threadIdx.x; i < V; i += SM_THREADS) {
+                float v = row[i];
+                if (v > best || (v == best && i < bi)) { best = v; bi = i; }
+            }
         }
 #pragma unroll
         for (int o = 32; o > 0; o >>= 1) {
@@ -224,7 +269,7 @@ __global__ __launch_bounds__(SM_THREADS) void k_sample(SampleArgs a) {
 extern "C" int xr_sample(int* out, float* logits, int W, int V, int ld, const float* temp, const int* top_k,
                          const float* top_p, const float* min_p, const float* repeat_penalty,
                          const float* draw, const int* recent, const int* n_recent, int recent_cap,
-                         const int* exempt, int n_exempt, hipStream_t stream) {
+                         const int* exempt, int n_exempt, float* greedy_ws, hipStream_t stream) {
     XR_REQUIRE(W >= 0 && V > 0 && ld >= V, "sample: bad sizes W=%d V=%d ld=%d", W, V, ld);
     XR_REQUIRE(V <= (1 << 24), "sample: vocabulary %d exceeds 2^24", V);
     XR_REQUIRE(out && logits && temp && draw, "sample: null operand");
@@ -234,6 +279,11 @@ extern "C" int xr_sample(int* out, float* logits, int W, int V, int ld, const fl
     a.out = out; a.logits = logits; a.ld = ld; a.V = V; a.temp = temp; a.top_k = top_k; a.top_p = top_p;
     a.min_p = min_p; a.repeat_penalty = repeat_penalty; a.draw = draw; a.recent = recent;
     a.n_recent = n_recent; a.recent_cap = recent_cap; a.exempt = exempt; a.n_exempt = exempt ? n_exempt : 0;
+    a.greedy_part = greedy_ws;
+    if (greedy_ws) {        // [W, GREEDY_SPLITS, 2] floats
+        k_greedy_partial<<<dim3(W, GREEDY_SPLITS), 256, 0, stream>>>(logits, ld, V, temp, greedy_ws);
+        XR_CHECK_LAUNCH("greedy_partial");
+    }
     k_sample<<<W, SM_THREADS, 0, stream>>>(a);
     XR_CHECK_LAUNCH("sample");
     return XR_OK;
