@@ -300,6 +300,10 @@ __global__ __launch_bounds__(256) void k_gemm_finish(GemmArgs g) {
 
 template <int BM, int BN, int WM_, int WN_, int ST>
 static int launch_tile_async(GemmArgs g, hipStream_t stream) {
+    if (g.epi == EPI_SWIGLU && (BN / WN_ / 32) % 2) {
+        xr_set_error("gemm: a %dx%d tile cannot pair gate and up columns", BM, BN);
+        return XR_BAD_ARG;
+    }
     size_t smem = (size_t)ST * (BM + BN) * 8 * 16;
     static bool attr_set = false;
     if (!attr_set) {
@@ -545,11 +549,24 @@ extern "C" int xr_gemm_bf16(void* out, const void* a, const void* w, const float
         } else if (M <= 64) {
             variant = 31;
         } else {
-            // the largest tile that still gives every compute unit a workgroup; if even the
-            // smallest does not, K is split as well
+            // The tile that keeps the chip busiest: larger tiles do more products for a byte that
+            // L1 delivers (what bounds this kernel), but their count may fill the 256 compute
+            // units badly.  A tile's worth is its measured rate with the chip full (relative to
+            // 256x256) times the share of the chip its rounds of workgroups keep busy; if even the
+            // smallest tile does not fill the chip, K is split as well.
             const int n_out = N;
             auto count = [&](int bm, int bn) { return ((M + bm - 1) / bm) * ((n_out + (sw ? bn / 2 : bn) - 1) / (sw ? bn / 2 : bn)); };
-            variant = count(256, 256) >= 180 ? 14 : (count(256, 128) >= 180 ? 12 : 17);
+            auto worth = [&](int bm, int bn, double rate) {
+                const int tiles = count(bm, bn);
+                return rate * tiles / (double)(((tiles + 255) / 256) * 256);
+            };
+            const double w256 = worth(256, 256, 1.0), w192 = sw ? 0.0 : worth(256, 192, 0.9);
+            const double w128 = worth(256, 128, 0.85), w64 = worth(128, 128, 0.78);
+            variant = 14;
+            double best = w256;
+            if (w192 > best) { variant = 26; best = w192; }
+            if (w128 > best) { variant = 12; best = w128; }
+            if (w64 > best) { variant = 17; best = w64; }
             g.m_fast = 1;
             if (variant == 17 && count(128, 128) < 160) g.splits = pick_splits(count(128, 128));
         }
@@ -592,6 +609,7 @@ extern "C" int xr_gemm_bf16(void* out, const void* a, const void* w, const float
     if (variant == 18) return launch_tile_async<256, 256, 2, 2, 2>(g, stream);
     if (variant == 19) return launch_tile_async<256, 128, 2, 2, 2>(g, stream);
     if (variant == 20) return launch_tile_async<128, 256, 2, 2, 2>(g, stream);
+    if (variant == 26) return launch_tile_async<256, 192, 4, 2, 2>(g, stream);
     if (variant == 30 || variant == 31) {       // few rows: 32 or 64 of them against 128 weight rows, K split
         const int bn_out = sw ? 64 : 128;
         g.splits = pick_splits((N + bn_out - 1) / bn_out);
