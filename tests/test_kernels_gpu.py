@@ -238,7 +238,9 @@ def scatter_pages(n_req_lens, page_size, seed):
 def ref_rope(x, pos, inv_freq, interleaved):
     T, H, D = x.shape
     half = inv_freq.numel()
-    ang = pos.double()[:, None] * inv_freq.double()[None, :]
+    # the angle is a 32-bit product, as the kernel's and the reference's is (position x frequency
+    # in float); its cosine and sine, and the rotation, in float64
+    ang = (pos.float()[:, None] * inv_freq.float()[None, :]).double()
     c, s = torch.cos(ang)[:, None, :], torch.sin(ang)[:, None, :]
     y = x.double().clone()
     i0 = torch.arange(half) * 2 if interleaved else torch.arange(half)
@@ -250,9 +252,11 @@ def ref_rope(x, pos, inv_freq, interleaved):
 
 @pytest.mark.parametrize("dt", ["float32", "bfloat16"])
 @pytest.mark.parametrize("H,Hk,D,rot,inter", [(4, 2, 16, 16, False), (3, 1, 48, 32, False), (6, 3, 80, 80, True), (8, 8, 128, 64, True)])
-def test_rope_kv_write(ops, dt, H, Hk, D, rot, inter):
-    ps = 8
-    starts, q_lens = [0, 13, 40], [9, 3, 1]
+@pytest.mark.parametrize("ps,starts,q_lens", [(8, [0, 13, 40], [9, 3, 1]), (64, [5, 64, 200, 0], [40, 17, 1, 8]),
+                                              (4, [2, 9], [7, 6])])
+def test_rope_kv_write(ops, dt, H, Hk, D, rot, inter, ps, starts, q_lens):
+    """Portions that bring whole aligned groups of 8 positions (their values go to the transposed
+    cache 8 at a time), groups cut at either end, single tokens, pages smaller than a group."""
     tables, n_pages = scatter_pages([s + n for s, n in zip(starts, q_lens)], ps, 1)
     ctx = FakeCtx(starts, q_lens, tables, ps)
     T = sum(q_lens)
@@ -279,6 +283,7 @@ def test_rope_kv_write(ops, dt, H, Hk, D, rot, inter):
             written[page, off] = True
             t += 1
     assert torch.isnan(kc.float().cpu().permute(0, 2, 1, 3)[~written]).all()      # nothing else was touched
+    assert torch.isnan(vc.float().cpu().permute(0, 3, 1, 2)[~written]).all()
     if rot < D:                                                               # channels beyond the rotary width pass through
         assert torch.equal(q_out.cpu().reshape(T, H, D)[..., rot:], qkv[:, :Q].cpu().reshape(T, H, D)[..., rot:].to(DT[dt]))
 

@@ -152,55 +152,91 @@ struct RopeArgs {
     const int* block_table; // [B, table_stride]
     int table_stride;
     const float* inv_freq;  // [rot/2] or null
-    int H, Hk, D, rot, interleaved;
+    int T, H, Hk, D, rot, interleaved;
     float mscale;
     int page_shift, page_mask, page_size;
+    int heads_per_block;
 };
 
-__device__ inline void rotate_pair(float x0, float x1, int pos, float f, float ms, float& y0, float& y1) {
-    float a = (float)pos * f;
-    float c = cosf(a) * ms, s = sinf(a) * ms;
-    y0 = x0 * c - x1 * s;
-    y1 = x0 * s + x1 * c;
+// 8 values of one channel at 8 consecutive positions of a page: 16 or 32 bytes side by side in
+// the transposed value cache.
+template <typename T> __device__ inline void store8(T* dst, const float* v);
+template <> __device__ inline void store8<float>(float* dst, const float* v) {
+    *reinterpret_cast<float4*>(dst) = make_float4(v[0], v[1], v[2], v[3]);
+    *reinterpret_cast<float4*>(dst + 4) = make_float4(v[4], v[5], v[6], v[7]);
+}
+template <> __device__ inline void store8<bf16_t>(bf16_t* dst, const float* v) {
+    *reinterpret_cast<uint4*>(dst) = make_uint4(pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3]),
+                                                pack_bf16x2(v[4], v[5]), pack_bf16x2(v[6], v[7]));
 }
 
+// A workgroup takes a token and some of its heads (heads_per_block, a wave a head at a time):
+// query heads are rotated into q_out, key heads rotated into their page, value heads written
+// to theirs.  The cosines and sines of the token's angles are computed once per workgroup into
+// LDS and serve every head (the exact cosf/sinf of 64 angles for each of 40 heads was what the
+// kernel's time went to).  Values are cached transposed ([channel][position]), so a token
+// alone writes one element every page_size: where the step brings the 8 positions of an
+// aligned group of a page (prompt portions), the wave of the group's first token writes all 8
+// side by side for each channel and the other seven leave their values to it.
 template <typename T>
-__global__ void k_rope_kv_write(RopeArgs a) {
-    int t = blockIdx.x;
-    int hs = blockIdx.y;
-    int pos = a.positions[t];
-    int D = a.D, half = a.rot >> 1;
-    if (hs < a.H) {
-        const float* src = a.q_in + (size_t)t * a.in_stride + (size_t)hs * D;
-        T* dst = (T*)a.q_out + ((size_t)t * a.H + hs) * D;
-        for (int j = threadIdx.x; j < half; j += blockDim.x) {
-            int i0 = a.interleaved ? 2 * j : j;
-            int i1 = a.interleaved ? 2 * j + 1 : j + half;
-            float y0, y1;
-            rotate_pair(src[i0], src[i1], pos, a.inv_freq[j], a.mscale, y0, y1);
-            st<T>(dst, i0, y0);
-            st<T>(dst, i1, y1);
+__global__ __launch_bounds__(256) void k_rope_kv_write(RopeArgs a) {
+    __shared__ float cs[2][128];
+    const int t = blockIdx.x;
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int pos = a.positions[t];
+    const int D = a.D, half = a.rot >> 1;
+    for (int j = threadIdx.x; j < half; j += 256) {
+        const float ang = (float)pos * a.inv_freq[j];
+        cs[0][j] = cosf(ang) * a.mscale;
+        cs[1][j] = sinf(ang) * a.mscale;
+    }
+    __syncthreads();
+    const int h_end = min(a.H + a.Hk, (int)(blockIdx.y + 1) * a.heads_per_block);
+    for (int hs = blockIdx.y * a.heads_per_block + wave; hs < h_end; hs += 4) {
+        if (hs < a.H) {
+            const float* src = a.q_in + (size_t)t * a.in_stride + (size_t)hs * D;
+            T* dst = (T*)a.q_out + ((size_t)t * a.H + hs) * D;
+            for (int j = lane; j < half; j += 64) {
+                const int i0 = a.interleaved ? 2 * j : j;
+                const int i1 = a.interleaved ? 2 * j + 1 : j + half;
+                const float x0 = src[i0], x1 = src[i1], c = cs[0][j], sn = cs[1][j];
+                st<T>(dst, i0, x0 * c - x1 * sn);
+                st<T>(dst, i1, x0 * sn + x1 * c);
+            }
+            for (int i = a.rot + lane; i < D; i += 64) st<T>(dst, i, src[i]);
+            continue;
         }
-        for (int i = a.rot + threadIdx.x; i < D; i += blockDim.x) st<T>(dst, i, src[i]);
-        return;
+        const int kvh = hs - a.H;
+        const int req = a.req_of_token[t];
+        PageRef pr = page_of(a.block_table, a.table_stride, req, pos, a.page_shift, a.page_mask);
+        const float* ks = a.k_in + (size_t)t * a.in_stride + (size_t)kvh * D;
+        const float* vs = a.v_in + (size_t)t * a.in_stride + (size_t)kvh * D;
+        T* kd = (T*)a.k_cache + (((size_t)pr.page * a.Hk + kvh) * a.page_size + pr.off) * D;
+        T* vd = (T*)a.v_cache + ((size_t)pr.page * a.Hk + kvh) * D * a.page_size + pr.off;
+        for (int j = lane; j < half; j += 64) {
+            const int i0 = a.interleaved ? 2 * j : j;
+            const int i1 = a.interleaved ? 2 * j + 1 : j + half;
+            const float x0 = ks[i0], x1 = ks[i1], c = cs[0][j], sn = cs[1][j];
+            st<T>(kd, i0, x0 * c - x1 * sn);
+            st<T>(kd, i1, x0 * sn + x1 * c);
+        }
+        for (int i = a.rot + lane; i < D; i += 64) st<T>(kd, i, ks[i]);
+        // the aligned group of 8 positions this token belongs to: whole in this step?  (A request's
+        // tokens of a step are consecutive rows at consecutive positions.)
+        const int lead = t - (pos & 7);
+        const bool whole = a.page_size >= 8 && lead >= 0 && lead + 7 < a.T && a.req_of_token[lead] == req &&
+                           a.req_of_token[lead + 7] == req && a.positions[lead] == pos - (pos & 7);
+        if (!whole) {
+            for (int i = lane; i < D; i += 64) st<T>(vd, (size_t)i * a.page_size, vs[i]);
+        } else if ((pos & 7) == 0) {
+            for (int i = lane; i < D; i += 64) {
+                float v[8];
+#pragma unroll
+                for (int j = 0; j < 8; ++j) v[j] = vs[(size_t)j * a.in_stride + i];
+                store8<T>(vd + (size_t)i * a.page_size, v);
+            }
+        }
     }
-    int kvh = hs - a.H;
-    int req = a.req_of_token[t];
-    PageRef pr = page_of(a.block_table, a.table_stride, req, pos, a.page_shift, a.page_mask);
-    const float* ks = a.k_in + (size_t)t * a.in_stride + (size_t)kvh * D;
-    const float* vs = a.v_in + (size_t)t * a.in_stride + (size_t)kvh * D;
-    T* kd = (T*)a.k_cache + (((size_t)pr.page * a.Hk + kvh) * a.page_size + pr.off) * D;
-    T* vd = (T*)a.v_cache + ((size_t)pr.page * a.Hk + kvh) * D * a.page_size + pr.off;
-    for (int j = threadIdx.x; j < half; j += blockDim.x) {
-        int i0 = a.interleaved ? 2 * j : j;
-        int i1 = a.interleaved ? 2 * j + 1 : j + half;
-        float y0, y1;
-        rotate_pair(ks[i0], ks[i1], pos, a.inv_freq[j], a.mscale, y0, y1);
-        st<T>(kd, i0, y0);
-        st<T>(kd, i1, y1);
-    }
-    for (int i = a.rot + threadIdx.x; i < D; i += blockDim.x) st<T>(kd, i, ks[i]);
-    for (int i = threadIdx.x; i < D; i += blockDim.x) st<T>(vd, (size_t)i * a.page_size, vs[i]);
 }
 
 extern "C" int xr_rope_kv_write(const float* q_in, const float* k_in, const float* v_in, int in_stride,
@@ -224,11 +260,18 @@ extern "C" int xr_rope_kv_write(const float* q_in, const float* k_in, const floa
     a.q_out = q_out; a.k_cache = k_cache; a.v_cache = v_cache;
     a.positions = positions; a.req_of_token = req_of_token;
     a.block_table = block_table; a.table_stride = table_stride; a.inv_freq = inv_freq;
-    a.H = H; a.Hk = Hk; a.D = D; a.rot = rot; a.interleaved = interleaved; a.mscale = mscale;
+    a.T = T; a.H = H; a.Hk = Hk; a.D = D; a.rot = rot; a.interleaved = interleaved; a.mscale = mscale;
     a.page_shift = shift < 0 ? 0 : shift; a.page_mask = page_size - 1; a.page_size = page_size;
-    dim3 grid(T, H + Hk);
-    if (dtype == XR_F32) k_rope_kv_write<float><<<grid, 64, 0, stream>>>(a);
-    else k_rope_kv_write<bf16_t><<<grid, 64, 0, stream>>>(a);
+    XR_REQUIRE(rot <= 256, "rope_kv_write: rotary width %d exceeds 256", rot);
+    // all heads of a token in one workgroup when there are tokens enough to fill the chip, else
+    // fewer heads each, down to one a wave
+    int groups = (1024 + T - 1) / T;
+    const int max_groups = (H + Hk + 3) / 4;
+    groups = groups < 1 ? 1 : (groups > max_groups ? max_groups : groups);
+    a.heads_per_block = (H + Hk + groups - 1) / groups;
+    dim3 grid(T, (H + Hk + a.heads_per_block - 1) / a.heads_per_block);
+    if (dtype == XR_F32) k_rope_kv_write<float><<<grid, 256, 0, stream>>>(a);
+    else k_rope_kv_write<bf16_t><<<grid, 256, 0, stream>>>(a);
     XR_CHECK_LAUNCH("rope_kv_write");
     return XR_OK;
 }
