@@ -185,7 +185,14 @@ __global__ __launch_bounds__(256, 2) void k_attn_cta(AttnArgs a) {
     extern __shared__ uint4 lds[];                          // [CTA_STAGES][STAGE_CHUNKS]
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int kvh = blockIdx.y;
-    const int* it = a.cta_items + (size_t)blockIdx.x * ITEM_INTS;
+    // Items come longest first.  Workgroups are handed to the compute units in the order of
+    // their numbers, two to a unit at this kernel's size, the second 256 numbers later.  When
+    // all of them run at once (at most 512), the upper half of the key/value heads takes the
+    // items in reverse, so that a unit's two workgroups are a long one and a short one (a
+    // causal prompt's blocks see 1 to n keys); with more, the longest must simply start first.
+    const bool pair_up = gridDim.x * gridDim.y <= 512 && blockIdx.y * 2 >= gridDim.y;
+    const int item_no = pair_up ? a.n_cta_items - 1 - (int)blockIdx.x : (int)blockIdx.x;
+    const int* it = a.cta_items + (size_t)item_no * ITEM_INTS;
     const int req = it[0], row0 = it[1] + wave * ROWS, kbeg = it[2], kend = it[3];
     const int slot = it[4] < 0 ? -1 : it[4] + wave;
     const int q0 = it[5], q_len = it[6], start = it[7];
