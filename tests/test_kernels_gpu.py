@@ -328,6 +328,9 @@ ATTN_CASES = [
     (5, 5, 80, 4, None, [10, 0], [3, 9]),          # small pages: the 32-bit kernel serves bfloat16 too
     (2, 1, 24, 8, 5, [0, 30], [12, 1]),            # head size no multiple of 16
     (32, 8, 128, 64, None, [2047, 1000], [1, 1]),  # decoding, long
+    (5, 1, 80, 32, None, [300, 10], [1, 3]),       # decoding with a head size that is no power of two
+    (4, 2, 256, 16, 600, [700, 3], [1, 2]),        # the largest head, small pages, a window that has given pages back
+    (6, 2, 48, 64, None, [5000], [1]),             # more than 64 pages: the page numbers are fetched again on the way
 ]
 
 
@@ -350,6 +353,40 @@ def test_attention(ops, dt, case):
     got = got.cpu().reshape(T, H, D)
     assert torch.isfinite(got.float()).all(), "read a slot no request owns"
     assert rel(got, want) < (3e-6 if dt == "float32" else 1.2e-2)
+
+
+def test_attention_items_longer_than_64_pages(ops):
+    """A work item keeps 64 page numbers in its lanes and fetches the next 64 on the way: items
+    that are not cut into key ranges (enough requests to fill the chip; a long portion left
+    whole) walk through several such sets."""
+    from xyntetik_runner_amd.engine.batch import plan_attention
+    torch.manual_seed(11)
+    # decoding: 32 requests x 8 key/value heads fill the chip, so nobody's 190 pages are cut
+    H, Hk, D, ps = 8, 8, 16, 16
+    starts = [2990 + 3 * i for i in range(32)]
+    q_lens = [1] * 32
+    assert all(it[4] == -1 for it in plan_attention(starts, q_lens, 1, None, Hk, ps)[1])
+    # a portion of 70 tokens after 3000, left whole: 96 pages of 32
+    for (H, Hk, D, ps, starts, q_lens, cta_tiles) in [(8, 8, 16, 16, starts, q_lens, None), (4, 2, 32, 32, [3000], [70], 1000)]:
+        lens = [s + n for s, n in zip(starts, q_lens)]
+        tables, n_pages = scatter_pages(lens, ps, 3)
+        ctx = FakeCtx(starts, q_lens, tables, ps, cta_tiles=cta_tiles)
+        T = sum(q_lens)
+        q = torch.randn(T, H, D).bfloat16()
+        k_seq = [torch.randn(n, Hk, D).bfloat16() for n in lens]
+        v_seq = [torch.randn(n, Hk, D).bfloat16() for n in lens]
+        # one key far back and one near the end stand out, in different sets of 64 pages
+        for b, n in enumerate(lens):
+            for far in (5, n - 40):
+                k_seq[b][far] = (q[sum(q_lens[:b])].float().reshape(Hk, H // Hk, D)[:, 0] * 3).bfloat16()
+        kc, vc = fill_cache(k_seq, v_seq, tables, n_pages, ps, torch.bfloat16)
+        scale = 1 / math.sqrt(D)
+        want = ref_attention(q.float(), [k.float() for k in k_seq], [v.float() for v in v_seq], starts, q_lens, scale, None)
+        got = ops.attention(q.to(DEV).reshape(T, H * D).contiguous(), kc, vc, ctx, 0, H, Hk, D, ps, scale, None)
+        got = got.cpu().reshape(T, H, D)
+        assert torch.isfinite(got.float()).all()
+        err = (got.double() - want).abs().amax(dim=(1, 2)) / want.abs().amax()
+        assert err.max() < 1.2e-2, f"token {int(err.argmax())}: {float(err.max())}"
 
 
 ATTN_WORKGROUP_CASES = [
