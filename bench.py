@@ -26,6 +26,12 @@ LLAMA_3_1_8B = {
                      "original_max_position_embeddings": 8192},
     "rms_norm_eps": 1e-5, "tie_word_embeddings": False, "max_position_embeddings": 8192, "hidden_act": "silu",
 }
+# other sizes of the same architecture (--shape); the default and the contract's line are the 8B shape
+LLAMA_2_7B = dict(LLAMA_3_1_8B, num_key_value_heads=32, intermediate_size=11008, vocab_size=32000, rope_theta=10000.0,
+                  rope_scaling=None, max_position_embeddings=4096)
+LLAMA_3_1_70B = dict(LLAMA_3_1_8B, num_hidden_layers=80, hidden_size=8192, num_attention_heads=64, intermediate_size=28672)
+SHAPES = {"llama-3.1-8b": ("Llama-3.1-8B shape", LLAMA_3_1_8B), "llama-2-7b": ("Llama-2-7B shape", LLAMA_2_7B),
+          "llama-3.1-70b": ("Llama-3.1-70B shape", LLAMA_3_1_70B)}
 PEAK = {"hbm_gbs": 8000.0, "bf16_flops": 2.5e15, "fp32_flops": 157.3e12}
 
 
@@ -44,7 +50,8 @@ def build_runner(cfg, dtype, max_tokens, max_requests, seed=0):
     spec = arch.build_spec(typed)
     t0 = time.time()
     state = random_state(Model.expected_tensors(spec), seed, device=torch.device("cuda:0"))
-    runner = ModelRunner(spec, state, dtype, max_tokens=max_tokens, page_size=64, max_requests=max_requests)
+    runner = ModelRunner(spec, state, dtype, max_tokens=max_tokens, page_size=64, max_requests=max_requests,
+                         consume_state=True)      # the 70B shape is half the card: it must not stand there twice
     del state
     torch.cuda.synchronize()
     log(f"model with {len(spec.layers)} layers on the GPU in {time.time() - t0:.1f} s")
@@ -109,6 +116,35 @@ def measure_decode(runner, cfg, batch, prompt_len, steps, warmup, seed):
     return batch * steps / dt, dt / steps, (ctx0 + ctx1) / 2
 
 
+def measure_mixed(runner, cfg, n_requests, steps_each, seed):
+    """A scheduler workload: `n_requests` prompts of 128..2048 tokens admitted at once, `steps_each`
+    tokens decoded for each, portions of prompts beside decoded tokens under a 2048-token budget.
+    Returns (prompt tokens, decoded tokens, seconds, steps)."""
+    import numpy as np
+    import torch
+    from xyntetik_runner_amd.engine import Engine
+    from xyntetik_runner_amd.sampling import SamplingParams
+    eng = Engine(runner, max_batched_tokens=2048, max_running=n_requests,
+                 max_model_len=cfg["max_position_embeddings"], stop_ids=[])
+    rng = np.random.default_rng(seed)
+    lens = [int(n) for n in rng.integers(128, 2049, size=n_requests)]
+    sp = SamplingParams(temperature=0.0, max_new_tokens=steps_each, ignore_eos=True)
+    for n in lens:
+        eng.add_request([int(t) for t in rng.integers(0, cfg["vocab_size"], size=n)], sp)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    n_steps = 0
+    while eng.has_work():
+        eng.step()
+        n_steps += 1
+    torch.cuda.synchronize()
+    secs = time.perf_counter() - t0
+    done = [eng.requests.pop(rid) for rid in list(eng.requests)]
+    if any(len(r.output) != steps_each for r in done):
+        raise RuntimeError("mixed workload: a request ended early")
+    return sum(lens), n_requests * steps_each, secs, n_steps
+
+
 def measure_prefill(runner, cfg, T, repeats, seed):
     import numpy as np
     import torch
@@ -138,17 +174,22 @@ def main():
     ap.add_argument("--prompt-len", type=int, default=2048)
     ap.add_argument("--no-points", action="store_true", help="skip decode at batch 1 and 64")
     ap.add_argument("--dtype", default="bfloat16")
+    ap.add_argument("--shape", default="llama-3.1-8b", choices=sorted(SHAPES), help="sizes of the model (same architecture)")
+    ap.add_argument("--mixed", type=int, default=0, metavar="N",
+                    help="also run N requests with prompts of 128..2048 tokens and 128 decoded tokens each through the scheduler")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU only: --gpus {args.gpus} is not supported by this engine", flush=True)
         return 2
-    cfg = dict(LLAMA_3_1_8B)
+    shape_name, shape_cfg = SHAPES[args.shape]
+    cfg = {k: v for k, v in shape_cfg.items() if v is not None}
     layers_full = cfg["num_hidden_layers"]
     layers = args.layers or layers_full
     cfg["num_hidden_layers"] = layers
     P, B = args.prompt_len, args.batch
     span = P + args.warmup + args.steps + 80 + max(64, B)
-    spec, runner = build_runner(cfg, args.dtype, max_tokens=max(64, B) * (-(-span // 64) * 64) + 4096, max_requests=64)
+    pool = max(max(64, B) * (-(-span // 64) * 64) + 4096, args.mixed * (2048 + 128 + 64))
+    spec, runner = build_runner(cfg, args.dtype, max_tokens=pool, max_requests=max(64, args.mixed))
 
     pre_s = measure_prefill(runner, cfg, 2048, repeats=3, seed=1)
     pre_frac = prefill_flops(cfg, layers, 2048) / pre_s / PEAK["bf16_flops" if args.dtype == "bfloat16" else "fp32_flops"]
@@ -166,12 +207,17 @@ def main():
             points[f"decode_b{b}"] = round(t, 1)
             log(f"decode batch {b}: {t:.1f} tok/s, {s * 1e3:.3f} ms/step, "
                 f"{decode_bytes(cfg, layers, b, c, elt) / s / 1e9:.0f} GB/s")
+    if args.mixed:
+        n_prompt, n_dec, secs, n_steps = measure_mixed(runner, cfg, args.mixed, 128, seed=9)
+        log(f"mixed: {args.mixed} requests, {n_prompt} prompt + {n_dec} decoded tokens in {secs:.2f} s "
+            f"({n_steps} steps): {(n_prompt + n_dec) / secs:.0f} tok/s in all, {n_dec / secs:.0f} decoded tok/s")
+        points["mixed_total_tok_s"] = round((n_prompt + n_dec) / secs, 1)
     line = {
-        "metric": "decode tokens/s, Llama-3.1-8B shape, batch 8, 2048-token prompts (random weights)",
+        "metric": f"decode tokens/s, {shape_name}, batch {B}, {P}-token prompts (random weights)",
         "value": round(tps, 1), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(step_s * 1e3, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16" if args.dtype == "bfloat16" else "fp32", "data": "synthetic",
-        "config": {"model": "Llama-3.1-8B shape", "layers": layers, "layers_in_config": layers_full,
+        "config": {"model": shape_name, "layers": layers, "layers_in_config": layers_full,
                    "hidden_size": cfg["hidden_size"], "heads": cfg["num_attention_heads"],
                    "kv_heads": cfg["num_key_value_heads"], "head_dim": cfg["head_dim"],
                    "intermediate_size": cfg["intermediate_size"], "vocab_size": cfg["vocab_size"],

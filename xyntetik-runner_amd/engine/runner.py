@@ -36,7 +36,7 @@ def parse_dtype(name) -> torch.dtype:
 
 class ModelRunner:
     def __init__(self, spec: ModelSpec, tensors_or_store, dtype, max_tokens: int, page_size: int = 64,
-                 max_requests: int = 64, device: str = "cuda:0", use_graphs: bool = True):
+                 max_requests: int = 64, device: str = "cuda:0", use_graphs: bool = True, consume_state: bool = False):
         if not torch.cuda.is_available():
             raise RuntimeError("no GPU: this engine runs on an MI355X only and has no CPU path")
         self.device = torch.device(device)
@@ -50,7 +50,7 @@ class ModelRunner:
         if isinstance(tensors_or_store, SafetensorsStore):
             tensors = load_tensors(tensors_or_store, expected, self.dtype, self.device)
         else:
-            tensors = load_state(tensors_or_store, expected, self.dtype, self.device)
+            tensors = load_state(tensors_or_store, expected, self.dtype, self.device, consume=consume_state)
         self.model.bind(tensors, self.rt)
         del tensors
         kv, st, of = self.model.cache_needs()

@@ -91,12 +91,14 @@ def load_tensors(store: SafetensorsStore, expected: Mapping[str, ParamSpec], com
 
 
 def load_state(tensors: Mapping[str, torch.Tensor], expected: Mapping[str, ParamSpec], compute: torch.dtype,
-               device: torch.device) -> Dict[str, torch.Tensor]:
-    """As ``load_tensors`` for tensors already in memory (the random-weights mode without a file)."""
+               device: torch.device, consume: bool = False) -> Dict[str, torch.Tensor]:
+    """As ``load_tensors`` for tensors already in memory (the random-weights mode without a file).
+    With ``consume`` the tensors are taken out of ``tensors`` (a dict) as they are used, so that a
+    model as large as half the memory does not stand there twice."""
     check_against(expected, tensors.keys(), lambda n: tuple(tensors[n].shape), lambda n: tensors[n].dtype)
     out = {}
     for name, spec in expected.items():
         if name in tensors:
-            t = tensors[name]
+            t = tensors.pop(name) if consume else tensors[name]
             out[name] = t.to(device=device, dtype=target_dtype(spec, t.dtype, compute)).contiguous()
     return out
