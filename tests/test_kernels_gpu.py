@@ -142,6 +142,67 @@ def test_linear_packed_weights_give_the_same(ops, M, N, K):
     assert torch.equal(got, ops.linear_swiglu(a, w2, bias=b2))
 
 
+@pytest.mark.parametrize("M", [1, 5, 16])
+@pytest.mark.parametrize("E,F,K", [(64, 96, 48), (200, 112, 72), (4096, 1024, 264), (72, 70000, 40), (5120, 8200, 256)])
+@pytest.mark.parametrize("wdtype", [torch.float32, torch.bfloat16])
+def test_rmsnorm_folded_into_the_products_around_it(ops, M, E, F, K, wdtype):
+    """residual += a @ w^T; h = rmsnorm(residual); y = h @ w2^T.  With the norm folded in, the
+    first product writes the weighted rows and partial sums of squares and the second applies
+    the scale: the residual keeps the same bits, y agrees with the norm done in 64-bit, and
+    neither depends on other rows of the batch."""
+    from xyntetik_runner_amd.csrc.ops import UnscaledRows
+    torch.manual_seed(M * 1000 + E)
+    a = (torch.randn(M, K, device=DEV) * 0.5).bfloat16()
+    w = ops.pack_weight((torch.randn(E, K, device=DEV) * 0.1).bfloat16())
+    nw = (1 + 0.2 * torch.randn(E, device=DEV)).to(wdtype)
+    w2 = (torch.randn(F, E, device=DEV) * 0.05).bfloat16()
+    bias2 = torch.randn(F, device=DEV) * 0.1
+    res0 = torch.randn(M, E, device=DEV) * torch.linspace(0.1, 30, M, device=DEV)[:, None]   # rows of very different size
+    eps = 1e-5
+
+    r_sep = res0.clone()
+    h_sep = ops.linear_add_rmsnorm(a, w, r_sep, nw, eps, torch.bfloat16)
+    assert isinstance(h_sep, torch.Tensor)
+    r_fold = res0.clone()
+    h = ops.linear_add_rmsnorm(a, w, r_fold, nw, eps, torch.bfloat16, defer=True)
+    assert isinstance(h, UnscaledRows) and h.shape == (M, E)
+    assert torch.equal(r_fold, r_sep)
+    x = r_fold.double()
+    assert rel(h.sumsq[:, :M].sum(0), (x * x).sum(1)) < 1e-5
+    want_h = x * torch.rsqrt((x * x).mean(1, keepdim=True) + eps) * nw.double()
+    y = ops.linear(h, w2, bias=bias2, out_dtype=torch.float32)
+    y_sep = ops.linear(h_sep, w2, bias=bias2, out_dtype=torch.float32)
+    want = want_h @ w2.double().T + bias2.double()
+    # (either way the normed rows are rounded to bfloat16 once, so the errors are alike)
+    assert rel(y, want) < 6e-3 and rel(y_sep, want) < 6e-3
+    pw2 = ops.pack_weight(w2)
+    assert torch.equal(ops.linear(h, pw2, bias=bias2, out_dtype=torch.float32), y)
+    if F % 32 == 0:
+        g = want_h @ w2.double().T
+        got = ops.linear_swiglu(h, ops.pack_weight(w2, gated=True))
+        assert rel(got, g[:, :F // 2] / (1 + torch.exp(-g[:, :F // 2])) * g[:, F // 2:]) < 8e-3
+    # a chain: the second product adds into the residual and hands on to a third
+    w3 = (torch.randn(E, F, device=DEV) * 0.05).bfloat16()
+    h2 = ops.linear_add_rmsnorm(ops.linear(h, w2), w3, r_fold, nw, eps, torch.bfloat16, defer=True)
+    r2 = r_sep.clone()
+    ops.linear(ops.linear(h_sep, w2), w3, out=r2, accumulate=True)
+    want_r2 = x + (want_h @ w2.double().T) @ w3.double().T
+    assert isinstance(h2, UnscaledRows) and rel(r_fold, want_r2) < 1e-2
+    assert rel(r2, want_r2) < 1e-2
+    # a row's result does not depend on the rows beside it
+    if M > 1:
+        r1 = res0[M - 1:].clone()
+        h1 = ops.linear_add_rmsnorm(a[M - 1:], w, r1, nw, eps, torch.bfloat16, defer=True)
+        assert torch.equal(r1, r_sep[M - 1:]) and torch.equal(h1.data, h.data[M - 1:])
+        assert torch.equal(ops.linear(h1, w2, bias=bias2, out_dtype=torch.float32), y[M - 1:])
+    # where the folded form is not served, the same call runs the norm's own kernel
+    a17 = (torch.randn(17, K, device=DEV) * 0.5).bfloat16()
+    assert isinstance(ops.linear_add_rmsnorm(a17, w, torch.zeros(17, E, device=DEV), nw, eps, torch.bfloat16, defer=True),
+                      torch.Tensor)
+    with pytest.raises(Exception, match="at most 16|MFMA"):
+        ops.linear(UnscaledRows(torch.zeros(17, E, device=DEV).bfloat16(), h.sumsq, eps), w2)
+
+
 def test_pack_weight_leaves_what_the_mfma_kernels_do_not_take(ops):
     w = torch.randn(40, 20, device=DEV).bfloat16()                      # width no multiple of 8
     assert ops.pack_weight(w) is w

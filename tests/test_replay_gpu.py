@@ -219,3 +219,39 @@ def test_graph_and_eager_decode_agree(models, dtype, tol):
             assert r.graphs.replays >= 25
     mx, mean = logit_error(outs[True], outs[False])
     assert mx <= tol and np.abs(outs[True]).max() > 0, (mx, mean)
+
+
+@pytest.mark.parametrize("which", ["A", "B"])
+def test_decoding_with_norms_folded_into_the_products(models, which):
+    """When few tokens are decoded in bfloat16, the norms between the products run inside the
+    products' kernels.  The norm's own kernel is then launched twice a step (the first layer's
+    first norm and the final norm) instead of 2 x layers + 1 times, and the logits agree with
+    the separate kernels' to bfloat16 rounding and with the plain implementation as before."""
+    from xyntetik_runner_amd.engine.batch import StepEntry
+    from xyntetik_runner_amd.engine.runner import ModelRunner
+    d, cfg, reqs, plens, want = models[which]
+    toks = reqs["r3"]
+    n0 = len(toks) - 12
+    outs, launches = {}, {}
+    for fold in (True, False):
+        r = ModelRunner.from_folder(d, dtype="bfloat16", max_tokens=512, page_size=16, max_requests=4, use_graphs=False)
+        count = [0]
+        plain_norm = r.ops.rmsnorm
+        def counting(*a, _f=plain_norm, _c=count, **k):
+            _c[0] += 1
+            return _f(*a, **k)
+        try:                        # (the kernels' object is shared by every runner of the process)
+            r.ops.fold_norms, r.ops.rmsnorm = fold, counting
+            r.step([StepEntry("p", toks[:n0], []), StepEntry("q", toks[:7], [])])
+            count[0] = 0
+            rows = [r.step([StepEntry("p", [toks[i]], [0]), StepEntry("q", [toks[i - n0 + 7]], [])]).cpu().numpy()
+                    for i in range(n0, len(toks))]
+        finally:
+            r.ops.fold_norms = True
+            del r.ops.rmsnorm       # the instance attribute that hid the method
+        outs[fold], launches[fold] = np.concatenate(rows), count[0] // 12
+    L = cfg["num_hidden_layers"]
+    assert launches == {True: 2, False: 2 * L + 1}
+    for fold in (True, False):
+        mx, mean = logit_error(outs[fold], want["r3"][n0:])
+        assert mx <= TOL["bfloat16"][0] and mean <= TOL["bfloat16"][1], (fold, mx, mean)

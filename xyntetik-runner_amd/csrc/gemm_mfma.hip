@@ -43,6 +43,31 @@ struct GemmArgs {
     int splits;        // > 1: K is cut into this many ranges, each workgroup writes raw sums to `partial`
     int k_per_split;   // columns per range (a multiple of 64)
     float* partial;    // [splits][M][rows of w]
+    // RMSNorm folded into the skinny kernel (all null or zero: off).
+    // Before: `a` holds rows x*weight that are not yet divided by their root mean square; ss_in
+    // [n_ss][16] holds partial sums of x^2 per row, and the product's row t is scaled by
+    // rsqrt(sum_p ss_in[p][t] * ss_inv_width + ss_eps) (exact: the scale is one factor per row).
+    const float* ss_in;
+    int n_ss;
+    float ss_inv_width, ss_eps;
+    // After (with EPI_ACCUM): the updated output row times norm_w goes to xg [M][N], and workgroup
+    // the sums of squares of columns 16p .. 16p+15 of the updated rows go to ss_out[p][16].
+    const void* norm_w;
+    int norm_w_bf16;
+    bf16_t* xg;
+    float* ss_out;
+};
+
+// what a caller passes to fold a norm into a product of at most 16 rows (see GemmArgs)
+struct XrGemmNorm {
+    const float* ss_in;
+    int n_ss;
+    float ss_inv_width, ss_eps;
+    const void* norm_w;
+    int norm_w_bf16;
+    void* xg;
+    float* ss_out;
+    int ss_out_rows;   // in: partial rows that ss_out has room for; out: partial rows written
 };
 
 __device__ inline uint4 ldg16(const bf16_t* p) { return *reinterpret_cast<const uint4*>(p); }
@@ -399,6 +424,21 @@ __global__ __launch_bounds__(64 * KSW) void k_gemm_skinny(GemmArgs g) {
 #pragma unroll
             for (int i = 0; i < MT; ++i) acc[t][r][i] = f32x4{0.f, 0.f, 0.f, 0.f};
 
+    // the first SS_AHEAD partial sums of squares of a folded norm are copied to LDS meanwhile
+    // (no registers are held for them; a wave's copy moves 16 partial rows)
+    constexpr int SS_AHEAD = 256;
+    float* scale_s = red + KSW * NWT * ROWS * MTOK;       // [16 parts][16 rows]
+    float* ss_s = scale_s + 256;                          // [SS_AHEAD][16 rows]
+    if (g.ss_in) {
+        const int chunks = (g.n_ss < SS_AHEAD ? g.n_ss : SS_AHEAD) * 4;      // pieces of 16 bytes
+        const uint32_t ss_lds = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) void*)ss_s;
+        for (int c0 = wave * 64; c0 < chunks; c0 += THREADS) {
+            const int c = c0 + lane;
+            const void* src = c < chunks ? (const void*)((const char*)g.ss_in + (size_t)c * 16) : (const void*)xr_zero_chunk;
+            lds_dma16(src, __builtin_amdgcn_readfirstlane(ss_lds + (uint32_t)c0 * 16));
+        }
+    }
+
     const uint4 zero = make_uint4(0, 0, 0, 0);
     for (int k0 = kbeg; k0 < kend; k0 += 32 * U) {
         uint4 wreg[U][NWT][RT], areg[U][MT];
@@ -441,11 +481,26 @@ __global__ __launch_bounds__(64 * KSW) void k_gemm_skinny(GemmArgs g) {
 #pragma unroll
                 for (int e = 0; e < 4; ++e)
                     red[((wave * NWT + t) * ROWS + r * 16 + lq * 4 + e) * MTOK + i * 16 + l16] = acc[t][r][i][e];
+    // the rows' scales, from the partial sums the producer of `a` left: thread (part, tok) of the
+    // first 256 sums every 16th partial, each thread of the last loop sums the 16 parts of its
+    // row; the order is the same in every instance of this kernel, so a row's scale does not
+    // depend on the batch
+    if (g.ss_in) {
+        wait_vmcnt<0>();
+        __syncthreads();                                  // every wave's copies have landed
+        if (tid < 256) {
+            float s = 0.f;
+            const int n_lds = g.n_ss < SS_AHEAD ? g.n_ss : SS_AHEAD;
+            for (int p = tid >> 4; p < n_lds; p += 16) s += ss_s[p * 16 + (tid & 15)];
+            for (int p = (tid >> 4) + SS_AHEAD; p < g.n_ss; p += 16) s += g.ss_in[p * 16 + (tid & 15)];
+            scale_s[tid] = s;
+        }
+    }
     __syncthreads();
     for (int q = tid; q < ROWS * MTOK; q += THREADS) {
         int col = q % ROWS, tok = q / ROWS;          // consecutive threads write consecutive columns
         int nn = n_base + col;
-        if (tok >= g.M || nn >= g.N) continue;
+        const bool ok = tok < g.M && nn < g.N;
         float v[NWT];
 #pragma unroll
         for (int t = 0; t < NWT; ++t) {
@@ -454,19 +509,48 @@ __global__ __launch_bounds__(64 * KSW) void k_gemm_skinny(GemmArgs g) {
             for (int k = 0; k < KSW; ++k) s += red[((k * NWT + t) * ROWS + col) * MTOK + tok];
             v[t] = s;
         }
+        if (g.ss_in) {
+            float ss = 0.f;
+#pragma unroll
+            for (int p = 0; p < 16; ++p) ss += scale_s[p * 16 + (tok & 15)];
+            const float scale = rsqrtf(ss * g.ss_inv_width + g.ss_eps);
+#pragma unroll
+            for (int t = 0; t < NWT; ++t) v[t] *= scale;
+        }
         if (SWIGLU) {
-            float bg = g.bias ? g.bias[nn] : 0.f, bu = g.bias ? g.bias[g.N + nn] : 0.f;
-            store_out(g, tok, nn, silu_f(v[0] + bg) * (v[NWT - 1] + bu));
-        } else {
+            if (ok) {
+                float bg = g.bias ? g.bias[nn] : 0.f, bu = g.bias ? g.bias[g.N + nn] : 0.f;
+                store_out(g, tok, nn, silu_f(v[0] + bg) * (v[NWT - 1] + bu));
+            }
+        } else if (g.xg) {
+            // the rows of the residual stream after this product, their weighted copy for the next
+            // product, and the sums of their squares over each 16 columns (16 lanes side by side)
+            float xn = 0.f;
+            if (ok) {
+                float* p = (float*)g.out + (size_t)tok * g.ldo + nn;
+                xn = *p + v[0] + (g.bias ? g.bias[nn] : 0.f);
+                *p = xn;
+                float nw = g.norm_w_bf16 ? bf16_to_f32(((const bf16_t*)g.norm_w)[nn]) : ((const float*)g.norm_w)[nn];
+                g.xg[(size_t)tok * g.N + nn] = f32_to_bf16(xn * nw);
+            }
+            float sq = xn * xn;
+#pragma unroll
+            for (int o = 8; o > 0; o >>= 1) sq += __shfl_xor(sq, o);
+            const int part = blockIdx.x * RT + (col >> 4);
+            if ((col & 15) == 0 && tok < 16 && part * 16 < g.N) g.ss_out[part * 16 + tok] = sq;
+        } else if (ok) {
             store_out(g, tok, nn, v[0] + (g.bias ? g.bias[nn] : 0.f));
         }
     }
 }
 
+// returns the number of workgroups, or an error (< 0)
+static inline int rc_of(int launched) { return launched < 0 ? launched : XR_OK; }
+
 template <int MT, int RT, int KSW, int U, bool SW, bool NT = false>
 static int launch_skinny(const GemmArgs& g, hipStream_t stream) {
     constexpr int NWT = SW ? 2 : 1;
-    size_t smem = (size_t)KSW * NWT * RT * 16 * MT * 16 * 4;
+    size_t smem = (size_t)KSW * NWT * RT * 16 * MT * 16 * 4 + 256 * 4 + 256 * 64;    // the sums of the waves, 256 partial scales, 256 rows of partial sums
     static bool attr_set = false;
     if (!attr_set) {
         hipError_t e = hipFuncSetAttribute((const void*)k_gemm_skinny<MT, RT, KSW, U, SW, NT>,
@@ -481,7 +565,7 @@ static int launch_skinny(const GemmArgs& g, hipStream_t stream) {
     unsigned blocks = (unsigned)((g.N + 16 * RT - 1) / (16 * RT));
     k_gemm_skinny<MT, RT, KSW, U, SW, NT><<<blocks, 64 * KSW, smem, stream>>>(g);
     XR_CHECK_LAUNCH("gemm_skinny");
-    return XR_OK;
+    return (int)blocks;
 }
 
 // ------------------------------------------------------------------------------ packing
@@ -518,7 +602,7 @@ extern "C" int xr_pack_weight(void* dst, const void* src, int N, int K, hipStrea
 // workspace (may be null): room for split products, workspace_bytes long; without it K is not split.
 extern "C" int xr_gemm_bf16(void* out, const void* a, const void* w, const float* bias, int M, int N, int K,
                             int lda, int ldo, int out_dtype, int epi, int variant, int w_packed, float* workspace,
-                            size_t workspace_bytes, hipStream_t stream) {
+                            size_t workspace_bytes, XrGemmNorm* norm, hipStream_t stream) {
     XR_REQUIRE(M >= 0 && N > 0 && K > 0, "gemm: bad sizes M=%d N=%d K=%d", M, N, K);
     XR_REQUIRE(lda >= K && ldo >= N, "gemm: row strides lda=%d ldo=%d are shorter than K=%d N=%d", lda, ldo, K, N);
     XR_REQUIRE(K % 8 == 0 && lda % 8 == 0, "gemm: the MFMA kernels need K (%d) and the row stride (%d) to be multiples of 8", K, lda);
@@ -532,6 +616,20 @@ extern "C" int xr_gemm_bf16(void* out, const void* a, const void* w, const float
     g.a = (const bf16_t*)a; g.w = (const bf16_t*)w; g.w_packed = w_packed ? 1 : 0; g.bias = bias; g.out = out;
     g.M = M; g.N = N; g.K = K; g.lda = lda; g.ldo = ldo; g.out_bf16 = out_dtype == XR_BF16; g.epi = epi;
     g.m_fast = 0; g.splits = 1; g.k_per_split = 0; g.partial = workspace;
+    g.ss_in = nullptr; g.n_ss = 0; g.ss_inv_width = 0.f; g.ss_eps = 0.f;
+    g.norm_w = nullptr; g.norm_w_bf16 = 0; g.xg = nullptr; g.ss_out = nullptr;
+    if (norm) {
+        XR_REQUIRE(M <= 16 && variant == 0, "gemm: a norm is folded only into products of at most 16 rows, got %d", M);
+        if (norm->ss_in) {
+            XR_REQUIRE(norm->n_ss > 0 && norm->ss_inv_width > 0.f, "gemm: bad partial sums of squares (%d of them)", norm->n_ss);
+            g.ss_in = norm->ss_in; g.n_ss = norm->n_ss; g.ss_inv_width = norm->ss_inv_width; g.ss_eps = norm->ss_eps;
+        }
+        if (norm->xg) {
+            XR_REQUIRE(epi == EPI_ACCUM && norm->norm_w && norm->ss_out, "gemm: the norm after a product needs the accumulating epilogue, a weight and room for the sums");
+            XR_REQUIRE(norm->ss_out_rows >= (N + 15) / 16, "gemm: room for %d partial sums of squares, %d needed", norm->ss_out_rows, (N + 15) / 16);
+            g.norm_w = norm->norm_w; g.norm_w_bf16 = norm->norm_w_bf16; g.xg = (bf16_t*)norm->xg; g.ss_out = norm->ss_out;
+        }
+    }
     if (variant >= 1000) { g.m_fast = 1; variant -= 1000; }
     const bool sw = epi == EPI_SWIGLU;
     const int w_rows = epi == EPI_SWIGLU ? 2 * N : N;
@@ -578,16 +676,20 @@ extern "C" int xr_gemm_bf16(void* out, const void* a, const void* w, const float
         if (M <= 16) {
             // measured on MI355X with packed weights at M = 1, 8 and 16 (waves per workgroup, loads
             // per batch): the output head, q/k/v, the down product, the output product
-            if (sw) return launch_skinny<1, 1, 8, 8, true>(g, stream);
-            if (N >= 65536) return M <= 8 ? launch_skinny<1, 1, 8, 8, false>(g, stream) : launch_skinny<1, 2, 4, 8, false>(g, stream);
-            if (N > 4096 && K <= 8192) return M <= 8 ? launch_skinny<1, 1, 4, 8, false>(g, stream) : launch_skinny<1, 2, 4, 8, false>(g, stream);
-            return launch_skinny<1, 1, 8, 4, false>(g, stream);
+            int blocks;
+            if (sw) blocks = launch_skinny<1, 1, 8, 8, true>(g, stream);
+            else if (N >= 65536) blocks = M <= 8 ? launch_skinny<1, 1, 8, 8, false>(g, stream) : launch_skinny<1, 2, 4, 8, false>(g, stream);
+            else if (N > 4096 && K <= 8192) blocks = M <= 8 ? launch_skinny<1, 1, 4, 8, false>(g, stream) : launch_skinny<1, 2, 4, 8, false>(g, stream);
+            else blocks = launch_skinny<1, 1, 8, 4, false>(g, stream);
+            if (blocks < 0) return blocks;
+            if (norm) norm->ss_out_rows = (N + 15) / 16;
+            return XR_OK;
         }
-        if (M <= 32) return sw ? launch_skinny<2, 1, 16, 8, true>(g, stream) : launch_skinny<2, 1, 16, 8, false>(g, stream);
-        return sw ? launch_skinny<4, 2, 8, 4, true>(g, stream) : launch_skinny<4, 2, 8, 4, false>(g, stream);
+        if (M <= 32) return rc_of(sw ? launch_skinny<2, 1, 16, 8, true>(g, stream) : launch_skinny<2, 1, 16, 8, false>(g, stream));
+        return rc_of(sw ? launch_skinny<4, 2, 8, 4, true>(g, stream) : launch_skinny<4, 2, 8, 4, false>(g, stream));
     }
 #ifdef XR_GEMM_SWEEP
-#define SK(id, MT, RT, KSW, U, NT) if (variant == id) return sw ? launch_skinny<MT, RT, KSW, U, true, NT>(g, stream) : launch_skinny<MT, RT, KSW, U, false, NT>(g, stream);
+#define SK(id, MT, RT, KSW, U, NT) if (variant == id) return rc_of(sw ? launch_skinny<MT, RT, KSW, U, true, NT>(g, stream) : launch_skinny<MT, RT, KSW, U, false, NT>(g, stream));
     SK(100, 1, 1, 16, 8, false) SK(101, 1, 1, 8, 8, false) SK(102, 1, 1, 8, 16, false) SK(103, 1, 1, 4, 16, false)
     SK(104, 1, 1, 4, 8, false) SK(105, 1, 2, 8, 8, false) SK(106, 1, 2, 4, 8, false) SK(107, 1, 1, 16, 4, false)
     SK(108, 1, 1, 16, 8, true) SK(109, 1, 1, 8, 8, true) SK(110, 1, 1, 8, 16, true) SK(111, 1, 2, 8, 8, true)

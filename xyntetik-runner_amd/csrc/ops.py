@@ -42,7 +42,7 @@ _PROTOS = {
     "xr_fill_rows": [_p, _p, _i, _sz, _u32, _p],
     "xr_convert": [_p, _p, _sz, _i, _i, _p],
     "xr_gemm_ref": [_p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _p],
-    "xr_gemm_bf16": [_p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _i, _p, _sz, _p],
+    "xr_gemm_bf16": [_p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _i, _p, _sz, _p, _p],
     "xr_pack_weight": [_p, _p, _i, _i, _p],
     "xr_attention_ref": [_p, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _f, _i, _i, _p],
     "xr_sample": [_p, _p, _i, _i, _i, _p, _p, _p, _p, _p, _p, _p, _p, _i, _p, _i, _p, _p],
@@ -79,6 +79,38 @@ class PackedWeight:
         return self.data.device
 
 
+class UnscaledRows:
+    """The rows of an RMSNorm that still lack their division by the root mean square:
+    ``data [M, E]`` (bfloat16) holds ``x * weight``, ``sumsq [P, 16]`` partial sums of ``x^2`` per
+    row (row t's sum is ``sumsq[:, t].sum()``), so the norm's row t is
+    ``data[t] * rsqrt(sumsq[:, t].sum() / E + eps)``.  As that factor is one number a row, a
+    product ``rows @ w^T`` may apply it to its result instead: ``Ops.linear`` and
+    ``Ops.linear_swiglu`` take this in place of the rows.  Made by ``Ops.linear_add_rmsnorm``."""
+
+    MAX_ROWS = 16
+
+    def __init__(self, data: torch.Tensor, sumsq: torch.Tensor, eps: float):
+        self.data, self.sumsq, self.eps = data, sumsq, eps
+
+    @property
+    def shape(self):
+        return self.data.shape
+
+    @property
+    def dtype(self):
+        return self.data.dtype
+
+    @property
+    def device(self):
+        return self.data.device
+
+
+class _GemmNorm(C.Structure):
+    """XrGemmNorm of the library."""
+    _fields_ = [("ss_in", _p), ("n_ss", _i), ("ss_inv_width", _f), ("ss_eps", _f), ("norm_w", _p),
+                ("norm_w_bf16", _i), ("xg", _p), ("ss_out", _p), ("ss_out_rows", _i)]
+
+
 class _Lib:
     def __init__(self, path: str, protos: Dict[str, list]):
         self.path = path
@@ -103,6 +135,7 @@ class Ops:
         self.lib = lib
         self._attn_libs: Dict[int, object] = {}
         self.use_mfma = True
+        self.fold_norms = True      # False: linear_add_rmsnorm always runs the norm's own kernel
 
     # -- checks -----------------------------------------------------------------
     @staticmethod
@@ -215,7 +248,7 @@ class Ops:
 
     def linear(self, a: torch.Tensor, w, bias: Optional[torch.Tensor] = None,
                out_dtype: Optional[torch.dtype] = None, out: Optional[torch.Tensor] = None,
-               accumulate: bool = False, variant: int = 0) -> torch.Tensor:
+               accumulate: bool = False, variant: int = 0, _then: Optional[_GemmNorm] = None) -> torch.Tensor:
         """``a [M, K] @ w [N, K]^T (+ bias)``; with ``accumulate`` added into 32-bit ``out``.
 
         bfloat16 operands run on the matrix cores (32-bit accumulation); float32 operands, and
@@ -224,6 +257,7 @@ class Ops:
         """
         packed = isinstance(w, PackedWeight)
         wt = w.data if packed else w
+        norm, a = self._norm_before(a, _then)
         self._dev(a, wt, bias, out)
         if a.dim() != 2 or len(w.shape) != 2 or a.shape[1] != w.shape[1]:
             raise KernelError(f"linear: shapes {tuple(a.shape)} x {tuple(w.shape)}^T do not fit")
@@ -246,8 +280,11 @@ class Ops:
             self.lib.check(self.lib.xr_gemm_bf16(out.data_ptr(), a.data_ptr(), wt.data_ptr(), _ptr(bias), M, N, K,
                                                  a.stride(0), out.stride(0), dtype_code(out.dtype),
                                                  1 if accumulate else 0, variant, 1 if packed else 0,
-                                                 *self._gemm_workspace(a.device), _stream()))
+                                                 *self._gemm_workspace(a.device),
+                                                 C.addressof(norm) if norm is not None else None, _stream()))
             return out
+        if norm is not None:
+            raise KernelError("linear: rows that still lack their norm's scale need the MFMA kernels")
         if packed:
             raise KernelError("linear: a packed weight needs bfloat16 rows that are 16-byte aligned")
         self.lib.check(self.lib.xr_gemm_ref(out.data_ptr(), a.data_ptr(), w.data_ptr(), _ptr(bias), M, N, K,
@@ -255,12 +292,52 @@ class Ops:
                                             dtype_code(out.dtype), 1 if accumulate else 0, _stream()))
         return out
 
+    @staticmethod
+    def _norm_before(a, then: Optional[_GemmNorm]):
+        """(what the library needs to know about a norm folded into this product, the rows)"""
+        if not isinstance(a, UnscaledRows):
+            return then, a
+        if a.data.shape[0] > UnscaledRows.MAX_ROWS:
+            raise KernelError(f"a product takes at most {UnscaledRows.MAX_ROWS} rows that still lack their norm's scale")
+        norm = then if then is not None else _GemmNorm()
+        norm.ss_in, norm.n_ss = a.sumsq.data_ptr(), a.sumsq.shape[0]
+        norm.ss_inv_width, norm.ss_eps = 1.0 / a.data.shape[1], float(a.eps)
+        return norm, a.data
+
+    def linear_add_rmsnorm(self, a, w, residual: torch.Tensor, norm_weight: Optional[torch.Tensor], eps: float,
+                           out_dtype: torch.dtype, bias: Optional[torch.Tensor] = None, defer: bool = False):
+        """``residual += a @ w^T (+ bias)``, then the RMSNorm of the updated rows.
+
+        With ``defer`` the caller says that what reads the result is a ``linear`` or
+        ``linear_swiglu``: for at most 16 bfloat16 rows the product's kernel then also writes the
+        weighted rows and their partial sums of squares, and an ``UnscaledRows`` comes back, whose
+        scale the next product applies; two launches of the norm's own kernel are saved.  In
+        every other case the norm's kernel runs and a tensor comes back."""
+        wt = w.data if isinstance(w, PackedWeight) else w
+        rows = a.data if isinstance(a, UnscaledRows) else a
+        M, N = rows.shape[0], w.shape[0]
+        if (defer and self.fold_norms and M <= UnscaledRows.MAX_ROWS and out_dtype == torch.bfloat16 and norm_weight is not None
+                and N % 8 == 0 and norm_weight.numel() == N and norm_weight.is_contiguous()
+                and residual.dtype == torch.float32 and self._mfma_ok(rows, wt)):
+            self._dev(norm_weight)
+            then = _GemmNorm()
+            xg = torch.empty((M, N), dtype=torch.bfloat16, device=rows.device)
+            parts = -(-N // 16)
+            sumsq = torch.empty((parts, 16), dtype=torch.float32, device=rows.device)
+            then.norm_w, then.norm_w_bf16 = norm_weight.data_ptr(), dtype_code(norm_weight.dtype)
+            then.xg, then.ss_out, then.ss_out_rows = xg.data_ptr(), sumsq.data_ptr(), parts
+            self.linear(a, w, bias=bias, out=residual, accumulate=True, _then=then)
+            return UnscaledRows(xg, sumsq[:then.ss_out_rows], eps)
+        self.linear(a, w, bias=bias, out=residual, accumulate=True)
+        return self.rmsnorm(residual, norm_weight, eps, out_dtype)
+
     def linear_swiglu(self, a: torch.Tensor, w, bias: Optional[torch.Tensor] = None,
                       variant: int = 0) -> torch.Tensor:
         """``silu(a @ w[:F]^T) * (a @ w[F:]^T)`` for ``w [2F, K]`` = gate rows then up rows
         (a matrix, or a ``PackedWeight`` made with ``gated=True``)."""
         packed = isinstance(w, PackedWeight)
         wt = w.data if packed else w
+        norm, a = self._norm_before(a, None)
         F = w.shape[0] // 2
         if w.shape[0] % 2:
             raise KernelError("linear_swiglu: the weight must have an even number of rows")
@@ -275,8 +352,11 @@ class Ops:
             out = torch.empty((M, F), dtype=a.dtype, device=a.device)
             self.lib.check(self.lib.xr_gemm_bf16(out.data_ptr(), a.data_ptr(), wt.data_ptr(), _ptr(bias), M, F, K,
                                                  a.stride(0), F, dtype_code(out.dtype), 2, variant,
-                                                 1 if packed else 0, *self._gemm_workspace(a.device), _stream()))
+                                                 1 if packed else 0, *self._gemm_workspace(a.device),
+                                                 C.addressof(norm) if norm is not None else None, _stream()))
             return out
+        if norm is not None:
+            raise KernelError("linear_swiglu: rows that still lack their norm's scale need the MFMA kernels")
         if packed:
             raise KernelError("linear_swiglu: a packed weight needs bfloat16 rows that are 16-byte aligned")
         return self.silu_mul(self.linear(a, w, bias=bias))

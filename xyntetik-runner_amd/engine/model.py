@@ -83,8 +83,16 @@ class Model:
     def forward(self, ctx, caches) -> torch.Tensor:
         """Run the step's tokens through every layer; returns the residual stream ``[T, E]`` (32-bit)."""
         x = self.embedding.forward(ctx, ctx.token_ids)
-        for i, step in enumerate(self.spec.order):
-            self.blocks[step.layer].forward(ctx, caches[i], x)
+        order = self.spec.order
+        h = None            # the result of the next block's first norm, if the block before made it
+        for i, step in enumerate(order):
+            block = self.blocks[step.layer]
+            if block.chained:
+                after = self.blocks[order[i + 1].layer].entry_norm() if i + 1 < len(order) else None
+                h = block.forward(ctx, caches[i], x, h=h, after=after)
+            else:
+                block.forward(ctx, caches[i], x)
+                h = None
         return x
 
     def logits(self, ctx, x: torch.Tensor, rows: torch.Tensor) -> torch.Tensor:

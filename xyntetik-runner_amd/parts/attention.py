@@ -22,6 +22,8 @@ from .base import KVSpec, Mixer, ParamSpec, make_part, register_mixer
 
 
 class PagedAttention(Mixer):
+    takes_unscaled_rows = True
+
     def __init__(self, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int,
                  position=None, window: Optional[int] = None, scale: Optional[float] = None,
                  bias: bool = False, out_bias: Optional[bool] = None, kv_shared: bool = False,
@@ -113,6 +115,13 @@ class PagedAttention(Mixer):
 
     def forward_add(self, ctx, cache, h, residual) -> None:
         self.rt.ops.linear(self._attend(ctx, cache, h), self.w_out, bias=self.b_out, out=residual, accumulate=True)
+
+    def forward_add_norm(self, ctx, cache, h, residual, norm, defer=False):
+        fold = norm.fold()
+        if fold is None:
+            return super().forward_add_norm(ctx, cache, h, residual, norm, defer)
+        return self.rt.ops.linear_add_rmsnorm(self._attend(ctx, cache, h), self.w_out, residual, fold[0], fold[1],
+                                              self.rt.dtype, bias=self.b_out, defer=defer)
 
 
 register_mixer("paged_attention", PagedAttention)

@@ -9,7 +9,8 @@ Families and what each must offer:
 
 * ``Norm``: ``forward(ctx, x, rows=None) -> h``.  ``x`` is the 32-bit residual
   stream ``[T, E]``; ``h`` is in the compute dtype.  ``rows`` (device int32)
-  selects rows of ``x``.
+  selects rows of ``x``.  ``fold()`` may return ``(weight, eps)`` if the norm is an
+  RMSNorm that the product before it may compute (see below).
 * ``PositionEncoding``: ``rotary()`` returns the parameters of a rotation that
   the attention kernels apply themselves, or ``None``; then ``apply(ctx, q, k)``
   is called on the 32-bit queries and keys before they are cached.
@@ -20,6 +21,18 @@ Families and what each must offer:
   overrides it).
 * ``FeedForward``: ``forward(ctx, h) -> y`` and ``forward_add(ctx, h, residual)``.
 * ``Block``: the arrangement; ``forward(ctx, cache, x)`` updates ``x`` in place.
+
+Optional, for fewer kernels when a few tokens are decoded: a mixer or feed-forward
+may override ``forward_add_norm(..., residual, norm, defer)``, which adds into the
+residual stream and returns ``norm`` of the result, so that its last product can do
+both (``Ops.linear_add_rmsnorm``).  With ``defer`` the result may be an
+``UnscaledRows`` (the rows still lack the division by their root mean square, which
+the next product applies to its own result); a caller sets ``defer`` only if the part
+that reads the result has ``takes_unscaled_rows`` set, which says that it hands ``h``
+to ``Ops.linear`` or ``Ops.linear_swiglu`` and reads nothing else of it than its
+``shape``, ``dtype`` and ``device``.  A block with ``chained`` set takes the result of
+its first norm from the block before it and makes the next block's
+(``entry_norm()``); every default does the plain thing.
 """
 from __future__ import annotations
 
@@ -86,6 +99,11 @@ class Norm(Part):
     def forward(self, ctx, x: torch.Tensor, rows: Optional[torch.Tensor] = None) -> torch.Tensor:
         raise NotImplementedError
 
+    def fold(self) -> Optional[Tuple[torch.Tensor, float]]:
+        """``(weight, eps)`` if this is ``x / sqrt(mean(x^2) + eps) * weight``, which the product
+        that writes ``x`` may compute in its own kernel; None for any other norm."""
+        return None
+
 
 @dataclass(frozen=True)
 class RotaryParams:
@@ -115,16 +133,32 @@ class Mixer(Part):
     def forward(self, ctx, cache, h: torch.Tensor) -> torch.Tensor:
         raise NotImplementedError
 
+    #: True if ``h`` may be an ``UnscaledRows`` (it only goes into ``Ops.linear``)
+    takes_unscaled_rows = False
+
     def forward_add(self, ctx, cache, h: torch.Tensor, residual: torch.Tensor) -> None:
         ctx.ops.add_(residual, self.forward(ctx, cache, h))
+
+    def forward_add_norm(self, ctx, cache, h, residual: torch.Tensor, norm: Norm, defer: bool = False):
+        """``forward_add``, then ``norm`` of the updated residual stream."""
+        self.forward_add(ctx, cache, h, residual)
+        return norm.forward(ctx, residual)
 
 
 class FeedForward(Part):
     def forward(self, ctx, h: torch.Tensor) -> torch.Tensor:
         raise NotImplementedError
 
+    #: True if ``h`` may be an ``UnscaledRows`` (it only goes into ``Ops.linear`` or ``Ops.linear_swiglu``)
+    takes_unscaled_rows = False
+
     def forward_add(self, ctx, h: torch.Tensor, residual: torch.Tensor) -> None:
         ctx.ops.add_(residual, self.forward(ctx, h))
+
+    def forward_add_norm(self, ctx, h, residual: torch.Tensor, norm: Norm, defer: bool = False):
+        """``forward_add``, then ``norm`` of the updated residual stream."""
+        self.forward_add(ctx, h, residual)
+        return norm.forward(ctx, residual)
 
 
 class Block:
@@ -139,6 +173,16 @@ class Block:
     def parts(self):
         return {"mixer_norm": self.mixer_norm, "mixer": self.mixer,
                 "feed_forward_norm": self.feed_forward_norm, "feed_forward": self.feed_forward}
+
+    #: True if ``forward`` also takes ``h`` (the result of this block's first norm, made by the
+    #: block before) and ``after`` (the next block's ``entry_norm()``), and returns the next
+    #: block's ``h`` or None
+    chained = False
+
+    def entry_norm(self) -> Optional[Tuple[Norm, bool]]:
+        """(the norm this block applies to the residual stream first, whether what reads its
+        result takes ``UnscaledRows``), if the block before may compute it; else None."""
+        return None
 
     def forward(self, ctx, cache, x: torch.Tensor) -> None:
         raise NotImplementedError

@@ -15,6 +15,8 @@ from .base import FeedForward, ParamSpec, register_feed_forward
 
 
 class GatedMLP(FeedForward):
+    takes_unscaled_rows = True
+
     def __init__(self, hidden_size: int, intermediate_size: int, activation: str = "silu", bias: bool = False,
                  gate_name: str = "gate_proj", up_name: str = "up_proj", down_name: str = "down_proj"):
         if activation != "silu":
@@ -54,6 +56,13 @@ class GatedMLP(FeedForward):
 
     def forward_add(self, ctx, h, residual) -> None:
         self.rt.ops.linear(self._hidden(ctx, h), self.w_down, bias=self.b_down, out=residual, accumulate=True)
+
+    def forward_add_norm(self, ctx, h, residual, norm, defer=False):
+        fold = norm.fold()
+        if fold is None:
+            return super().forward_add_norm(ctx, h, residual, norm, defer)
+        return self.rt.ops.linear_add_rmsnorm(self._hidden(ctx, h), self.w_down, residual, fold[0], fold[1],
+                                              self.rt.dtype, bias=self.b_down, defer=defer)
 
 
 register_feed_forward("gated_mlp", GatedMLP)

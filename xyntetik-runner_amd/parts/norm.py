@@ -28,5 +28,8 @@ class RMSNorm(Norm):
     def forward(self, ctx, x, rows=None):
         return self.rt.ops.rmsnorm(x, self.weight, self.eps, self.rt.dtype, rows=rows)
 
+    def fold(self):
+        return (self.weight, self.eps) if self.weight is not None else None
+
 
 register_norm("rmsnorm", RMSNorm)
