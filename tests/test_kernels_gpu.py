@@ -349,6 +349,68 @@ def test_rope_kv_write(ops, dt, H, Hk, D, rot, inter, ps, starts, q_lens):
         assert torch.equal(q_out.cpu().reshape(T, H, D)[..., rot:], qkv[:, :Q].cpu().reshape(T, H, D)[..., rot:].to(DT[dt]))
 
 
+@pytest.mark.parametrize("dt", ["float32", "bfloat16"])
+@pytest.mark.parametrize("H,Hk,D,rot,inter", [(4, 2, 16, 16, False), (3, 1, 48, 32, False), (6, 3, 80, 80, True),
+                                               (8, 8, 128, 64, True), (5, 1, 128, 128, False), (2, 2, 32, 0, False)])
+@pytest.mark.parametrize("ps,starts,q_lens", [(16, [0, 13, 40], [9, 3, 1]), (64, [70], [1]), (8, [2, 9, 100, 7], [5, 6, 1, 4]),
+                                              (16, [3, 0], [30, 8])])
+@pytest.mark.parametrize("bias", [False, True])
+def test_projection_with_rotation_and_cache_write(ops, dt, H, Hk, D, rot, inter, ps, starts, q_lens, bias):
+    """q, k and v from one product, rotated and cached.  Up to 16 bfloat16 rows the product's own
+    kernel does all of it (with the weight's rows in paired order where a pair is (j, j + rot/2));
+    more rows, or 32-bit, run the product and the rotation kernel.  Both against float64 from
+    the weights in their natural order; and the two bfloat16 ways against each other."""
+    from xyntetik_runner_amd.csrc.ops import paired_order
+    torch.manual_seed(H * 100 + D + ps)
+    tables, n_pages = scatter_pages([s + n for s, n in zip(starts, q_lens)], ps, 2)
+    ctx = FakeCtx(starts, q_lens, tables, ps)
+    T, E, Q, K = sum(q_lens), 72, H * D, Hk * D
+    h = (torch.randn(T, E, device=DEV) * 0.5).to(DT[dt])
+    w = (torch.randn(Q + 2 * K, E, device=DEV) * 0.2).to(DT[dt])
+    b = torch.randn(Q + 2 * K, device=DEV) * 0.3 if bias else None
+    inv = (10000.0 ** (-torch.arange(rot // 2, dtype=torch.float64) * 2 / rot)).float().to(DEV) if rot else None
+    paired = rot > 0 and not inter and rot % 16 == 0
+    wp, bp = w, b
+    if paired:
+        order = paired_order(D, rot)
+        assert sorted(order) == list(range(D))
+        index = torch.tensor([hd * D + c for hd in range(H + Hk) for c in order] + list(range(Q + K, Q + 2 * K)), device=DEV)
+        wp, bp = w.index_select(0, index), (b.index_select(0, index) if bias else None)
+    proj = h.double() @ w.double().T + (b.double() if bias else 0)
+    pos = ctx.positions.cpu()
+    rotate = (lambda x: ref_rope(x, pos, inv.cpu(), inter)) if rot else (lambda x: x.double())
+    want_q = rotate(proj[:, :Q].cpu().reshape(T, H, D))
+    want_k = rotate(proj[:, Q:Q + K].cpu().reshape(T, Hk, D))
+    want_v = proj[:, Q + K:].cpu().reshape(T, Hk, D)
+    tol = 1e-5 if dt == "float32" else 6e-3
+    results = []
+    for fuse in (True, False):
+        kc = torch.full((n_pages, Hk, ps, D), float("nan"), device=DEV, dtype=DT[dt])
+        vc = torch.full((n_pages, Hk, D, ps), float("nan"), device=DEV, dtype=DT[dt])
+        ops.fuse_rope = fuse
+        try:
+            q = ops.project_rope_kv_write(h, ops.pack_weight(wp), bp, kc, vc, ctx.positions, ctx.req_of_token,
+                                          ctx.block_table(0), inv, H, Hk, D, rot, inter, 1.0, ps, paired=paired)
+        finally:
+            ops.fuse_rope = True
+        assert q.dtype == DT[dt] and rel(q.cpu().reshape(T, H, D), want_q) < tol
+        written = torch.zeros(n_pages, ps, dtype=torch.bool)
+        t = 0
+        for r, (s, n) in enumerate(zip(starts, q_lens)):
+            for p in range(s, s + n):
+                page, off = tables[r][p // ps], p % ps
+                assert rel(kc[page, :, off, :].cpu(), want_k[t]) < tol
+                assert rel(vc[page, :, :, off].cpu(), want_v[t]) < tol
+                written[page, off] = True
+                t += 1
+        assert torch.isnan(kc.float().cpu().permute(0, 2, 1, 3)[~written]).all()      # nothing else was touched
+        assert torch.isnan(vc.float().cpu().permute(0, 3, 1, 2)[~written]).all()
+        results.append((q.float().cpu(), torch.nan_to_num(kc.float().cpu()), torch.nan_to_num(vc.float().cpu())))
+    if dt == "bfloat16":
+        for one, two in zip(*results):          # the same sums and formulas: at most a rounding apart
+            assert rel(one, two) < 4e-3
+
+
 def ref_attention(q, k_seq, v_seq, starts, q_lens, scale, window):
     """float64 attention per request; k_seq/v_seq[b]: [len, Hk, D] of the whole request."""
     outs = []

@@ -156,6 +156,7 @@ struct RopeArgs {
     float mscale;
     int page_shift, page_mask, page_size;
     int heads_per_block;
+    int paired;             // queries and keys come in paired order (paired_col)
 };
 
 // 8 values of one channel at 8 consecutive positions of a page: 16 or 32 bytes side by side in
@@ -199,7 +200,8 @@ __global__ __launch_bounds__(256) void k_rope_kv_write(RopeArgs a) {
             for (int j = lane; j < half; j += 64) {
                 const int i0 = a.interleaved ? 2 * j : j;
                 const int i1 = a.interleaved ? 2 * j + 1 : j + half;
-                const float x0 = src[i0], x1 = src[i1], c = cs[0][j], sn = cs[1][j];
+                const float x0 = src[a.paired ? paired_col(i0, a.rot) : i0], x1 = src[a.paired ? paired_col(i1, a.rot) : i1];
+                const float c = cs[0][j], sn = cs[1][j];
                 st<T>(dst, i0, x0 * c - x1 * sn);
                 st<T>(dst, i1, x0 * sn + x1 * c);
             }
@@ -216,7 +218,8 @@ __global__ __launch_bounds__(256) void k_rope_kv_write(RopeArgs a) {
         for (int j = lane; j < half; j += 64) {
             const int i0 = a.interleaved ? 2 * j : j;
             const int i1 = a.interleaved ? 2 * j + 1 : j + half;
-            const float x0 = ks[i0], x1 = ks[i1], c = cs[0][j], sn = cs[1][j];
+            const float x0 = ks[a.paired ? paired_col(i0, a.rot) : i0], x1 = ks[a.paired ? paired_col(i1, a.rot) : i1];
+            const float c = cs[0][j], sn = cs[1][j];
             st<T>(kd, i0, x0 * c - x1 * sn);
             st<T>(kd, i1, x0 * sn + x1 * c);
         }
@@ -243,7 +246,7 @@ extern "C" int xr_rope_kv_write(const float* q_in, const float* k_in, const floa
                                 void* q_out, void* k_cache, void* v_cache, const int* positions,
                                 const int* req_of_token, const int* block_table, int table_stride,
                                 const float* inv_freq, int T, int H, int Hk, int D, int rot,
-                                int interleaved, float mscale, int page_size, int dtype,
+                                int interleaved, float mscale, int page_size, int dtype, int paired,
                                 hipStream_t stream) {
     XR_REQUIRE(T >= 0 && H >= 0 && Hk >= 0 && D > 0, "rope_kv_write: bad sizes T=%d H=%d Hk=%d D=%d", T, H, Hk, D);
     XR_REQUIRE(rot >= 0 && rot <= D && (rot % 2) == 0, "rope_kv_write: rotary width %d must be even and at most head_dim %d", rot, D);
@@ -263,6 +266,8 @@ extern "C" int xr_rope_kv_write(const float* q_in, const float* k_in, const floa
     a.T = T; a.H = H; a.Hk = Hk; a.D = D; a.rot = rot; a.interleaved = interleaved; a.mscale = mscale;
     a.page_shift = shift < 0 ? 0 : shift; a.page_mask = page_size - 1; a.page_size = page_size;
     XR_REQUIRE(rot <= 256, "rope_kv_write: rotary width %d exceeds 256", rot);
+    XR_REQUIRE(!paired || (!interleaved && rot % 16 == 0), "rope_kv_write: paired order needs pairs (j, j + width/2) and a rotary width (%d) that is a multiple of 16", rot);
+    a.paired = paired ? 1 : 0;
     // all heads of a token in one workgroup when there are tokens enough to fill the chip, else
     // fewer heads each, down to one a wave
     int groups = (1024 + T - 1) / T;

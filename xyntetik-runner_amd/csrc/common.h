@@ -108,6 +108,16 @@ __device__ inline PageRef page_of(const int* __restrict__ block_table, int table
     return r;
 }
 
+// "Paired order" of a head's channels: where a rotation pairs channel j with j + rot/2, the
+// product that makes queries and keys may have its weight rows ordered so that both lie in
+// one group of 16 columns: channel j < rot/2 at column (j/8)*16 + j%8, its partner 8 further
+// (rot a multiple of 16); channels from rot on stay where they are.
+__host__ __device__ inline int paired_col(int d, int rot) {
+    if (d >= rot) return d;
+    const int half = rot >> 1, hi = d >= half ? 1 : 0, j = hi ? d - half : d;
+    return (j >> 3) * 16 + hi * 8 + (j & 7);
+}
+
 static inline int ilog2_exact(int v) {   // -1 if v is not a power of two
     if (v <= 0 || (v & (v - 1))) return -1;
     int s = 0;

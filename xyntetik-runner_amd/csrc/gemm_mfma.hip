@@ -30,6 +30,25 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 #define EPI_ACCUM 1
 #define EPI_SWIGLU 2
 
+// Rotation and cache write in the epilogue of the skinny kernel (on: q_out not null).  The
+// product's columns are [query heads | key heads | value heads], each head D wide; what would
+// be its output row is rotated and stored like k_rope_kv_write does, and nothing else is
+// written.  With pairs (j, j + rot/2) the weight rows must be in paired order (see
+// paired_col in common.h), so that both halves of a pair lie in one group of 16 columns.
+struct RopeFuse {
+    const int* positions;      // [M]
+    const int* req_of_token;   // [M]
+    const int* block_table;    // [requests, table_stride]
+    int table_stride;
+    const float* inv_freq;     // [rot/2] or null
+    int H, Hk, D, rot, interleaved;
+    float mscale;
+    int page_shift, page_mask, page_size;
+    bf16_t* q_out;             // [M, H*D]
+    bf16_t* k_cache;
+    bf16_t* v_cache;
+};
+
 struct GemmArgs {
     const bf16_t* a;   // [M, lda]
     const bf16_t* w;   // [N or 2N, K] row-major, or packed (see k_pack_weight)
@@ -50,12 +69,28 @@ struct GemmArgs {
     const float* ss_in;
     int n_ss;
     float ss_inv_width, ss_eps;
-    // After (with EPI_ACCUM): the updated output row times norm_w goes to xg [M][N], and workgroup
+    // After (with EPI_ACCUM): the updated output row times norm_w goes to xg [M][N], and
     // the sums of squares of columns 16p .. 16p+15 of the updated rows go to ss_out[p][16].
     const void* norm_w;
     int norm_w_bf16;
     bf16_t* xg;
     float* ss_out;
+    RopeFuse rope;     // rotation and cache write in place of the output (on: rope.q_out not null)
+};
+
+// what a caller passes to have the product's row rotated and cached (see RopeFuse)
+struct XrGemmRope {
+    const int* positions;
+    const int* req_of_token;
+    const int* block_table;
+    int table_stride;
+    const float* inv_freq;
+    int H, Hk, D, rot, interleaved;
+    float mscale;
+    int page_size;
+    void* q_out;
+    void* k_cache;
+    void* v_cache;
 };
 
 // what a caller passes to fold a norm into a product of at most 16 rows (see GemmArgs)
@@ -522,6 +557,40 @@ __global__ __launch_bounds__(64 * KSW) void k_gemm_skinny(GemmArgs g) {
                 float bg = g.bias ? g.bias[nn] : 0.f, bu = g.bias ? g.bias[g.N + nn] : 0.f;
                 store_out(g, tok, nn, silu_f(v[0] + bg) * (v[NWT - 1] + bu));
             }
+        } else if (g.rope.q_out) {
+            // queries and keys rotated (the partner of a pair is 8 lanes away, or 1), queries to
+            // their buffer, keys and values to their pages; formulas as in k_rope_kv_write
+            const RopeFuse& rp = g.rope;
+            const float val = v[0] + (ok && g.bias ? g.bias[nn] : 0.f);
+            const float partner = __shfl_xor(val, rp.interleaved ? 1 : 8);
+            if (ok) {
+                const int Q = rp.H * rp.D, KV = rp.Hk * rp.D;
+                const int sec = nn < Q ? 0 : (nn < Q + KV ? 1 : 2);
+                const int rel = nn - (sec == 0 ? 0 : (sec == 1 ? Q : Q + KV));
+                const int hs = rel / rp.D, c = rel - hs * rp.D;
+                const int pos = rp.positions[tok];
+                int d = c;
+                float o = val;
+                if (sec < 2 && c < rp.rot) {
+                    int j, hi;
+                    if (rp.interleaved) { j = c >> 1; hi = c & 1; }
+                    else { hi = (c >> 3) & 1; j = (c >> 4) * 8 + (c & 7); d = j + hi * (rp.rot >> 1); }
+                    const float ang = (float)pos * rp.inv_freq[j];
+                    const float cs = cosf(ang) * rp.mscale, sn = sinf(ang) * rp.mscale;
+                    const float x0 = hi ? partner : val, x1 = hi ? val : partner;
+                    o = hi ? x0 * sn + x1 * cs : x0 * cs - x1 * sn;
+                }
+                if (sec == 0) {
+                    rp.q_out[((size_t)tok * rp.H + hs) * rp.D + d] = f32_to_bf16(o);
+                } else {
+                    const PageRef pr = page_of(rp.block_table, rp.table_stride, rp.req_of_token[tok], pos,
+                                               rp.page_shift, rp.page_mask);
+                    if (sec == 1)
+                        rp.k_cache[(((size_t)pr.page * rp.Hk + hs) * rp.page_size + pr.off) * rp.D + d] = f32_to_bf16(o);
+                    else
+                        rp.v_cache[(((size_t)pr.page * rp.Hk + hs) * rp.D + d) * rp.page_size + pr.off] = f32_to_bf16(o);
+                }
+            }
         } else if (g.xg) {
             // the rows of the residual stream after this product, their weighted copy for the next
             // product, and the sums of their squares over each 16 columns (16 lanes side by side)
@@ -602,7 +671,7 @@ extern "C" int xr_pack_weight(void* dst, const void* src, int N, int K, hipStrea
 // workspace (may be null): room for split products, workspace_bytes long; without it K is not split.
 extern "C" int xr_gemm_bf16(void* out, const void* a, const void* w, const float* bias, int M, int N, int K,
                             int lda, int ldo, int out_dtype, int epi, int variant, int w_packed, float* workspace,
-                            size_t workspace_bytes, XrGemmNorm* norm, hipStream_t stream) {
+                            size_t workspace_bytes, XrGemmNorm* norm, const XrGemmRope* rope, hipStream_t stream) {
     XR_REQUIRE(M >= 0 && N > 0 && K > 0, "gemm: bad sizes M=%d N=%d K=%d", M, N, K);
     XR_REQUIRE(lda >= K && ldo >= N, "gemm: row strides lda=%d ldo=%d are shorter than K=%d N=%d", lda, ldo, K, N);
     XR_REQUIRE(K % 8 == 0 && lda % 8 == 0, "gemm: the MFMA kernels need K (%d) and the row stride (%d) to be multiples of 8", K, lda);
@@ -629,6 +698,27 @@ extern "C" int xr_gemm_bf16(void* out, const void* a, const void* w, const float
             XR_REQUIRE(norm->ss_out_rows >= (N + 15) / 16, "gemm: room for %d partial sums of squares, %d needed", norm->ss_out_rows, (N + 15) / 16);
             g.norm_w = norm->norm_w; g.norm_w_bf16 = norm->norm_w_bf16; g.xg = (bf16_t*)norm->xg; g.ss_out = norm->ss_out;
         }
+    }
+    g.rope.q_out = nullptr;
+    if (rope) {
+        XR_REQUIRE(M <= 16 && variant == 0 && epi == EPI_STORE && !(norm && norm->xg),
+                   "gemm: rotation and cache write are folded only into a plain product of at most 16 rows");
+        XR_REQUIRE(rope->H >= 0 && rope->Hk >= 0 && rope->D > 0 && rope->D % 16 == 0 && N == (rope->H + 2 * rope->Hk) * rope->D,
+                   "gemm: %d columns are not %d query and 2 x %d key/value heads of a size (%d) that is a multiple of 16",
+                   N, rope->H, rope->Hk, rope->D);
+        XR_REQUIRE(rope->rot >= 0 && rope->rot <= rope->D && rope->rot % 2 == 0 && (rope->interleaved || rope->rot % 16 == 0),
+                   "gemm: rotary width %d (head size %d): pairs (j, j + width/2) need a multiple of 16", rope->rot, rope->D);
+        XR_REQUIRE(rope->rot == 0 || rope->inv_freq, "gemm: rotary width %d without a frequency table", rope->rot);
+        const int shift = ilog2_exact(rope->page_size);
+        XR_REQUIRE(rope->Hk == 0 || shift >= 0, "gemm: page size %d is not a power of two", rope->page_size);
+        XR_REQUIRE(rope->positions && rope->q_out && (rope->Hk == 0 || (rope->k_cache && rope->v_cache && rope->block_table && rope->req_of_token)),
+                   "gemm: rotation and cache write with a null operand");
+        g.rope.positions = rope->positions; g.rope.req_of_token = rope->req_of_token; g.rope.block_table = rope->block_table;
+        g.rope.table_stride = rope->table_stride; g.rope.inv_freq = rope->inv_freq;
+        g.rope.H = rope->H; g.rope.Hk = rope->Hk; g.rope.D = rope->D; g.rope.rot = rope->rot; g.rope.interleaved = rope->interleaved;
+        g.rope.mscale = rope->mscale; g.rope.page_shift = shift < 0 ? 0 : shift; g.rope.page_mask = rope->page_size - 1;
+        g.rope.page_size = rope->page_size;
+        g.rope.q_out = (bf16_t*)rope->q_out; g.rope.k_cache = (bf16_t*)rope->k_cache; g.rope.v_cache = (bf16_t*)rope->v_cache;
     }
     if (variant >= 1000) { g.m_fast = 1; variant -= 1000; }
     const bool sw = epi == EPI_SWIGLU;

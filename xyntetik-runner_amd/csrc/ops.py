@@ -36,13 +36,13 @@ _p, _i, _f, _sz, _u32 = C.c_void_p, C.c_int, C.c_float, C.c_size_t, C.c_uint32
 _PROTOS = {
     "xr_embedding": [_p, _p, _p, _i, _i, _i, _f, _i, _p],
     "xr_rmsnorm": [_p, _p, _p, _p, _i, _i, _i, _f, _i, _i, _p],
-    "xr_rope_kv_write": [_p, _p, _p, _i, _p, _p, _p, _p, _p, _p, _i, _p, _i, _i, _i, _i, _i, _i, _f, _i, _i, _p],
+    "xr_rope_kv_write": [_p, _p, _p, _i, _p, _p, _p, _p, _p, _p, _i, _p, _i, _i, _i, _i, _i, _i, _f, _i, _i, _i, _p],
     "xr_silu_mul": [_p, _p, _i, _i, _i, _i, _p],
     "xr_add": [_p, _p, _sz, _i, _p],
     "xr_fill_rows": [_p, _p, _i, _sz, _u32, _p],
     "xr_convert": [_p, _p, _sz, _i, _i, _p],
     "xr_gemm_ref": [_p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _p],
-    "xr_gemm_bf16": [_p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _i, _p, _sz, _p, _p],
+    "xr_gemm_bf16": [_p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _i, _p, _sz, _p, _p, _p],
     "xr_pack_weight": [_p, _p, _i, _i, _p],
     "xr_attention_ref": [_p, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _f, _i, _i, _p],
     "xr_sample": [_p, _p, _i, _i, _i, _p, _p, _p, _p, _p, _p, _p, _p, _i, _p, _i, _p, _p],
@@ -111,6 +111,27 @@ class _GemmNorm(C.Structure):
                 ("norm_w_bf16", _i), ("xg", _p), ("ss_out", _p), ("ss_out_rows", _i)]
 
 
+class _GemmRope(C.Structure):
+    """XrGemmRope of the library."""
+    _fields_ = [("positions", _p), ("req_of_token", _p), ("block_table", _p), ("table_stride", _i),
+                ("inv_freq", _p), ("H", _i), ("Hk", _i), ("D", _i), ("rot", _i), ("interleaved", _i),
+                ("mscale", _f), ("page_size", _i), ("q_out", _p), ("k_cache", _p), ("v_cache", _p)]
+
+
+def paired_order(D: int, rot: int) -> list:
+    """``order[c]`` = the channel of a head that stands at column ``c`` in "paired order": a
+    rotation's pairs ``(j, j + rot/2)`` side by side in groups of 16 columns (8 first halves, then
+    their 8 partners), channels from ``rot`` on in place.  ``rot`` must be a multiple of 16."""
+    if rot % 16 or rot > D:
+        raise ValueError(f"paired order needs a rotary width that is a multiple of 16 and at most {D}, got {rot}")
+    order = list(range(D))
+    half = rot // 2
+    for d in range(rot):
+        hi, j = (1, d - half) if d >= half else (0, d)
+        order[(j // 8) * 16 + hi * 8 + j % 8] = d
+    return order
+
+
 class _Lib:
     def __init__(self, path: str, protos: Dict[str, list]):
         self.path = path
@@ -136,6 +157,7 @@ class Ops:
         self._attn_libs: Dict[int, object] = {}
         self.use_mfma = True
         self.fold_norms = True      # False: linear_add_rmsnorm always runs the norm's own kernel
+        self.fuse_rope = True       # False: project_rope_kv_write always runs two kernels
 
     # -- checks -----------------------------------------------------------------
     @staticmethod
@@ -281,7 +303,7 @@ class Ops:
                                                  a.stride(0), out.stride(0), dtype_code(out.dtype),
                                                  1 if accumulate else 0, variant, 1 if packed else 0,
                                                  *self._gemm_workspace(a.device),
-                                                 C.addressof(norm) if norm is not None else None, _stream()))
+                                                 C.addressof(norm) if norm is not None else None, None, _stream()))
             return out
         if norm is not None:
             raise KernelError("linear: rows that still lack their norm's scale need the MFMA kernels")
@@ -353,7 +375,7 @@ class Ops:
             self.lib.check(self.lib.xr_gemm_bf16(out.data_ptr(), a.data_ptr(), wt.data_ptr(), _ptr(bias), M, F, K,
                                                  a.stride(0), F, dtype_code(out.dtype), 2, variant,
                                                  1 if packed else 0, *self._gemm_workspace(a.device),
-                                                 C.addressof(norm) if norm is not None else None, _stream()))
+                                                 C.addressof(norm) if norm is not None else None, None, _stream()))
             return out
         if norm is not None:
             raise KernelError("linear_swiglu: rows that still lack their norm's scale need the MFMA kernels")
@@ -364,10 +386,11 @@ class Ops:
     # -- attention --------------------------------------------------------------
     def rope_kv_write(self, q_in, k_in, v_in, q_out, k_cache, v_cache, positions, req_of_token,
                       block_table, inv_freq, H: int, Hk: int, D: int, rot: int, interleaved: bool,
-                      mscale: float, page_size: int) -> None:
+                      mscale: float, page_size: int, paired: bool = False) -> None:
         """Rotate queries (into ``q_out``) and keys, and write keys and values to their pages.
 
-        ``q_in``/``k_in``/``v_in`` are 32-bit views with one common row stride.
+        ``q_in``/``k_in``/``v_in`` are 32-bit views with one common row stride.  ``paired``: the
+        channels of every query and key head come in ``paired_order``.
         """
         self._dev(q_in, k_in, v_in, q_out, k_cache, v_cache, positions, req_of_token, block_table, inv_freq)
         T = positions.numel()
@@ -385,7 +408,56 @@ class Ops:
             _ptr(q_in), _ptr(k_in), _ptr(v_in), stride, _ptr(q_out), _ptr(k_cache), _ptr(v_cache),
             positions.data_ptr(), _ptr(req_of_token), _ptr(block_table),
             block_table.stride(0) if block_table is not None else 0, _ptr(inv_freq), T, H, Hk, D, rot,
-            1 if interleaved else 0, float(mscale), page_size, dtype_code(store.dtype), _stream()))
+            1 if interleaved else 0, float(mscale), page_size, dtype_code(store.dtype), 1 if paired else 0,
+            _stream()))
+
+    def project_rope_kv_write(self, h, w, bias, k_cache, v_cache, positions, req_of_token, block_table,
+                              inv_freq, H: int, Hk: int, D: int, rot: int, interleaved: bool, mscale: float,
+                              page_size: int, paired: bool = False) -> torch.Tensor:
+        """``[q | k | v] = h @ w^T (+ bias)``, queries and keys rotated, keys and values written
+        to their pages; returns the rotated queries ``[T, H*D]`` in the compute dtype.
+
+        ``w`` holds ``H`` query heads, then ``Hk`` key heads and ``Hk`` value heads (``Hk`` = 0 and
+        no caches: queries alone); with ``paired`` its query and key rows are in ``paired_order``.
+        Up to 16 bfloat16 rows (``h`` may be an ``UnscaledRows``) the product's kernel rotates and
+        stores its own result, which saves a kernel and the 32-bit copy of the projections;
+        otherwise the product and ``rope_kv_write`` run one after the other."""
+        rows = h.data if isinstance(h, UnscaledRows) else h
+        wt = w.data if isinstance(w, PackedWeight) else w
+        T, Q, KV = rows.shape[0], H * D, Hk * D
+        if w.shape[0] != Q + 2 * KV:
+            raise KernelError(f"projection has {w.shape[0]} rows, {H} query and 2 x {Hk} key/value heads of {D} need {Q + 2 * KV}")
+        q = torch.empty((T, Q), dtype=rows.dtype, device=rows.device)
+        if (self.fuse_rope and T <= UnscaledRows.MAX_ROWS and self._mfma_ok(rows, wt) and D % 16 == 0
+                and (Hk == 0 or (k_cache.dtype == torch.bfloat16 and v_cache.dtype == torch.bfloat16))
+                and (rot == 0 or interleaved or (paired and rot % 16 == 0))):
+            self._dev(rows, wt, bias, k_cache, v_cache, positions, req_of_token, block_table, inv_freq)
+            self._contig(wt, "projection weight")
+            if rows.shape[1] != w.shape[1] or rows.stride(1) != 1:
+                raise KernelError(f"projection: shapes {tuple(rows.shape)} x {tuple(w.shape)}^T do not fit")
+            if bias is not None and (bias.dtype != torch.float32 or bias.numel() != w.shape[0]):
+                raise KernelError("projection: bias must be float32 [N]")
+            norm, rows = self._norm_before(h, None)
+            rp = _GemmRope()
+            rp.positions, rp.req_of_token, rp.block_table = positions.data_ptr(), _ptr(req_of_token), _ptr(block_table)
+            rp.table_stride = block_table.stride(0) if block_table is not None else 0
+            rp.inv_freq, rp.H, rp.Hk, rp.D, rp.rot = _ptr(inv_freq), H, Hk, D, rot
+            rp.interleaved, rp.mscale, rp.page_size = 1 if interleaved else 0, float(mscale), page_size
+            rp.q_out, rp.k_cache, rp.v_cache = q.data_ptr(), _ptr(k_cache) if Hk else None, _ptr(v_cache) if Hk else None
+            self.lib.check(self.lib.xr_gemm_bf16(None, rows.data_ptr(), wt.data_ptr(), _ptr(bias), T, w.shape[0],
+                                                 rows.shape[1], rows.stride(0), w.shape[0], XR_F32, 0, 0,
+                                                 1 if isinstance(w, PackedWeight) else 0,
+                                                 *self._gemm_workspace(rows.device),
+                                                 C.addressof(norm) if norm is not None else None,
+                                                 C.addressof(rp), _stream()))
+            return q
+        proj = self.linear(h, w, bias=bias, out_dtype=torch.float32)
+        k_in = proj[:, Q:Q + KV] if Hk else None
+        v_in = proj[:, Q + KV:Q + 2 * KV] if Hk else None
+        self.rope_kv_write(proj[:, :Q], k_in, v_in, q, k_cache if Hk else None, v_cache if Hk else None, positions,
+                           req_of_token, block_table, inv_freq, H, Hk, D, rot, interleaved, mscale, page_size,
+                           paired=paired)
+        return q
 
     def attention(self, q, k_cache, v_cache, ctx, group: int, H: int, Hk: int, D: int, page_size: int,
                   scale: float, window: Optional[int] = None) -> torch.Tensor:

@@ -72,41 +72,67 @@ class PagedAttention(Mixer):
 
     def bind(self, tensors, rt) -> None:
         self.rt = rt
+        if self.position is not None:
+            self.position.bind({}, rt)
         q, k, v, o = self.names
+        H, Hk, D = self.num_heads, self.num_kv_heads, self.head_dim
         mats = [tensors[f"{q}.weight"]]
         if not self.kv_shared:
             mats += [tensors[f"{k}.weight"], tensors[f"{v}.weight"]]
-        self.w_in = rt.ops.pack_weight(torch.cat(mats, dim=0).contiguous() if len(mats) > 1 else mats[0])
-        self.w_out = rt.ops.pack_weight(tensors[f"{o}.weight"])
+        w_in = torch.cat(mats, dim=0).contiguous() if len(mats) > 1 else mats[0]
+        b_in = None
         if self.bias:
             bs = [tensors[f"{q}.bias"]]
             if not self.kv_shared:
                 bs += [tensors[f"{k}.bias"], tensors[f"{v}.bias"]]
-            self.b_in = torch.cat([b.float() for b in bs]).contiguous()
+            b_in = torch.cat([b.float() for b in bs]).contiguous()
+        # A rotation that pairs channel j with j + rot/2: the rows of every query and key head go
+        # in paired order, so that the product's kernel has both halves of a pair at hand when
+        # it rotates its own result (a few decoded tokens); the rotation kernel reads that order too.
+        rot = self.position.rotary() if self.position is not None else None
+        self.paired = rot is not None and not rot.interleaved and rot.rotary_dim % 16 == 0 and D % 16 == 0
+        if self.paired:
+            from ..csrc.ops import paired_order
+            order = paired_order(D, rot.rotary_dim)
+            heads = H + (0 if self.kv_shared else Hk)
+            rows = [h * D + c for h in range(heads) for c in order] + list(range(heads * D, w_in.shape[0]))
+            index = torch.tensor(rows, dtype=torch.int64, device=w_in.device)
+            w_in = w_in.index_select(0, index)
+            if b_in is not None:
+                b_in = b_in.index_select(0, index)
+        self.w_in, self.b_in = rt.ops.pack_weight(w_in), b_in
+        self.w_out = rt.ops.pack_weight(tensors[f"{o}.weight"])
         if self.out_bias:
             self.b_out = tensors[f"{o}.bias"].float().contiguous()
-        if self.position is not None:
-            self.position.bind({}, rt)
 
     def _attend(self, ctx, cache, h):
         ops, rt = self.rt.ops, self.rt
         Q, K, H, Hk, D = self.q_size, self.kv_size, self.num_heads, self.num_kv_heads, self.head_dim
         T = h.shape[0]
-        proj = ops.linear(h, self.w_in, bias=self.b_in, out_dtype=torch.float32)
         writes = not self.kv_shared and cache.owns
-        q_in = proj[:, :Q]
-        k_in = proj[:, Q:Q + K] if writes else None
-        v_in = proj[:, Q + K:Q + 2 * K] if writes else None
         rot = self.position.rotary() if self.position is not None else None
-        if self.position is not None and rot is None:
-            self.position.apply(ctx, q_in.unflatten(1, (H, D)), k_in.unflatten(1, (Hk, D)) if writes else None)
-        q = torch.empty((T, Q), dtype=rt.dtype, device=h.device)
         table = ctx.block_table(cache.group)
-        ops.rope_kv_write(q_in, k_in, v_in, q, cache.k if writes else None, cache.v if writes else None,
-                          ctx.positions, ctx.req_of_token, table,
-                          rot.inv_freq if rot else None, H, Hk if writes else 0, D,
-                          rot.rotary_dim if rot else 0, rot.interleaved if rot else False,
-                          rot.mscale if rot else 1.0, cache.page_size)
+        if (self.position is None or rot is not None) and writes == (not self.kv_shared):
+            q = ops.project_rope_kv_write(
+                h, self.w_in, self.b_in, cache.k if writes else None, cache.v if writes else None, ctx.positions,
+                ctx.req_of_token, table, rot.inv_freq if rot else None, H, Hk if writes else 0, D,
+                rot.rotary_dim if rot else 0, rot.interleaved if rot else False, rot.mscale if rot else 1.0,
+                cache.page_size, paired=self.paired)
+        else:
+            # a position encoding of its own works on the 32-bit queries and keys before they are
+            # cached; or the keys and values this layer computes are another layer's to store
+            proj = ops.linear(h, self.w_in, bias=self.b_in, out_dtype=torch.float32)
+            q_in = proj[:, :Q]
+            k_in = proj[:, Q:Q + K] if writes else None
+            v_in = proj[:, Q + K:Q + 2 * K] if writes else None
+            if self.position is not None and rot is None:
+                self.position.apply(ctx, q_in.unflatten(1, (H, D)), k_in.unflatten(1, (Hk, D)) if writes else None)
+            q = torch.empty((T, Q), dtype=rt.dtype, device=h.device)
+            ops.rope_kv_write(q_in, k_in, v_in, q, cache.k if writes else None, cache.v if writes else None,
+                              ctx.positions, ctx.req_of_token, table,
+                              rot.inv_freq if rot else None, H, Hk if writes else 0, D,
+                              rot.rotary_dim if rot else 0, rot.interleaved if rot else False,
+                              rot.mscale if rot else 1.0, cache.page_size, paired=self.paired)
         return ops.attention(q, cache.k, cache.v, ctx, cache.group, H, Hk, D, cache.page_size, self.scale,
                              self.window)
 
