@@ -203,6 +203,31 @@ def test_rmsnorm_folded_into_the_products_around_it(ops, M, E, F, K, wdtype):
         ops.linear(UnscaledRows(torch.zeros(17, E, device=DEV).bfloat16(), h.sumsq, eps), w2)
 
 
+def test_linear_whose_tiles_do_not_fill_the_last_round(ops):
+    """314 tiles of 256x256 make a full round of 256 and a round of 58: the columns of the full
+    round go to that tile and the rest to a second launch with a smaller tile.  Every column
+    must be computed once (an accumulating epilogue would show a second time), also where the
+    two launches meet and at the ragged end."""
+    torch.manual_seed(5)
+    M, N, K = 512, 40008, 64
+    a = (torch.randn(M, K, device=DEV) * 0.5).bfloat16()
+    w = (torch.randn(N, K, device=DEV) * 0.1).bfloat16()
+    b = torch.randn(N, device=DEV) * 0.1
+    want = a.double() @ w.double().T
+    for wt in (w, ops.pack_weight(w)):
+        assert rel(ops.linear(a, wt, bias=b, out_dtype=torch.float32), want + b.double()) < 1e-5
+        base = torch.randn(M, N, device=DEV)
+        out = base.clone()
+        ops.linear(a, wt, out=out, accumulate=True)
+        assert rel(out, base.double() + want) < 1e-5
+        assert rel(out[:, 32768 - 300:32768 + 300], (base.double() + want)[:, 32768 - 300:32768 + 300]) < 1e-5
+    F = 20000
+    w2 = (torch.randn(2 * F, K, device=DEV) * 0.1).bfloat16()
+    r = a.double() @ w2.double().T
+    got = ops.linear_swiglu(a, ops.pack_weight(w2, gated=True))
+    assert rel(got, r[:, :F] / (1 + torch.exp(-r[:, :F])) * r[:, F:]) < 6e-3
+
+
 def test_pack_weight_leaves_what_the_mfma_kernels_do_not_take(ops):
     w = torch.randn(40, 20, device=DEV).bfloat16()                      # width no multiple of 8
     assert ops.pack_weight(w) is w

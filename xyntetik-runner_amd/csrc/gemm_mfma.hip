@@ -62,6 +62,7 @@ struct GemmArgs {
     int splits;        // > 1: K is cut into this many ranges, each workgroup writes raw sums to `partial`
     int k_per_split;   // columns per range (a multiple of 64)
     float* partial;    // [splits][M][rows of w]
+    int col0, col1;    // the tile kernel computes output columns col0 .. col1-1 (col0 a multiple of the tile's width)
     // RMSNorm folded into the skinny kernel (all null or zero: off).
     // Before: `a` holds rows x*weight that are not yet divided by their root mean square; ss_in
     // [n_ss][16] holds partial sums of x^2 per row, and the product's row t is scaled by
@@ -187,10 +188,12 @@ __global__ __launch_bounds__(64 * WARPS_M * WARPS_N) void k_gemm_tile_async(Gemm
     // workgroups go to different XCDs, so with 8 row tiles each XCD keeps one activation tile
     // in its L2 while the weight tile of the moment is fetched once from memory for all.
     const int tiles_m = (g.M + BM - 1) / BM;
-    const int tiles_n = (g.N + (g.epi == EPI_SWIGLU ? BN / 2 : BN) - 1) / (g.epi == EPI_SWIGLU ? BN / 2 : BN);
+    constexpr int BN_OUT_S = BN / 2;
+    const int bn_out = g.epi == EPI_SWIGLU ? BN_OUT_S : BN;
+    const int tiles_n = (g.col1 - g.col0 + bn_out - 1) / bn_out;
     const int tile_ = (int)(blockIdx.x / g.splits), split_ = (int)(blockIdx.x % g.splits);
     const int bm_ = g.m_fast ? tile_ % tiles_m : tile_ / tiles_n;
-    const int bx = g.m_fast ? tile_ / tiles_m : tile_ % tiles_n;
+    const int bx = g.col0 / bn_out + (g.m_fast ? tile_ / tiles_m : tile_ % tiles_n);
     const int k_begin = split_ * g.k_per_split;
     const int k_end = (k_begin + g.k_per_split) < g.K ? (k_begin + g.k_per_split) : g.K;
     const int m0 = bm_ * BM;
@@ -377,9 +380,14 @@ static int launch_tile_async(GemmArgs g, hipStream_t stream) {
         attr_set = true;
     }
     int n_out_tile = g.epi == EPI_SWIGLU ? BN / 2 : BN;
-    unsigned tiles_n = (unsigned)((g.N + n_out_tile - 1) / n_out_tile), tiles_m = (unsigned)((g.M + BM - 1) / BM);
+    if (g.col1 <= 0 || g.col1 > g.N) g.col1 = g.N;
+    if (g.col0 < 0 || g.col0 % n_out_tile || g.col0 >= g.col1 || (g.col1 < g.N && g.col1 % n_out_tile)) {
+        xr_set_error("gemm: columns %d..%d do not start at a %d-column tile", g.col0, g.col1, n_out_tile);
+        return XR_BAD_ARG;
+    }
+    unsigned tiles_n = (unsigned)((g.col1 - g.col0 + n_out_tile - 1) / n_out_tile), tiles_m = (unsigned)((g.M + BM - 1) / BM);
     unsigned tiles = tiles_n * tiles_m;
-    if (g.splits < 1 || !g.partial) g.splits = 1;
+    if (g.splits < 1 || !g.partial || g.col0 > 0 || g.col1 < g.N) g.splits = 1;
     if (g.splits > 1) {
         int slices = (g.K + 63) / 64;
         int per = (slices + g.splits - 1) / g.splits;
@@ -613,6 +621,23 @@ __global__ __launch_bounds__(64 * KSW) void k_gemm_skinny(GemmArgs g) {
     }
 }
 
+static int launch_tile_variant(int variant, const GemmArgs& g, hipStream_t stream) {
+    if (variant == 10) return launch_tile_async<128, 128, 2, 2, 3>(g, stream);
+    if (variant == 11) return launch_tile_async<128, 128, 2, 2, 4>(g, stream);
+    if (variant == 12) return launch_tile_async<256, 128, 4, 2, 3>(g, stream);
+    if (variant == 13) return launch_tile_async<256, 256, 2, 4, 2>(g, stream);
+    if (variant == 14) return launch_tile_async<256, 256, 4, 2, 2>(g, stream);
+    if (variant == 15) return launch_tile_async<256, 128, 2, 2, 3>(g, stream);
+    if (variant == 16) return launch_tile_async<128, 256, 2, 4, 3>(g, stream);
+    if (variant == 17) return launch_tile_async<128, 128, 2, 2, 2>(g, stream);
+    if (variant == 18) return launch_tile_async<256, 256, 2, 2, 2>(g, stream);
+    if (variant == 19) return launch_tile_async<256, 128, 2, 2, 2>(g, stream);
+    if (variant == 20) return launch_tile_async<128, 256, 2, 2, 2>(g, stream);
+    if (variant == 26) return launch_tile_async<256, 192, 4, 2, 2>(g, stream);
+    xr_set_error("gemm: unknown variant %d", variant);
+    return XR_BAD_ARG;
+}
+
 // returns the number of workgroups, or an error (< 0)
 static inline int rc_of(int launched) { return launched < 0 ? launched : XR_OK; }
 
@@ -684,7 +709,7 @@ extern "C" int xr_gemm_bf16(void* out, const void* a, const void* w, const float
     GemmArgs g;
     g.a = (const bf16_t*)a; g.w = (const bf16_t*)w; g.w_packed = w_packed ? 1 : 0; g.bias = bias; g.out = out;
     g.M = M; g.N = N; g.K = K; g.lda = lda; g.ldo = ldo; g.out_bf16 = out_dtype == XR_BF16; g.epi = epi;
-    g.m_fast = 0; g.splits = 1; g.k_per_split = 0; g.partial = workspace;
+    g.m_fast = 0; g.splits = 1; g.k_per_split = 0; g.partial = workspace; g.col0 = 0; g.col1 = N;
     g.ss_in = nullptr; g.n_ss = 0; g.ss_inv_width = 0.f; g.ss_eps = 0.f;
     g.norm_w = nullptr; g.norm_w_bf16 = 0; g.xg = nullptr; g.ss_out = nullptr;
     if (norm) {
@@ -741,24 +766,44 @@ extern "C" int xr_gemm_bf16(void* out, const void* a, const void* w, const float
         } else {
             // The tile that keeps the chip busiest: larger tiles do more products for a byte that
             // L1 delivers (what bounds this kernel), but their count may fill the 256 compute
-            // units badly.  A tile's worth is its measured rate with the chip full (relative to
-            // 256x256) times the share of the chip its rounds of workgroups keep busy; if even the
-            // smallest tile does not fill the chip, K is split as well.
-            const int n_out = N;
-            auto count = [&](int bm, int bn) { return ((M + bm - 1) / bm) * ((n_out + (sw ? bn / 2 : bn) - 1) / (sw ? bn / 2 : bn)); };
-            auto worth = [&](int bm, int bn, double rate) {
-                const int tiles = count(bm, bn);
-                return rate * tiles / (double)(((tiles + 255) / 256) * 256);
-            };
-            const double w256 = worth(256, 256, 1.0), w192 = sw ? 0.0 : worth(256, 192, 0.9);
-            const double w128 = worth(256, 128, 0.85), w64 = worth(128, 128, 0.78);
-            variant = 14;
-            double best = w256;
-            if (w192 > best) { variant = 26; best = w192; }
-            if (w128 > best) { variant = 12; best = w128; }
-            if (w64 > best) { variant = 17; best = w64; }
+            // units badly.  A tile's time is its area over its measured rate with the chip full
+            // (relative to 256x256); a launch takes as many of these as its tiles make rounds of
+            // 256.  When the last round of the best tile would leave most of the chip idle, the
+            // columns of the full rounds go to that tile and the rest to a second launch with a
+            // smaller one (3 rounds + 1 of half-size tiles instead of 4).  If even the smallest
+            // tile does not fill the chip, K is split as well.
+            struct Cand { int variant, bm, bn; double rate; };
+            const Cand cands[4] = {{14, 256, 256, 1.0}, {26, 256, 192, 0.9}, {12, 256, 128, 0.85}, {17, 128, 128, 0.78}};
+            auto width = [&](const Cand& c) { return sw ? c.bn / 2 : c.bn; };
+            auto usable = [&](const Cand& c) { return !(sw && c.variant == 26); };
+            auto count = [&](const Cand& c, int cols) { return ((M + c.bm - 1) / c.bm) * ((cols + width(c) - 1) / width(c)); };
+            auto time_of = [&](const Cand& c, int cols) { return (double)((count(c, cols) + 255) / 256) * c.bm * c.bn / c.rate; };
+            int best = 0, second = -1, cols_first = N;
+            double t_best = time_of(cands[0], N);
+            for (int i = 1; i < 4; ++i)
+                if (usable(cands[i]) && time_of(cands[i], N) < t_best) { best = i; t_best = time_of(cands[i], N); }
+            for (int i = 0; i < 3; ++i) {
+                if (!usable(cands[i])) continue;
+                const int tm = (M + cands[i].bm - 1) / cands[i].bm, full = count(cands[i], N) / 256;
+                const int cols = full * 256 / tm * width(cands[i]);          // the columns of the full rounds
+                if (full < 1 || count(cands[i], N) % 256 == 0 || cols <= 0 || cols >= N) continue;
+                for (int j = i + 1; j < 4; ++j) {
+                    if (!usable(cands[j]) || cols % width(cands[j])) continue;
+                    const double t = time_of(cands[i], cols) + time_of(cands[j], N - cols);
+                    if (t < 0.97 * t_best) { best = i; second = j; cols_first = cols; t_best = t; }
+                }
+            }
+            variant = cands[best].variant;
             g.m_fast = 1;
-            if (variant == 17 && count(128, 128) < 160) g.splits = pick_splits(count(128, 128));
+            if (second >= 0) {
+                GemmArgs g2 = g;
+                g.col1 = cols_first;
+                g2.col0 = cols_first;
+                const int rc = launch_tile_variant(variant, g, stream);
+                return rc != XR_OK ? rc : launch_tile_variant(cands[second].variant, g2, stream);
+            }
+            auto count_of = [&](int bm, int bn) { return ((M + bm - 1) / bm) * ((N + (sw ? bn / 2 : bn) - 1) / (sw ? bn / 2 : bn)); };
+            if (variant == 17 && count_of(128, 128) < 160) g.splits = pick_splits(count_of(128, 128));
         }
     }
     if (variant == 1) {
@@ -792,24 +837,11 @@ extern "C" int xr_gemm_bf16(void* out, const void* a, const void* w, const float
     SK(124, 1, 4, 8, 4, false) SK(125, 1, 2, 16, 8, false) SK(126, 1, 4, 2, 8, false)
 #undef SK
 #endif
-    if (variant == 10) return launch_tile_async<128, 128, 2, 2, 3>(g, stream);
-    if (variant == 11) return launch_tile_async<128, 128, 2, 2, 4>(g, stream);
-    if (variant == 12) return launch_tile_async<256, 128, 4, 2, 3>(g, stream);
-    if (variant == 13) return launch_tile_async<256, 256, 2, 4, 2>(g, stream);
-    if (variant == 14) return launch_tile_async<256, 256, 4, 2, 2>(g, stream);
-    if (variant == 15) return launch_tile_async<256, 128, 2, 2, 3>(g, stream);
-    if (variant == 16) return launch_tile_async<128, 256, 2, 4, 3>(g, stream);
-    if (variant == 17) return launch_tile_async<128, 128, 2, 2, 2>(g, stream);
-    if (variant == 18) return launch_tile_async<256, 256, 2, 2, 2>(g, stream);
-    if (variant == 19) return launch_tile_async<256, 128, 2, 2, 2>(g, stream);
-    if (variant == 20) return launch_tile_async<128, 256, 2, 2, 2>(g, stream);
-    if (variant == 26) return launch_tile_async<256, 192, 4, 2, 2>(g, stream);
     if (variant == 30 || variant == 31) {       // few rows: 32 or 64 of them against 128 weight rows, K split
         const int bn_out = sw ? 64 : 128;
         g.splits = pick_splits((N + bn_out - 1) / bn_out);
         if (variant == 30) return launch_tile_async<32, 128, 1, 2, 3>(g, stream);
         return launch_tile_async<64, 128, 2, 2, 3>(g, stream);
     }
-    xr_set_error("gemm: unknown variant %d", variant);
-    return XR_BAD_ARG;
+    return launch_tile_variant(variant, g, stream);
 }
