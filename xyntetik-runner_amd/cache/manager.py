@@ -61,6 +61,8 @@ class CacheManager:
         self.groups = [GroupInfo(s, page_size, Pool(pages_per_group, first=1, what="page")) for s in group_specs]
         self.slots = Pool(n_slots, what="state slot")
         self.requests: Dict[Hashable, RequestCache] = {}
+        self._no_pages = [0] * len(self.groups)
+        self._windowed = [gi for gi, g in enumerate(self.groups) if g.spec.window is not None]
 
     # ------------------------------------------------------------------ sizes
     @property
@@ -86,10 +88,15 @@ class CacheManager:
         return self.slots.n_free > 0
 
     def _new_pages_needed(self, rc: RequestCache, new_len: int) -> List[int]:
+        want = self.pages_for(new_len)
+        for t in rc.tables:
+            if len(t) < want:
+                break
+        else:
+            return self._no_pages           # the usual case of a decoded token (callers only read it)
         need = []
         for gi, g in enumerate(self.groups):
             have = len(rc.tables[gi])
-            want = self.pages_for(new_len)
             # pages wholly below the window of the first new query are never read or written
             lo_page = first_needed_position(rc.n_tokens, g.spec.window) // self.page_size
             need.append(sum(1 for i in range(have, want) if i >= lo_page))
@@ -113,6 +120,8 @@ class CacheManager:
         if new_len < rc.n_tokens:
             raise ValueError(f"request {req_id!r} holds {rc.n_tokens} tokens, cannot shrink to {new_len}")
         need = self._new_pages_needed(rc, new_len)
+        if need is self._no_pages:
+            return
         for gi, g in enumerate(self.groups):
             if need[gi] > g.pool.n_free:
                 raise OutOfPages(f"request {req_id!r} needs {need[gi]} more pages in group {gi}, "
@@ -130,9 +139,8 @@ class CacheManager:
             raise ValueError(f"request {req_id!r}: {new_len} tokens were not reserved")
         rc.n_tokens = new_len
         rc.fresh = False
-        for gi, g in enumerate(self.groups):
-            if g.spec.window is None:
-                continue
+        for gi in self._windowed:
+            g = self.groups[gi]
             lo_page = first_needed_position(new_len, g.spec.window) // self.page_size
             table = rc.tables[gi]
             for i in range(min(lo_page, len(table))):

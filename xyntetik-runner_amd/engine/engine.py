@@ -83,13 +83,13 @@ class Engine:
             return outs
         entries = []
         for req, n in plan.entries:
-            toks = req.tokens[req.n_computed:req.n_computed + n]
+            toks = req.token_slice(req.n_computed, req.n_computed + n)
             last = req.n_computed + n == req.n_tokens
             entries.append(StepEntry(req.id, toks, [n - 1] if last else []))
             # the sampler's window sees every token of the request once, prompt included
             # (/root/reference/src/engine.c:881)
             upto = req.n_computed + n
-            for t in req.tokens[req.n_accepted:upto]:
+            for t in req.token_slice(req.n_accepted, upto):
                 req.sampler.accept(t)
             req.n_accepted = max(req.n_accepted, upto)
         t0 = time.perf_counter()
@@ -105,7 +105,6 @@ class Engine:
                     self.stats.generated_tokens += 1
                 outs.append(StepOutput(req.id, new, done, req.finish_reason))
         dt = time.perf_counter() - t0
-        n_prompt = sum(n for r, n in plan.entries if n > 1 or r.n_computed <= len(r.prompt))
         if any(n > 1 for _, n in plan.entries):
             self.stats.prefill_seconds += dt
         else:

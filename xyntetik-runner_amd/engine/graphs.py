@@ -48,8 +48,11 @@ def splits_for(batch_cap: int, max_tiles: int, n_kv_heads: int) -> int:
 class StaticDecodeContext:
     """A ``StepContext`` for one token per request whose device arrays never move."""
 
-    def __init__(self, ops, device, batch_cap: int, n_splits: int, table_widths: List[int]):
+    def __init__(self, ops, device, batch_cap: int, n_splits: int, table_widths: List[int],
+                 windowed: Optional[List[bool]] = None):
         self.ops, self.device = ops, device
+        # groups whose requests give pages back while they live (their table rows are rewritten every step)
+        self.windowed = list(windowed) if windowed is not None else [True] * len(table_widths)
         self.B = self.T = batch_cap
         self.S = n_splits
         self.table_width = list(table_widths)
@@ -74,6 +77,12 @@ class StaticDecodeContext:
         total = int(offs[-1]) + n_plan
         self._offs = offs
         self._host = torch.zeros((total,), dtype=torch.int32).pin_memory()
+        # what each row of each block table in the pinned buffer holds: (the request's cache record, pages)
+        self._rows = [[None] * B for _ in self.table_width]
+        for g, w in enumerate(self.table_width):
+            tab = self._host.numpy()[offs[9 + g]:offs[10 + g]].reshape(B, w)
+            tab[:] = -1
+            tab[:, 0] = NULL_PAGE
         self._dev = torch.zeros((total,), dtype=torch.int32, device=self.device)
         d, o = self._dev, offs
         self.token_ids, self.positions, self.req_of_token = d[o[0]:o[1]], d[o[1]:o[2]], d[o[2]:o[3]]
@@ -130,13 +139,25 @@ class StaticDecodeContext:
         h[o[8]:o[9]] = np.arange(B, dtype=np.int32)
         for g, w in enumerate(self.table_width):
             tab = h[o[9 + g]:o[10 + g]].reshape(B, w)
-            tab[:] = -1
-            tab[:, 0] = NULL_PAGE
-            for b, rc in enumerate(rcs):
+            held = self._rows[g]
+            for b in range(B):
+                rc = rcs[b] if b < n else None
+                if rc is None:
+                    if held[b] is not None:
+                        tab[b, :] = -1
+                        tab[b, 0] = NULL_PAGE
+                        held[b] = None
+                    continue
                 t = rc.tables[g]
+                # a table only grows at its end while its request lives, unless a window gives pages back
+                if not self.windowed[g] and held[b] is not None and held[b][0] is rc and held[b][1] == len(t):
+                    continue
                 if len(t) > w:
                     raise ValueError("a request outgrew the block table of its graph bucket")
+                tab[b, :] = -1
+                tab[b, 0] = NULL_PAGE
                 tab[b, :len(t)] = t
+                held[b] = (rc, len(t))
         self.starts = [int(s) for s in starts]
         self.seq_lens = [s + 1 for s in self.starts]
         self.max_seq_len = max(self.seq_lens)
@@ -217,7 +238,8 @@ class DecodeGraphs:
             self.replays += 1
             return logits[:n]
         # first time: run the step eagerly on the static context, then record it for later
-        ctx = StaticDecodeContext(r.ops, r.device, cap, S, width)
+        ctx = StaticDecodeContext(r.ops, r.device, cap, S, width,
+                                  windowed=[g.spec.window is not None for g in r.manager.groups])
         ctx.fill(entries, rcs)
         x = r.model.forward(ctx, r.storage.layers)
         out = r.model.logits(ctx, x, ctx.want_rows)

@@ -15,6 +15,7 @@ class Request:
             raise ValueError("a request needs at least one prompt token")
         self.id = req_id
         self.prompt = [int(t) for t in prompt]
+        self._n_prompt = len(self.prompt)      # (the prompt never changes)
         self.params = params
         self.output: List[int] = []
         self.n_computed = 0          # tokens of prompt + output whose keys and values are cached
@@ -28,14 +29,23 @@ class Request:
     def tokens(self) -> List[int]:
         return self.prompt + self.output
 
+    def token_slice(self, a: int, b: int) -> List[int]:
+        """``tokens[a:b]`` without putting prompt and output together first."""
+        n = self._n_prompt
+        if a >= n:
+            return self.output[a - n:b - n]
+        if b <= n:
+            return self.prompt[a:b]
+        return self.prompt[a:] + self.output[:b - n]
+
     @property
     def n_tokens(self) -> int:
-        return len(self.prompt) + len(self.output)
+        return self._n_prompt + len(self.output)
 
     @property
     def remaining(self) -> int:
         """Tokens that still have to run before the next one can be sampled."""
-        return self.n_tokens - self.n_computed
+        return self._n_prompt + len(self.output) - self.n_computed
 
     @property
     def finished(self) -> bool:

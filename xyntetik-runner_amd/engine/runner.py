@@ -101,11 +101,12 @@ class ModelRunner:
         mgr = self.manager
         rcs = [mgr.get(e.req_id) for e in entries]
         # reserve for all or for none
-        spare = [0] * len(mgr.groups)
+        spare = None
         for e, rc in zip(entries, rcs):
             need = mgr.pages_needed(e.req_id, rc.n_tokens + len(e.tokens))
-            spare = [s + n for s, n in zip(spare, need)]
-        for gi, g in enumerate(mgr.groups):
+            if any(need):
+                spare = [s + n for s, n in zip(spare, need)] if spare else list(need)
+        for gi, g in enumerate(mgr.groups if spare else ()):
             if spare[gi] > g.pool.n_free:
                 raise OutOfPages(f"this step needs {spare[gi]} new pages in group {gi}, {g.pool.n_free} of {g.pool.size} are free")
         for e, rc in zip(entries, rcs):

@@ -91,9 +91,12 @@ class Scheduler:
         budget = self.max_batched_tokens
         mgr = self.manager
         # running requests: decoding ones first, then prompts under way
-        order = [r for r in self.running if r.remaining == 1] + [r for r in self.running if r.remaining > 1]
+        order, prompts = [], []
+        for r in self.running:
+            (order if r.remaining == 1 else prompts).append(r)
+        order += prompts
         for req in order:
-            if req not in self.running or budget <= 0:      # preempted meanwhile / nothing left
+            if budget <= 0 or (plan.preempted and req not in self.running):      # nothing left / preempted meanwhile
                 continue
             n = min(req.remaining, budget)
             while True:
