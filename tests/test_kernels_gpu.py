@@ -228,6 +228,46 @@ def test_linear_whose_tiles_do_not_fill_the_last_round(ops):
     assert rel(got, r[:, :F] / (1 + torch.exp(-r[:, :F])) * r[:, F:]) < 6e-3
 
 
+@pytest.mark.parametrize("M", [17, 33, 64])
+@pytest.mark.parametrize("E,K", [(64, 48), (200, 520), (4096, 1024), (5120, 264)])
+@pytest.mark.parametrize("wdtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("bias", [False, True])
+def test_rmsnorm_by_the_kernel_that_adds_up_a_split_product(ops, M, E, K, wdtype, bias):
+    """17 to 64 rows: residual += a @ w^T (+ bias) and the norm of the result from the product and
+    one more kernel; against the product and the norm's own kernel (the residual to the bit when
+    the K ranges are the same, else to rounding) and against float64."""
+    torch.manual_seed(M + E)
+    a = (torch.randn(M, K, device=DEV) * 0.5).bfloat16()
+    w = ops.pack_weight((torch.randn(E, K, device=DEV) * 0.1).bfloat16())
+    b = torch.randn(E, device=DEV) * 0.2 if bias else None
+    nw = (1 + 0.2 * torch.randn(E, device=DEV)).to(wdtype)
+    res0 = torch.randn(M, E + 4, device=DEV)[:, :E] * torch.linspace(0.1, 30, M, device=DEV)[:, None]
+    eps = 1e-6
+    r1, r2 = res0.clone(), res0.clone()
+    assert r1.stride(0) == E
+    h1 = ops.linear_add_rmsnorm(a, w, r1, nw, eps, torch.bfloat16, bias=b)
+    ops.fold_norms = False
+    try:
+        h2 = ops.linear_add_rmsnorm(a, w, r2, nw, eps, torch.bfloat16, bias=b)
+    finally:
+        ops.fold_norms = True
+    assert isinstance(h1, torch.Tensor) and h1.dtype == torch.bfloat16 and h1.shape == (M, E)
+    from xyntetik_runner_amd.csrc.ops import PackedWeight
+    wd = w.data if isinstance(w, PackedWeight) else w
+    x = res0.double() + a.double() @ _unpack(wd, E, K).double().T + (b.double() if bias else 0)
+    assert rel(r1, x) < 1e-5 and rel(r2, x) < 1e-5
+    want = x * torch.rsqrt((x * x).mean(1, keepdim=True) + eps) * nw.double()
+    assert rel(h1, want) < 6e-3 and rel(h2, want) < 6e-3
+    assert rel(h1, h2.float()) < 8e-3           # a bfloat16 rounding apart at most
+
+
+def _unpack(data, N, K):
+    """A packed weight back in rows."""
+    if data.dim() == 2:
+        return data
+    return data.permute(0, 2, 1, 3).reshape(data.shape[0] * 16, data.shape[1] * 32)[:N, :K]
+
+
 def test_pack_weight_leaves_what_the_mfma_kernels_do_not_take(ops):
     w = torch.randn(40, 20, device=DEV).bfloat16()                      # width no multiple of 8
     assert ops.pack_weight(w) is w
@@ -378,11 +418,12 @@ def test_rope_kv_write(ops, dt, H, Hk, D, rot, inter, ps, starts, q_lens):
 @pytest.mark.parametrize("H,Hk,D,rot,inter", [(4, 2, 16, 16, False), (3, 1, 48, 32, False), (6, 3, 80, 80, True),
                                                (8, 8, 128, 64, True), (5, 1, 128, 128, False), (2, 2, 32, 0, False)])
 @pytest.mark.parametrize("ps,starts,q_lens", [(16, [0, 13, 40], [9, 3, 1]), (64, [70], [1]), (8, [2, 9, 100, 7], [5, 6, 1, 4]),
-                                              (16, [3, 0], [30, 8])])
+                                              (16, [3, 0], [30, 8]), (16, [5, 0, 77], [60, 20, 3])])
 @pytest.mark.parametrize("bias", [False, True])
 def test_projection_with_rotation_and_cache_write(ops, dt, H, Hk, D, rot, inter, ps, starts, q_lens, bias):
     """q, k and v from one product, rotated and cached.  Up to 16 bfloat16 rows the product's own
-    kernel does all of it (with the weight's rows in paired order where a pair is (j, j + rot/2));
+    kernel does all of it (with the weight's rows in paired order where a pair is (j, j + rot/2)),
+    up to 64 the kernel that adds the product's K ranges up;
     more rows, or 32-bit, run the product and the rotation kernel.  Both against float64 from
     the weights in their natural order; and the two bfloat16 ways against each other."""
     from xyntetik_runner_amd.csrc.ops import paired_order

@@ -62,6 +62,8 @@ struct GemmArgs {
     int splits;        // > 1: K is cut into this many ranges, each workgroup writes raw sums to `partial`
     int k_per_split;   // columns per range (a multiple of 64)
     float* partial;    // [splits][M][rows of w]
+    int raw;           // 1: raw sums go to `partial` also when K is whole (an epilogue of k_gemm_finish is wanted)
+    int norm_whole;    // 1: k_gemm_finish_norm writes the whole norm of the updated rows to xg
     int col0, col1;    // the tile kernel computes output columns col0 .. col1-1 (col0 a multiple of the tile's width)
     // RMSNorm folded into the skinny kernel (all null or zero: off).
     // Before: `a` holds rows x*weight that are not yet divided by their root mean square; ss_in
@@ -135,6 +137,37 @@ __device__ inline void store_out(const GemmArgs& g, int m, int n, float v) {
     } else {
         ((float*)g.out)[o] = v;
     }
+}
+
+// One element of a projection's result, column nn of row tok, to where it belongs: queries and
+// keys rotated (`partner` is the value 8 columns away in paired order, or 1 with interleaved
+// pairs), queries to their buffer, keys and values to their pages; formulas as in k_rope_kv_write.
+__device__ inline void rope_store(const RopeFuse& rp, int tok, int nn, float val, float partner) {
+    const int Q = rp.H * rp.D, KV = rp.Hk * rp.D;
+    const int sec = nn < Q ? 0 : (nn < Q + KV ? 1 : 2);
+    const int rel = nn - (sec == 0 ? 0 : (sec == 1 ? Q : Q + KV));
+    const int hs = rel / rp.D, c = rel - hs * rp.D;
+    const int pos = rp.positions[tok];
+    int d = c;
+    float o = val;
+    if (sec < 2 && c < rp.rot) {
+        int j, hi;
+        if (rp.interleaved) { j = c >> 1; hi = c & 1; }
+        else { hi = (c >> 3) & 1; j = (c >> 4) * 8 + (c & 7); d = j + hi * (rp.rot >> 1); }
+        const float ang = (float)pos * rp.inv_freq[j];
+        const float cs = cosf(ang) * rp.mscale, sn = sinf(ang) * rp.mscale;
+        const float x0 = hi ? partner : val, x1 = hi ? val : partner;
+        o = hi ? x0 * sn + x1 * cs : x0 * cs - x1 * sn;
+    }
+    if (sec == 0) {
+        rp.q_out[((size_t)tok * rp.H + hs) * rp.D + d] = f32_to_bf16(o);
+        return;
+    }
+    const PageRef pr = page_of(rp.block_table, rp.table_stride, rp.req_of_token[tok], pos, rp.page_shift, rp.page_mask);
+    if (sec == 1)
+        rp.k_cache[(((size_t)pr.page * rp.Hk + hs) * rp.page_size + pr.off) * rp.D + d] = f32_to_bf16(o);
+    else
+        rp.v_cache[(((size_t)pr.page * rp.Hk + hs) * rp.D + d) * rp.page_size + pr.off] = f32_to_bf16(o);
 }
 
 // ------------------------------------------------------------------------------ tile kernel
@@ -291,7 +324,7 @@ __global__ __launch_bounds__(64 * WARPS_M * WARPS_N) void k_gemm_tile_async(Gemm
 #undef ASYNC_ISSUE_PART
     wait_vmcnt<0>();                                     // the trailing loads of zeros
 
-    if (g.splits > 1) {
+    if (g.splits > 1 || g.raw) {
         // raw sums of this K range, by weight row: the epilogue belongs to k_gemm_finish
         const int ldp = g.epi == EPI_SWIGLU ? 2 * g.N : g.N;
         float* part = g.partial + (size_t)split_ * g.M * ldp;
@@ -346,18 +379,72 @@ __global__ __launch_bounds__(64 * WARPS_M * WARPS_N) void k_gemm_tile_async(Gemm
 __global__ __launch_bounds__(256) void k_gemm_finish(GemmArgs g) {
     const int ldp = g.epi == EPI_SWIGLU ? 2 * g.N : g.N;
     const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
-    if (idx >= (size_t)g.M * g.N) return;
-    const int m = (int)(idx / g.N), n = (int)(idx % g.N);
+    const bool ok = idx < (size_t)g.M * g.N;
+    if (!ok && !g.rope.q_out) return;
+    const int m = ok ? (int)(idx / g.N) : 0, n = ok ? (int)(idx % g.N) : 0;
     const size_t step = (size_t)g.M * ldp;
     const float* p = g.partial + (size_t)m * ldp + n;
     float v = 0.f, u = 0.f;
     for (int s = 0; s < g.splits; ++s) v += p[s * step];
-    if (g.epi == EPI_SWIGLU) {
+    if (g.rope.q_out) {
+        // (N is a multiple of 16 here, so the 16 columns of a group are 16 lanes side by side)
+        const float val = v + (g.bias ? g.bias[n] : 0.f);
+        const float partner = __shfl_xor(val, g.rope.interleaved ? 1 : 8);
+        if (ok) rope_store(g.rope, m, n, val, partner);
+    } else if (g.epi == EPI_SWIGLU) {
         for (int s = 0; s < g.splits; ++s) u += p[s * step + g.N];
         const float bg = g.bias ? g.bias[n] : 0.f, bu = g.bias ? g.bias[g.N + n] : 0.f;
         store_out(g, m, n, silu_f(v + bg) * (u + bu));
     } else {
         store_out(g, m, n, v + (g.bias ? g.bias[n] : 0.f));
+    }
+}
+
+// The same for a product that adds into the 32-bit residual stream and is followed by an
+// RMSNorm: a workgroup takes a whole row, so it can also sum the squares of the updated row
+// (threads, then waves, in a fixed order) and write the normed row, times the norm's weight,
+// to xg.  N is a multiple of 4.
+__global__ __launch_bounds__(1024) void k_gemm_finish_norm(GemmArgs g) {
+    __shared__ float wave_sq[16];
+    __shared__ float rstd_s;
+    const int m = blockIdx.x, tid = threadIdx.x;
+    const size_t step = (size_t)g.M * g.N;
+    float* xrow = (float*)g.out + (size_t)m * g.ldo;
+    float sq = 0.f;
+    for (int n = tid * 4; n < g.N; n += 1024 * 4) {
+        const float* p = g.partial + (size_t)m * g.N + n;
+        float4 v = *reinterpret_cast<const float4*>(p);
+        for (int s = 1; s < g.splits; ++s) {
+            const float4 w = *reinterpret_cast<const float4*>(p + s * step);
+            v.x += w.x; v.y += w.y; v.z += w.z; v.w += w.w;
+        }
+        if (g.bias) { v.x += g.bias[n]; v.y += g.bias[n + 1]; v.z += g.bias[n + 2]; v.w += g.bias[n + 3]; }
+        float4 x = *reinterpret_cast<const float4*>(xrow + n);
+        x.x += v.x; x.y += v.y; x.z += v.z; x.w += v.w;
+        *reinterpret_cast<float4*>(xrow + n) = x;
+        sq += x.x * x.x + x.y * x.y + x.z * x.z + x.w * x.w;
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) sq += __shfl_xor(sq, o);
+    if ((tid & 63) == 0) wave_sq[tid >> 6] = sq;
+    __syncthreads();
+    if (tid == 0) {
+        float t = 0.f;
+        for (int w = 0; w < 16; ++w) t += wave_sq[w];
+        rstd_s = rsqrtf(t * g.ss_inv_width + g.ss_eps);
+    }
+    __syncthreads();
+    const float rstd = rstd_s;
+    for (int n = tid * 4; n < g.N; n += 1024 * 4) {
+        const float4 x = *reinterpret_cast<const float4*>(xrow + n);     // what this thread wrote above
+        float w[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+            w[i] = g.norm_w_bf16 ? bf16_to_f32(((const bf16_t*)g.norm_w)[n + i]) : ((const float*)g.norm_w)[n + i];
+        uint2 o;
+        o.x = pack_bf16x2(x.x * rstd * w[0], x.y * rstd * w[1]);
+        o.y = pack_bf16x2(x.z * rstd * w[2], x.w * rstd * w[3]);
+        *reinterpret_cast<uint2*>(g.xg + (size_t)m * g.N + n) = o;
     }
 }
 
@@ -395,9 +482,16 @@ static int launch_tile_async(GemmArgs g, hipStream_t stream) {
         g.splits = (slices + per - 1) / per;            // no empty range
     }
     if (g.splits == 1) g.k_per_split = ((g.K + 63) / 64) * 64;
+    if (g.raw && (!g.partial || g.col0 > 0 || g.col1 < g.N)) {
+        xr_set_error("gemm: no room for the raw sums of a product whose epilogue is a kernel of its own");
+        return XR_BAD_ARG;
+    }
     k_gemm_tile_async<BM, BN, WM_, WN_, ST><<<tiles * g.splits, 64 * WM_ * WN_, smem, stream>>>(g);
     XR_CHECK_LAUNCH("gemm_tile_async");
-    if (g.splits > 1) {
+    if (g.norm_whole) {
+        k_gemm_finish_norm<<<(unsigned)g.M, 1024, 0, stream>>>(g);
+        XR_CHECK_LAUNCH("gemm_finish_norm");
+    } else if (g.splits > 1 || g.raw) {
         size_t n = (size_t)g.M * g.N;
         k_gemm_finish<<<(unsigned)((n + 255) / 256), 256, 0, stream>>>(g);
         XR_CHECK_LAUNCH("gemm_finish");
@@ -566,39 +660,10 @@ __global__ __launch_bounds__(64 * KSW) void k_gemm_skinny(GemmArgs g) {
                 store_out(g, tok, nn, silu_f(v[0] + bg) * (v[NWT - 1] + bu));
             }
         } else if (g.rope.q_out) {
-            // queries and keys rotated (the partner of a pair is 8 lanes away, or 1), queries to
-            // their buffer, keys and values to their pages; formulas as in k_rope_kv_write
-            const RopeFuse& rp = g.rope;
+            // rotated and cached (the partner of a pair is 8 lanes away, or 1)
             const float val = v[0] + (ok && g.bias ? g.bias[nn] : 0.f);
-            const float partner = __shfl_xor(val, rp.interleaved ? 1 : 8);
-            if (ok) {
-                const int Q = rp.H * rp.D, KV = rp.Hk * rp.D;
-                const int sec = nn < Q ? 0 : (nn < Q + KV ? 1 : 2);
-                const int rel = nn - (sec == 0 ? 0 : (sec == 1 ? Q : Q + KV));
-                const int hs = rel / rp.D, c = rel - hs * rp.D;
-                const int pos = rp.positions[tok];
-                int d = c;
-                float o = val;
-                if (sec < 2 && c < rp.rot) {
-                    int j, hi;
-                    if (rp.interleaved) { j = c >> 1; hi = c & 1; }
-                    else { hi = (c >> 3) & 1; j = (c >> 4) * 8 + (c & 7); d = j + hi * (rp.rot >> 1); }
-                    const float ang = (float)pos * rp.inv_freq[j];
-                    const float cs = cosf(ang) * rp.mscale, sn = sinf(ang) * rp.mscale;
-                    const float x0 = hi ? partner : val, x1 = hi ? val : partner;
-                    o = hi ? x0 * sn + x1 * cs : x0 * cs - x1 * sn;
-                }
-                if (sec == 0) {
-                    rp.q_out[((size_t)tok * rp.H + hs) * rp.D + d] = f32_to_bf16(o);
-                } else {
-                    const PageRef pr = page_of(rp.block_table, rp.table_stride, rp.req_of_token[tok], pos,
-                                               rp.page_shift, rp.page_mask);
-                    if (sec == 1)
-                        rp.k_cache[(((size_t)pr.page * rp.Hk + hs) * rp.page_size + pr.off) * rp.D + d] = f32_to_bf16(o);
-                    else
-                        rp.v_cache[(((size_t)pr.page * rp.Hk + hs) * rp.D + d) * rp.page_size + pr.off] = f32_to_bf16(o);
-                }
-            }
+            const float partner = __shfl_xor(val, g.rope.interleaved ? 1 : 8);
+            if (ok) rope_store(g.rope, tok, nn, val, partner);
         } else if (g.xg) {
             // the rows of the residual stream after this product, their weighted copy for the next
             // product, and the sums of their squares over each 16 columns (16 lanes side by side)
@@ -710,24 +775,39 @@ extern "C" int xr_gemm_bf16(void* out, const void* a, const void* w, const float
     g.a = (const bf16_t*)a; g.w = (const bf16_t*)w; g.w_packed = w_packed ? 1 : 0; g.bias = bias; g.out = out;
     g.M = M; g.N = N; g.K = K; g.lda = lda; g.ldo = ldo; g.out_bf16 = out_dtype == XR_BF16; g.epi = epi;
     g.m_fast = 0; g.splits = 1; g.k_per_split = 0; g.partial = workspace; g.col0 = 0; g.col1 = N;
+    g.raw = 0; g.norm_whole = 0;
     g.ss_in = nullptr; g.n_ss = 0; g.ss_inv_width = 0.f; g.ss_eps = 0.f;
     g.norm_w = nullptr; g.norm_w_bf16 = 0; g.xg = nullptr; g.ss_out = nullptr;
     if (norm) {
-        XR_REQUIRE(M <= 16 && variant == 0, "gemm: a norm is folded only into products of at most 16 rows, got %d", M);
+        XR_REQUIRE(M <= 64 && variant == 0, "gemm: a norm is folded only into products of at most 64 rows, got %d", M);
+        XR_REQUIRE(M <= 16 || !norm->ss_in, "gemm: rows that lack their norm's scale: at most 16, got %d", M);
         if (norm->ss_in) {
             XR_REQUIRE(norm->n_ss > 0 && norm->ss_inv_width > 0.f, "gemm: bad partial sums of squares (%d of them)", norm->n_ss);
             g.ss_in = norm->ss_in; g.n_ss = norm->n_ss; g.ss_inv_width = norm->ss_inv_width; g.ss_eps = norm->ss_eps;
         }
         if (norm->xg) {
-            XR_REQUIRE(epi == EPI_ACCUM && norm->norm_w && norm->ss_out, "gemm: the norm after a product needs the accumulating epilogue, a weight and room for the sums");
-            XR_REQUIRE(norm->ss_out_rows >= (N + 15) / 16, "gemm: room for %d partial sums of squares, %d needed", norm->ss_out_rows, (N + 15) / 16);
+            XR_REQUIRE(epi == EPI_ACCUM && norm->norm_w, "gemm: the norm after a product needs the accumulating epilogue and a weight");
+            XR_REQUIRE(M > 16 || (norm->ss_out && norm->ss_out_rows >= (N + 15) / 16),
+                       "gemm: room for %d partial sums of squares, %d needed", norm->ss_out ? norm->ss_out_rows : 0, (N + 15) / 16);
             g.norm_w = norm->norm_w; g.norm_w_bf16 = norm->norm_w_bf16; g.xg = (bf16_t*)norm->xg; g.ss_out = norm->ss_out;
+            if (M > 16) {
+                // 17 to 64 rows: the finishing kernel of the split product writes the whole norm
+                XR_REQUIRE(N % 4 == 0 && ldo % 4 == 0 && workspace && (size_t)M * N * 4 <= workspace_bytes,
+                           "gemm: the norm after a product of %d rows needs a width (%d) that is a multiple of 4 and a workspace", M, N);
+                XR_REQUIRE(norm->ss_inv_width > 0.f, "gemm: the norm's width is missing");
+                g.norm_whole = 1; g.raw = 1; g.ss_inv_width = norm->ss_inv_width; g.ss_eps = norm->ss_eps;
+                norm->ss_out_rows = -1;       // tells the caller that xg holds the finished norm
+            }
         }
     }
     g.rope.q_out = nullptr;
     if (rope) {
-        XR_REQUIRE(M <= 16 && variant == 0 && epi == EPI_STORE && !(norm && norm->xg),
-                   "gemm: rotation and cache write are folded only into a plain product of at most 16 rows");
+        XR_REQUIRE(M <= 64 && variant == 0 && epi == EPI_STORE && !(norm && norm->xg),
+                   "gemm: rotation and cache write are folded only into a plain product of at most 64 rows");
+        if (M > 16) {
+            XR_REQUIRE(workspace && (size_t)M * N * 4 <= workspace_bytes, "gemm: rotation after a product of %d rows needs a workspace", M);
+            g.raw = 1;
+        }
         XR_REQUIRE(rope->H >= 0 && rope->Hk >= 0 && rope->D > 0 && rope->D % 16 == 0 && N == (rope->H + 2 * rope->Hk) * rope->D,
                    "gemm: %d columns are not %d query and 2 x %d key/value heads of a size (%d) that is a multiple of 16",
                    N, rope->H, rope->Hk, rope->D);

@@ -239,6 +239,7 @@ class Ops:
 
     # -- matrix product ---------------------------------------------------------
     GEMM_WORKSPACE_BYTES = 32 << 20
+    FINISH_ROWS = 64        # up to here a product's epilogue may be the kernel that adds its K ranges up
 
     def _gemm_workspace(self, device):
         """Room for the sums of K ranges when a product with few rows is split (one buffer per process;
@@ -333,22 +334,31 @@ class Ops:
         With ``defer`` the caller says that what reads the result is a ``linear`` or
         ``linear_swiglu``: for at most 16 bfloat16 rows the product's kernel then also writes the
         weighted rows and their partial sums of squares, and an ``UnscaledRows`` comes back, whose
-        scale the next product applies; two launches of the norm's own kernel are saved.  In
-        every other case the norm's kernel runs and a tensor comes back."""
+        scale the next product applies.  From 17 to 64 rows the kernel that adds up the product's K
+        ranges takes whole rows and writes the finished norm.  In every other case the norm's own
+        kernel runs.  A tensor comes back in both."""
         wt = w.data if isinstance(w, PackedWeight) else w
         rows = a.data if isinstance(a, UnscaledRows) else a
         M, N = rows.shape[0], w.shape[0]
-        if (defer and self.fold_norms and M <= UnscaledRows.MAX_ROWS and out_dtype == torch.bfloat16 and norm_weight is not None
+        fits = (self.fold_norms and out_dtype == torch.bfloat16 and norm_weight is not None
                 and N % 8 == 0 and norm_weight.numel() == N and norm_weight.is_contiguous()
-                and residual.dtype == torch.float32 and self._mfma_ok(rows, wt)):
+                and residual.dtype == torch.float32 and self._mfma_ok(rows, wt))
+        deferred = fits and defer and M <= UnscaledRows.MAX_ROWS
+        # 17 to 64 rows: the product is split over K anyway, and the kernel that adds the parts
+        # up takes whole rows and writes the finished norm
+        whole = fits and UnscaledRows.MAX_ROWS < M <= self.FINISH_ROWS and residual.stride(0) % 4 == 0
+        if deferred or whole:
             self._dev(norm_weight)
             then = _GemmNorm()
             xg = torch.empty((M, N), dtype=torch.bfloat16, device=rows.device)
             parts = -(-N // 16)
-            sumsq = torch.empty((parts, 16), dtype=torch.float32, device=rows.device)
+            sumsq = torch.empty((parts, 16), dtype=torch.float32, device=rows.device) if deferred else None
             then.norm_w, then.norm_w_bf16 = norm_weight.data_ptr(), dtype_code(norm_weight.dtype)
-            then.xg, then.ss_out, then.ss_out_rows = xg.data_ptr(), sumsq.data_ptr(), parts
+            then.xg, then.ss_out, then.ss_out_rows = xg.data_ptr(), _ptr(sumsq), parts
+            then.ss_inv_width, then.ss_eps = 1.0 / N, float(eps)
             self.linear(a, w, bias=bias, out=residual, accumulate=True, _then=then)
+            if then.ss_out_rows < 0:
+                return xg                                   # the finished norm
             return UnscaledRows(xg, sumsq[:then.ss_out_rows], eps)
         self.linear(a, w, bias=bias, out=residual, accumulate=True)
         return self.rmsnorm(residual, norm_weight, eps, out_dtype)
@@ -420,15 +430,17 @@ class Ops:
         ``w`` holds ``H`` query heads, then ``Hk`` key heads and ``Hk`` value heads (``Hk`` = 0 and
         no caches: queries alone); with ``paired`` its query and key rows are in ``paired_order``.
         Up to 16 bfloat16 rows (``h`` may be an ``UnscaledRows``) the product's kernel rotates and
-        stores its own result, which saves a kernel and the 32-bit copy of the projections;
-        otherwise the product and ``rope_kv_write`` run one after the other."""
+        stores its own result, up to 64 the kernel that adds the product's K ranges up does,
+        which saves a kernel and the 32-bit copy of the projections; otherwise the product and
+        ``rope_kv_write`` run one after the other."""
         rows = h.data if isinstance(h, UnscaledRows) else h
         wt = w.data if isinstance(w, PackedWeight) else w
         T, Q, KV = rows.shape[0], H * D, Hk * D
         if w.shape[0] != Q + 2 * KV:
             raise KernelError(f"projection has {w.shape[0]} rows, {H} query and 2 x {Hk} key/value heads of {D} need {Q + 2 * KV}")
         q = torch.empty((T, Q), dtype=rows.dtype, device=rows.device)
-        if (self.fuse_rope and T <= UnscaledRows.MAX_ROWS and self._mfma_ok(rows, wt) and D % 16 == 0
+        if (self.fuse_rope and T <= self.FINISH_ROWS and self._mfma_ok(rows, wt) and D % 16 == 0
+                and T * w.shape[0] * 4 <= self.GEMM_WORKSPACE_BYTES
                 and (Hk == 0 or (k_cache.dtype == torch.bfloat16 and v_cache.dtype == torch.bfloat16))
                 and (rot == 0 or interleaved or (paired and rot % 16 == 0))):
             self._dev(rows, wt, bias, k_cache, v_cache, positions, req_of_token, block_table, inv_freq)
