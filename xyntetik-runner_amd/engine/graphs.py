@@ -108,17 +108,17 @@ class StaticDecodeContext:
             if torch.cuda.is_current_stream_capturing():
                 raise RuntimeError("an attention plan was first asked for during graph capture")
             self._plan_keys.append(key)
-            entries, rcs = self._last
             self._alloc()
-            self.fill(entries, rcs)
+            self.fill(*self._last)
         return self._plans[key]
 
     # ------------------------------------------------------------------ per step
-    def fill(self, entries: List[StepEntry], rcs) -> None:
-        """Write this step's data into the pinned buffer and copy it to the device."""
+    def fill(self, entries: List[StepEntry], rcs, token_source: Optional[torch.Tensor] = None) -> None:
+        """Write this step's data into the pinned buffer and copy it to the device; the tokens
+        come from ``token_source`` (on the device) if there is one."""
         if self._copied is not None:
             self._copied.synchronize()          # the last copy has read the pinned buffer
-        self._last = (entries, rcs)
+        self._last = (entries, rcs, token_source)
         B, S, o = self.B, self.S, self._offs
         n = len(entries)
         h = self._host.numpy()
@@ -167,6 +167,8 @@ class StaticDecodeContext:
         ev = torch.cuda.Event()
         ev.record()
         self._copied = ev
+        if token_source is not None:
+            self.token_ids[:n].copy_(token_source)
 
     def _fill_plan(self, h, base: int, key, starts) -> None:
         group_size, window, _ = key
@@ -218,8 +220,9 @@ class DecodeGraphs:
     def applies(self, entries: List[StepEntry]) -> bool:
         return self.usable and all(len(e.tokens) == 1 for e in entries) and bucket_for(len(entries)) is not None
 
-    def run(self, entries: List[StepEntry], rcs) -> torch.Tensor:
-        """Logits ``[len(entries), V]`` of a step of single tokens (pages are reserved already)."""
+    def run(self, entries: List[StepEntry], rcs, token_source: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """Logits ``[len(entries), V]`` of a step of single tokens (pages are reserved already).
+        ``token_source``: the tokens, on the device (the entries' own are placeholders)."""
         r = self.runner
         n = len(entries)
         cap = bucket_for(n)
@@ -233,14 +236,14 @@ class DecodeGraphs:
         hit = self.graphs.get(key)
         if hit is not None:
             ctx, graph, logits = hit
-            ctx.fill(entries, rcs)
+            ctx.fill(entries, rcs, token_source)
             graph.replay()
             self.replays += 1
             return logits[:n]
         # first time: run the step eagerly on the static context, then record it for later
         ctx = StaticDecodeContext(r.ops, r.device, cap, S, width,
                                   windowed=[g.spec.window is not None for g in r.manager.groups])
-        ctx.fill(entries, rcs)
+        ctx.fill(entries, rcs, token_source)
         x = r.model.forward(ctx, r.storage.layers)
         out = r.model.logits(ctx, x, ctx.want_rows)
         torch.cuda.synchronize()

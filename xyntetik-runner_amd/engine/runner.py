@@ -86,11 +86,18 @@ class ModelRunner:
         return self.manager.get(req_id).n_tokens
 
     # ------------------------------------------------------------------ the step
-    def step(self, entries: Sequence[StepEntry]) -> Optional[torch.Tensor]:
-        """Run ``entries`` as one batch; logits ``[wanted, V]`` float32 on the device (None if nothing is wanted)."""
+    def step(self, entries: Sequence[StepEntry], token_source: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
+        """Run ``entries`` as one batch; logits ``[wanted, V]`` float32 on the device (None if nothing is wanted).
+
+        ``token_source`` (int32 on the device, one per entry): the entries' single tokens are
+        taken from there instead (theirs are placeholders), so that a decode step can be queued
+        before the host has seen the tokens the step before it picked.  Only for steps that a
+        recorded graph runs (``takes_token_source``)."""
         entries = [e for e in entries if len(e.tokens) > 0]
         if not entries:
             return None
+        if token_source is not None and not self.takes_token_source(entries):
+            raise ValueError("tokens on the device are taken only by a recorded decode step")
         seen = set()
         for e in entries:
             if e.req_id in seen:
@@ -112,7 +119,7 @@ class ModelRunner:
         for e, rc in zip(entries, rcs):
             mgr.reserve(e.req_id, rc.n_tokens + len(e.tokens))
         if self.graphs is not None and self.graphs.applies(entries):
-            out = self._step_graph(entries, rcs)
+            out = self._step_graph(entries, rcs, token_source)
         else:
             ctx = StepContext(self.ops, self.device, entries, rcs, len(mgr.groups))
             self._zero_fresh_state(ctx)
@@ -122,12 +129,15 @@ class ModelRunner:
             mgr.advance(e.req_id, rc.n_tokens + len(e.tokens))
         return out
 
-    def _step_graph(self, entries, rcs) -> Optional[torch.Tensor]:
+    def takes_token_source(self, entries: Sequence[StepEntry]) -> bool:
+        return self.graphs is not None and self.graphs.applies(list(entries))
+
+    def _step_graph(self, entries, rcs, token_source=None) -> Optional[torch.Tensor]:
         """A step of single tokens through a captured graph; the result is valid until the next step."""
         for e in entries:
             if any(w != 0 for w in e.want):
                 raise ValueError(f"request {e.req_id!r}: wanted place outside its one token")
-        logits = self.graphs.run(entries, rcs)
+        logits = self.graphs.run(entries, rcs, token_source)
         rows = [i for i, e in enumerate(entries) for _ in e.want]
         if not rows:
             return None

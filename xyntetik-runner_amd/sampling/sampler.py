@@ -20,15 +20,24 @@ class Sampler:
         ex = list(exempt_ids)[:12]
         self.exempt = torch.tensor(ex, dtype=torch.int32, device=device) if ex else None
 
+    @staticmethod
+    def uses_history(states: List[SamplerState]) -> bool:
+        """Whether a row's pick depends on the tokens its request got before (a repeat penalty)."""
+        return any((not s.params.greedy) and s.params.repeat_penalty != 1.0 for s in states)
+
     def sample(self, logits: torch.Tensor, states: List[SamplerState]) -> List[int]:
         """``logits [W, V]`` float32 on the device, one state per row -> token ids."""
-        W = logits.shape[0]
-        assert W == len(states)
-        if W == 0:
+        if logits.shape[0] == 0:
             return []
+        return [int(t) for t in self.launch(logits, states).cpu().tolist()]
+
+    def launch(self, logits: torch.Tensor, states: List[SamplerState]) -> torch.Tensor:
+        """The same without waiting for the result: token ids ``[W]`` int32 on the device."""
+        W = logits.shape[0]
+        assert W == len(states) and W > 0
         all_greedy = all(s.params.greedy for s in states)
         # floats: temp, top_p, min_p, rp, draw ; ints: top_k, n_recent ; window
-        need_window = any((not s.params.greedy) and s.params.repeat_penalty != 1.0 for s in states)
+        need_window = self.uses_history(states)
         nf = 5 * W
         ni = 2 * W + (W * RECENT_WINDOW if need_window else 0)
         host = torch.empty((nf + ni,), dtype=torch.int32, pin_memory=True)
@@ -57,4 +66,4 @@ class Sampler:
                 logits, f[0], f[4], top_k=i[:W], top_p=f[1], min_p=f[2], repeat_penalty=f[3],
                 recent=i[2 * W:].view(W, RECENT_WINDOW) if need_window else None,
                 n_recent=i[W:2 * W] if need_window else None, exempt=self.exempt)
-        return [int(t) for t in out.cpu().tolist()]
+        return out
