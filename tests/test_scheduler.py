@@ -151,3 +151,16 @@ def test_no_starvation_under_random_load():
         assert len(ids) == len(set(ids))
     assert all(r.finished and r.finish_reason == "length" for r in reqs), [(r.id, r.finish_reason) for r in reqs]
     assert m.free_pages() == 12
+
+
+def test_a_slice_of_a_requests_tokens():
+    """Prompt and output are two lists; a slice across them equals the slice of both together."""
+    req = Request("r", [5, 6, 7, 8], SamplingParams())
+    req.output.extend([20, 21, 22])
+    whole = req.tokens
+    assert whole == [5, 6, 7, 8, 20, 21, 22] and req.n_tokens == 7
+    for a in range(9):
+        for b in range(a, 10):
+            assert req.token_slice(a, b) == whole[a:b], (a, b)
+    req.n_computed = 5
+    assert req.remaining == 2
