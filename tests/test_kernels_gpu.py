@@ -268,6 +268,50 @@ def _unpack(data, N, K):
     return data.permute(0, 2, 1, 3).reshape(data.shape[0] * 16, data.shape[1] * 32)[:N, :K]
 
 
+def test_long_products_with_few_tiles_are_split_over_k(ops):
+    """2048 x 4096 x 14336 (a down product): 128 tiles of 256x256 would fill half the chip, so K is
+    split in two and a second kernel adds the halves into the residual stream; asked for the
+    norm that follows, that kernel writes it too and the norm's own kernel is not launched."""
+    torch.manual_seed(11)
+    M, N, K = 2048, 4096, 14336
+    a = (torch.randn(M, K, device=DEV) * 0.3).bfloat16()
+    w = (torch.randn(N, K, device=DEV) * 0.05).bfloat16()
+    pw = ops.pack_weight(w)
+    b = torch.randn(N, device=DEV) * 0.1
+    nw = (1 + 0.2 * torch.randn(N, device=DEV)).bfloat16()
+    base = torch.randn(M, N, device=DEV)
+    x = base.double() + a.double() @ w.double().T + b.double()
+    out = base.clone()
+    ops.linear(a, pw, bias=b, out=out, accumulate=True)
+    assert rel(out, x) < 1e-5
+    launches = [0]
+    plain_norm = ops.rmsnorm
+    def counting(*args, **kw):
+        launches[0] += 1
+        return plain_norm(*args, **kw)
+    out2 = base.clone()
+    try:
+        ops.rmsnorm = counting
+        h = ops.linear_add_rmsnorm(a, pw, out2, nw, 1e-5, torch.bfloat16, bias=b)
+    finally:
+        del ops.rmsnorm
+    assert launches[0] == 0 and torch.equal(out2, out)
+    want = x * torch.rsqrt((x * x).mean(1, keepdim=True) + 1e-5) * nw.double()
+    assert h.dtype == torch.bfloat16 and rel(h, want) < 6e-3
+    # a product the library does not split: the same call runs the norm's kernel
+    a2 = (torch.randn(300, 64, device=DEV)).bfloat16()
+    w2 = (torch.randn(N, 64, device=DEV) * 0.1).bfloat16()
+    r2 = torch.randn(300, N, device=DEV)
+    x2 = r2.double() + a2.double() @ w2.double().T
+    try:
+        ops.rmsnorm = counting
+        h2 = ops.linear_add_rmsnorm(a2, w2, r2, nw, 1e-5, torch.bfloat16)
+    finally:
+        del ops.rmsnorm
+    assert launches[0] == 1 and rel(r2, x2) < 1e-5
+    assert rel(h2, x2 * torch.rsqrt((x2 * x2).mean(1, keepdim=True) + 1e-5) * nw.double()) < 6e-3
+
+
 def test_pack_weight_leaves_what_the_mfma_kernels_do_not_take(ops):
     w = torch.randn(40, 20, device=DEV).bfloat16()                      # width no multiple of 8
     assert ops.pack_weight(w) is w

@@ -776,10 +776,11 @@ extern "C" int xr_gemm_bf16(void* out, const void* a, const void* w, const float
     g.M = M; g.N = N; g.K = K; g.lda = lda; g.ldo = ldo; g.out_bf16 = out_dtype == XR_BF16; g.epi = epi;
     g.m_fast = 0; g.splits = 1; g.k_per_split = 0; g.partial = workspace; g.col0 = 0; g.col1 = N;
     g.raw = 0; g.norm_whole = 0;
+    bool want_whole_norm = false;      // a norm after a product of more than 16 rows is asked for and possible
     g.ss_in = nullptr; g.n_ss = 0; g.ss_inv_width = 0.f; g.ss_eps = 0.f;
     g.norm_w = nullptr; g.norm_w_bf16 = 0; g.xg = nullptr; g.ss_out = nullptr;
     if (norm) {
-        XR_REQUIRE(M <= 64 && variant == 0, "gemm: a norm is folded only into products of at most 64 rows, got %d", M);
+        XR_REQUIRE(variant == 0, "gemm: a norm is folded only into a product whose kernel the library chooses");
         XR_REQUIRE(M <= 16 || !norm->ss_in, "gemm: rows that lack their norm's scale: at most 16, got %d", M);
         if (norm->ss_in) {
             XR_REQUIRE(norm->n_ss > 0 && norm->ss_inv_width > 0.f, "gemm: bad partial sums of squares (%d of them)", norm->n_ss);
@@ -791,12 +792,14 @@ extern "C" int xr_gemm_bf16(void* out, const void* a, const void* w, const float
                        "gemm: room for %d partial sums of squares, %d needed", norm->ss_out ? norm->ss_out_rows : 0, (N + 15) / 16);
             g.norm_w = norm->norm_w; g.norm_w_bf16 = norm->norm_w_bf16; g.xg = (bf16_t*)norm->xg; g.ss_out = norm->ss_out;
             if (M > 16) {
-                // 17 to 64 rows: the finishing kernel of the split product writes the whole norm
-                XR_REQUIRE(N % 4 == 0 && ldo % 4 == 0 && workspace && (size_t)M * N * 4 <= workspace_bytes,
-                           "gemm: the norm after a product of %d rows needs a width (%d) that is a multiple of 4 and a workspace", M, N);
+                // The kernel that adds up the K ranges of a split product takes whole rows and writes the
+                // finished norm: always from 17 to 64 rows; above, if the product is split (else the
+                // request is declined: ss_out_rows stays as it is and the caller runs the norm's kernel).
                 XR_REQUIRE(norm->ss_inv_width > 0.f, "gemm: the norm's width is missing");
-                g.norm_whole = 1; g.raw = 1; g.ss_inv_width = norm->ss_inv_width; g.ss_eps = norm->ss_eps;
-                norm->ss_out_rows = -1;       // tells the caller that xg holds the finished norm
+                want_whole_norm = N % 4 == 0 && ldo % 4 == 0 && workspace && (size_t)M * N * 4 <= workspace_bytes;
+                XR_REQUIRE(want_whole_norm || M > 64, "gemm: the norm after a product of %d rows needs a width (%d) that is a multiple of 4 and a workspace", M, N);
+                g.ss_inv_width = norm->ss_inv_width; g.ss_eps = norm->ss_eps;
+                if (M <= 64) { g.norm_whole = 1; g.raw = 1; norm->ss_out_rows = -1; }
             }
         }
     }
@@ -871,6 +874,26 @@ extern "C" int xr_gemm_bf16(void* out, const void* a, const void* w, const float
                     if (!usable(cands[j]) || cols % width(cands[j])) continue;
                     const double t = time_of(cands[i], cols) + time_of(cands[j], N - cols);
                     if (t < 0.97 * t_best) { best = i; second = j; cols_first = cols; t_best = t; }
+                }
+            }
+            // Few large tiles and a long K (the down product): 256x256 tiles with K split in two or
+            // more, and the kernel that adds the parts up (which also writes the norm that follows,
+            // if one was asked for).  Times here are in products of a tile at full rate; the adding
+            // kernel moves (ranges + 2) x M x N x 4 bytes at about 4.5 TB/s, a tile does about
+            // 4 TFLOP/s.  Measured (2048 x 4096 x 14336): 264 us against 281 us with 256x128 tiles.
+            if (!sw && workspace && count(cands[0], N) <= 128 && count(cands[0], N) >= 64) {
+                const int s2 = pick_splits(count(cands[0], N));
+                if (s2 >= 2) {
+                    const double unit = 0.5e-12;       // seconds per product-column of a 256x256 tile's row
+                    const double adding = ((double)(s2 + 2) * M * N * 4 / 4.5e12 + 3e-6) / unit;
+                    const double saved = want_whole_norm ? 11e-6 / unit : 0.0;
+                    const double t = 65536.0 * K / s2 + adding - saved;
+                    if (t < 0.97 * t_best * K) {
+                        g.m_fast = 1;
+                        g.splits = s2;
+                        if (want_whole_norm) { g.norm_whole = 1; norm->ss_out_rows = -1; }
+                        return launch_tile_variant(14, g, stream);
+                    }
                 }
             }
             variant = cands[best].variant;

@@ -238,7 +238,7 @@ class Ops:
         return out
 
     # -- matrix product ---------------------------------------------------------
-    GEMM_WORKSPACE_BYTES = 32 << 20
+    GEMM_WORKSPACE_BYTES = 96 << 20
     FINISH_ROWS = 64        # up to here a product's epilogue may be the kernel that adds its K ranges up
 
     def _gemm_workspace(self, device):
@@ -344,9 +344,10 @@ class Ops:
                 and N % 8 == 0 and norm_weight.numel() == N and norm_weight.is_contiguous()
                 and residual.dtype == torch.float32 and self._mfma_ok(rows, wt))
         deferred = fits and defer and M <= UnscaledRows.MAX_ROWS
-        # 17 to 64 rows: the product is split over K anyway, and the kernel that adds the parts
-        # up takes whole rows and writes the finished norm
-        whole = fits and UnscaledRows.MAX_ROWS < M <= self.FINISH_ROWS and residual.stride(0) % 4 == 0
+        # More rows: where the product is split over K (always from 17 to 64 rows, above that when
+        # its tiles are few and K is long), the kernel that adds the parts up takes whole rows and
+        # writes the finished norm; the library says whether it did.
+        whole = fits and M > UnscaledRows.MAX_ROWS and N % 4 == 0 and residual.stride(0) % 4 == 0
         if deferred or whole:
             self._dev(norm_weight)
             then = _GemmNorm()
@@ -359,7 +360,9 @@ class Ops:
             self.linear(a, w, bias=bias, out=residual, accumulate=True, _then=then)
             if then.ss_out_rows < 0:
                 return xg                                   # the finished norm
-            return UnscaledRows(xg, sumsq[:then.ss_out_rows], eps)
+            if deferred:
+                return UnscaledRows(xg, sumsq[:then.ss_out_rows], eps)
+            return self.rmsnorm(residual, norm_weight, eps, out_dtype)      # the library declined
         self.linear(a, w, bias=bias, out=residual, accumulate=True)
         return self.rmsnorm(residual, norm_weight, eps, out_dtype)
 
