@@ -873,7 +873,7 @@ extern "C" int xr_gemm_bf16(void* out, const void* a, const void* w, const float
                 for (int j = i + 1; j < 4; ++j) {
                     if (!usable(cands[j]) || cols % width(cands[j])) continue;
                     const double t = time_of(cands[i], cols) + time_of(cands[j], N - cols);
-                    if (t < 0.97 * t_best) { best = i; second = j; cols_first = cols; t_best = t; }
+                    if (t < 0.92 * t_best) { best = i; second = j; cols_first = cols; t_best = t; }   // (a second launch costs a little, too)
                 }
             }
             // Few large tiles and a long K (the down product): 256x256 tiles with K split in two or
