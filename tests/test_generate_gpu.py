@@ -229,6 +229,34 @@ def test_decode_steps_queued_ahead_change_nothing(folders, dtype):
     assert len(results[True][4]) == 16
 
 
+def test_an_engine_is_used_again_and_a_request_is_aborted_while_a_step_is_queued_ahead(folders):
+    """Generations one after the other on one engine (a step queued ahead for requests that have
+    all ended is forgotten), and a request taken out between two steps while the next step,
+    with its row in it, is already queued: the others go on as if it had never been there."""
+    from xyntetik_runner_amd.engine import Engine, ModelRunner
+    from xyntetik_runner_amd.sampling import SamplingParams
+    cfg, w = P.load_folder(folders["A"])
+    prompts = [prompt_ids(n, 256, 60 + i) for i, n in enumerate([11, 23, 8])]
+    refs = [P.greedy(cfg, w, p, 12) for p in prompts]
+    runner = ModelRunner.from_folder(folders["A"], dtype="float32", max_tokens=512, page_size=16, max_requests=4)
+    eng = Engine(runner, stop_ids=[])
+    sp = SamplingParams(max_new_tokens=12)
+    assert eng.generate(prompts[:2], sp) == refs[:2]
+    assert eng.generate(prompts[1:], sp) == refs[1:]                  # again, with what the first left behind
+    assert eng.stats.steps_ahead > 0
+    ids = [eng.add_request(p, sp) for p in prompts]
+    for _ in range(5):
+        eng.step()
+    assert eng._ahead is not None                                     # a step with all three rows is on its way
+    eng.scheduler.abort(eng.requests[ids[1]])
+    while eng.has_work():
+        eng.step()
+    assert [eng.requests[i].output for i in (ids[0], ids[2])] == [refs[0], refs[2]]
+    assert len(eng.requests[ids[1]].output) < 12
+    runner.manager.check()
+    assert not runner.manager.requests and runner.manager.free_pages() == runner.manager.pages_per_group
+
+
 def test_stop_token_ends_a_request(folders):
     from xyntetik_runner_amd.engine import Engine, ModelRunner
     from xyntetik_runner_amd.sampling import SamplingParams
