@@ -17,6 +17,11 @@
 // Epilogues: store (float or bfloat16), add into a float output (the residual stream),
 // and SwiGLU: with w = [gate rows; up rows] the kernel writes silu(gate) * up, so the
 // [M, 2F] intermediate never reaches memory (/root/reference/src/model.c:6399-6404).
+// Up to 64 rows two more things ride on a product, in the skinny kernel's epilogue (up to 16
+// rows) or in the kernel that adds up a split product's K ranges: the RMSNorm that follows a
+// product into the residual stream (/root/reference/src/model.c:3386-3392), and for the
+// q/k/v product the rotation of queries and keys and the write of keys and values to their
+// pages (RopeFuse), so that a decode step launches 6 kernels a layer.
 // The reference's float-weight "GEMM" is a multi-column matvec (/root/reference/src/kernels.cu:116-144);
 // its tensor-core kernels (:856) exist for quantised weights only.
 #include "common.h"
