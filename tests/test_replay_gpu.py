@@ -255,3 +255,43 @@ def test_decoding_with_norms_folded_into_the_products(models, which):
     for fold in (True, False):
         mx, mean = logit_error(outs[fold], want["r3"][n0:])
         assert mx <= TOL["bfloat16"][0] and mean <= TOL["bfloat16"][1], (fold, mx, mean)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_the_references_batch_workload(models, dtype):
+    """The workload of the reference's own batching test (/root/reference/tests/test_batch.c:49-60,
+    :203-215): 8 sequences with prompts of 5, 11, 8, 17, 6, 14, 9 and 20 tokens, ids
+    ((seq+1)*7919 + i*104729) mod V, 24 greedy steps, decoded 1, 2, 4 and 8 at a time, so that
+    every sequence of a batch sits at another position in every step.  Whole logits rows are
+    compared, not only tokens, and they must not be all zero (its anti-vacuity rule)."""
+    from xyntetik_runner_amd.engine.batch import StepEntry
+    from xyntetik_runner_amd.engine.runner import ModelRunner
+    d, cfg, _, _, _ = models["A"]
+    _, w = P.load_folder(d)
+    V, steps = cfg["vocab_size"], 24
+    plen = [5, 11, 8, 17, 6, 14, 9, 20]
+    prompts = [[((s + 1) * 7919 + i * 104729) % V for i in range(n)] for s, n in enumerate(plen)]
+    full = [p + P.greedy(cfg, w, p, steps) for p in prompts]
+    want = [P.forward(cfg, w, toks[:-1]) for toks in full]                  # row t: logits after token t
+    runner = ModelRunner.from_folder(d, dtype=dtype, max_tokens=8 * 64, page_size=16, max_requests=8)
+    for width in (1, 2, 4, 8):
+        for g0 in range(0, 8, width):
+            group = list(range(g0, g0 + width))
+            got = {s: [] for s in group}
+            out = runner.step([StepEntry(s, prompts[s], [plen[s] - 1]) for s in group])
+            for r, s in enumerate(group):
+                got[s].append(out[r].cpu().numpy())
+            for k in range(steps - 1):
+                out = runner.step([StepEntry(s, [full[s][plen[s] + k]], [0]) for s in group])
+                for r, s in enumerate(group):
+                    got[s].append(out[r].cpu().numpy())
+            for s in group:
+                rows = np.stack(got[s])
+                assert np.abs(rows).max() > 0
+                mx, mean = logit_error(rows, want[s][plen[s] - 1:])
+                assert mx <= TOL[dtype][0] and mean <= TOL[dtype][1], (width, s, mx, mean)
+                if dtype == "float32":                                      # and the greedy tokens are the same
+                    assert [int(np.argmax(r)) for r in rows] == full[s][plen[s]:]
+                runner.finish(s)
+        runner.manager.check()
+        assert runner.manager.free_pages() == runner.manager.pages_per_group
