@@ -295,3 +295,14 @@ def test_the_references_batch_workload(models, dtype):
                 runner.finish(s)
         runner.manager.check()
         assert runner.manager.free_pages() == runner.manager.pages_per_group
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("page_size", [1, 2])
+def test_the_smallest_pages(models, tmp_path, dtype, page_size):
+    """Pages of one and of two positions: every key has its own entry in the block table."""
+    d, cfg, reqs, plens, want = models["A"]
+    few = {rid: reqs[rid] for rid in ("r0", "r1", "r2")}
+    steps = traces.mixed(few, plens, max_live=3, seed=page_size)
+    out, runner = run_replay(d, dtype, steps, tmp_path, page_size)
+    check(traces.collect(steps, out, cfg["vocab_size"]), {rid: want[rid] for rid in few}, dtype, f"pages of {page_size}")
