@@ -89,6 +89,9 @@ def test_sampling_kernel_matches_plain_sampler():
     cases.append((64, all_equal, dict(temp=1.0, draw=0.5, top_k=0, top_p=1.0, min_p=0.0, repeat_penalty=1.0, recent=[])))
     cases.append((64, all_equal, dict(temp=1.0, draw=0.99, top_k=10, top_p=1.0, min_p=0.0, repeat_penalty=1.0, recent=[])))
     cases.append((64, all_equal, dict(temp=0.0, draw=0.99, top_k=0, top_p=1.0, min_p=0.0, repeat_penalty=1.0, recent=[])))
+    # the reference's own penalty vector (/root/reference/tests/test_sampler.c:200-206): token 1
+    cases.append((4, np.array([10.0, 9.0, 1.0, 0.5], dtype=np.float32),
+                  dict(temp=0.01, draw=0.7, top_k=0, top_p=1.0, min_p=0.0, repeat_penalty=2.0, recent=[0])))
     exempt = [3]
     for V, lg, kw in cases:
         want = P.sample_pick(lg, kw["temp"], kw["draw"], kw["top_k"], kw["top_p"], kw["min_p"],
@@ -129,6 +132,9 @@ def test_sampling_kernel_distribution_and_many_rows():
     mixed_t = torch.tensor([0.0, 1.0] * (n // 2), device=dev)
     got2 = ops.sample(rows, mixed_t, torch.tensor(draws, dtype=torch.float32, device=dev)).cpu().numpy()
     assert np.all(got2[0::2] == 5) and np.array_equal(got2[1::2], got[1::2])
+    # a temperature near zero picks like greedy whatever is drawn (/root/reference/tests/test_sampler.c:200-206)
+    cold = ops.sample(rows, torch.full((n,), 0.01, device=dev), torch.tensor(draws, dtype=torch.float32, device=dev))
+    assert np.all(cold.cpu().numpy() == 5)
 
 
 def test_greedy_pick_over_a_long_row_split_in_ranges():

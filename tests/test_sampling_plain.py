@@ -36,6 +36,10 @@ def test_greedy_vectors():
     assert P.sample_pick(lg, 1.0, 0.0, repeat_penalty=10.0, recent=[1]) == 0    # sampling applies it
     assert P.sample_pick(lg, 1.0, 0.0, repeat_penalty=10.0, recent=[1], exempt=[1]) == 1
     assert P.sample_pick(lg, 1.0, 0.0, repeat_penalty=10.0, recent=[7, -1, 1000]) == 1   # ids outside are ignored
+    # the reference's own vector: token 0 was seen, a penalty of 2 halves its 10 to 5, below token 1's 9,
+    # and a temperature of 0.01 leaves no choice (/root/reference/tests/test_sampler.c:200-206)
+    for draw in (0.0, 0.3, 0.999):
+        assert P.sample_pick([10.0, 9.0, 1.0, 0.5], 0.01, draw, repeat_penalty=2.0, recent=[0]) == 1
 
 
 def test_temperature_follows_softmax_and_converges_to_greedy():
