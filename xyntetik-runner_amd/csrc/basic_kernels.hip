@@ -192,22 +192,45 @@ __global__ __launch_bounds__(256) void k_rope_kv_write(RopeArgs a) {
         cs[1][j] = sinf(ang) * a.mscale;
     }
     __syncthreads();
-    const int h_end = min(a.H + a.Hk, (int)(blockIdx.y + 1) * a.heads_per_block);
-    for (int hs = blockIdx.y * a.heads_per_block + wave; hs < h_end; hs += 4) {
-        if (hs < a.H) {
-            const float* src = a.q_in + (size_t)t * a.in_stride + (size_t)hs * D;
-            T* dst = (T*)a.q_out + ((size_t)t * a.H + hs) * D;
-            for (int j = lane; j < half; j += 64) {
-                const int i0 = a.interleaved ? 2 * j : j;
-                const int i1 = a.interleaved ? 2 * j + 1 : j + half;
-                const float x0 = src[a.paired ? paired_col(i0, a.rot) : i0], x1 = src[a.paired ? paired_col(i1, a.rot) : i1];
-                const float c = cs[0][j], sn = cs[1][j];
-                st<T>(dst, i0, x0 * c - x1 * sn);
-                st<T>(dst, i1, x0 * sn + x1 * c);
-            }
-            for (int i = a.rot + lane; i < D; i += 64) st<T>(dst, i, src[i]);
-            continue;
+    const int h_begin = blockIdx.y * a.heads_per_block;
+    const int h_end = min(a.H + a.Hk, h_begin + a.heads_per_block);
+    // query heads, four at a time per wave: the loads of all four are on their way before the
+    // first is used (one head at a time, a wave waited out a memory latency per head)
+    const int hq_end = min(h_end, a.H);
+    for (int hb = h_begin + wave * 4; hb < hq_end; hb += 16) {
+        const float* src[4];
+        T* dst[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const int hs = hb + u < hq_end ? hb + u : hb;
+            src[u] = a.q_in + (size_t)t * a.in_stride + (size_t)hs * D;
+            dst[u] = (T*)a.q_out + ((size_t)t * a.H + hs) * D;
         }
+        for (int j = lane; j < half; j += 64) {
+            const int i0 = a.interleaved ? 2 * j : j;
+            const int i1 = a.interleaved ? 2 * j + 1 : j + half;
+            const int c0 = a.paired ? paired_col(i0, a.rot) : i0, c1 = a.paired ? paired_col(i1, a.rot) : i1;
+            float x0[4], x1[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) { x0[u] = src[u][c0]; x1[u] = src[u][c1]; }
+            const float c = cs[0][j], sn = cs[1][j];
+#pragma unroll
+            for (int u = 0; u < 4; ++u)
+                if (hb + u < hq_end) {
+                    st<T>(dst[u], i0, x0[u] * c - x1[u] * sn);
+                    st<T>(dst[u], i1, x0[u] * sn + x1[u] * c);
+                }
+        }
+        for (int i = a.rot + lane; i < D; i += 64) {
+            float x[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) x[u] = src[u][i];
+#pragma unroll
+            for (int u = 0; u < 4; ++u)
+                if (hb + u < hq_end) st<T>(dst[u], i, x[u]);
+        }
+    }
+    for (int hs = max(h_begin, a.H) + wave; hs < h_end; hs += 4) {
         const int kvh = hs - a.H;
         const int req = a.req_of_token[t];
         PageRef pr = page_of(a.block_table, a.table_stride, req, pos, a.page_shift, a.page_mask);
