@@ -295,7 +295,7 @@ def test_long_products_with_few_tiles_are_split_over_k(ops):
         h = ops.linear_add_rmsnorm(a, pw, out2, nw, 1e-5, torch.bfloat16, bias=b)
     finally:
         del ops.rmsnorm
-    assert launches[0] == 0 and torch.equal(out2, out)
+    assert launches[0] == 0 and rel(out2, x) < 1e-5      # (the product alone may take other tiles: another order of 32-bit sums)
     want = x * torch.rsqrt((x * x).mean(1, keepdim=True) + 1e-5) * nw.double()
     assert h.dtype == torch.bfloat16 and rel(h, want) < 6e-3
     # a product the library does not split: the same call runs the norm's kernel

@@ -70,6 +70,7 @@ struct GemmArgs {
     int raw;           // 1: raw sums go to `partial` also when K is whole (an epilogue of k_gemm_finish is wanted)
     int norm_whole;    // 1: k_gemm_finish_norm writes the whole norm of the updated rows to xg
     int col0, col1;    // the tile kernel computes output columns col0 .. col1-1 (col0 a multiple of the tile's width)
+    int vec_out;       // 1: the tile kernel may write 4 columns a lane (widths and row strides are multiples of 4, bases 16-byte aligned)
     // RMSNorm folded into the skinny kernel (all null or zero: off).
     // Before: `a` holds rows x*weight that are not yet divided by their root mean square; ss_in
     // [n_ss][16] holds partial sums of x^2 per row, and the product's row t is scaled by
@@ -131,6 +132,11 @@ __device__ inline uint4 keep_if(bool ok, uint4 v) {
     return make_uint4(ok ? v.x : 0u, ok ? v.y : 0u, ok ? v.z : 0u, ok ? v.w : 0u);
 }
 __device__ inline float silu_f(float g) { return g / (1.0f + expf(-g)); }
+// the same with the hardware's 2^x and reciprocal (1 ulp each), for the tile kernel, where a lane
+// has 64 of them to do while nothing else runs on its compute unit
+__device__ inline float silu_fast(float g) {
+    return g * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(g * -1.44269504f));
+}
 
 __device__ inline void store_out(const GemmArgs& g, int m, int n, float v) {
     size_t o = (size_t)m * g.ldo + n;
@@ -175,6 +181,44 @@ __device__ inline void rope_store(const RopeFuse& rp, int tok, int nn, float val
         rp.v_cache[(((size_t)pr.page * rp.Hk + hs) * rp.D + d) * rp.page_size + pr.off] = f32_to_bf16(o);
 }
 
+// NT side-by-side 32x32 tiles in the accumulator layout of v_mfma_f32_32x32x16 (a lane holds one
+// column and 16 rows) go to rows m_base.., columns col_base.. of a row-major matrix through the
+// wave's own LDS area, so that a lane then holds 4 consecutive columns of one row: a store
+// instruction writes whole 128-byte runs instead of 2 or 4 bytes a lane.  (Measured on a
+// 256x256 tile with bfloat16 output: 21 us of a tile's 137 us went to 128 two-byte stores a
+// lane and their addresses.)  mode: 0 store float, 1 add into float, 2 store bfloat16.
+// A wave's LDS accesses are served in order, so it needs no barrier for an area of its own.
+constexpr int STAGE_FLOATS = 32 * (64 + 4);      // a wave's area: 32 rows of 64 columns, rows 16 bytes apart in the banks
+template <int NT>
+__device__ inline void write_tiles(float* stage, const f32x16 (&t)[NT], void* dst, int ld, int mode,
+                                   int m_base, int M, int col_base, int col_end, int lane) {
+    constexpr int SW = 32 * NT, LD = SW + 4, CPR = SW / 4, RPI = 64 / CPR;
+    const int lr = lane & 31, lg = lane >> 5;
+#pragma unroll
+    for (int n = 0; n < NT; ++n)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) stage[((e / 4) * 8 + lg * 4 + (e % 4)) * LD + n * 32 + lr] = t[n][e];
+    const int ch = lane % CPR, col = col_base + ch * 4;
+#pragma unroll
+    for (int it = 0; it < 32 / RPI; ++it) {
+        const int row = it * RPI + lane / CPR, m = m_base + row;
+        const float4 x = *reinterpret_cast<const float4*>(stage + row * LD + ch * 4);
+        if (m >= M || col >= col_end) continue;
+        const size_t o = (size_t)m * ld + col;
+        if (mode == 2) {
+            uint2 v;
+            v.x = pack_bf16x2(x.x, x.y);
+            v.y = pack_bf16x2(x.z, x.w);
+            *reinterpret_cast<uint2*>((bf16_t*)dst + o) = v;
+        } else {
+            float4* q = reinterpret_cast<float4*>((float*)dst + o);
+            float4 y = x;
+            if (mode == 1) { const float4 old = *q; y.x += old.x; y.y += old.y; y.z += old.z; y.w += old.w; }
+            *q = y;
+        }
+    }
+}
+
 // ------------------------------------------------------------------------------ tile kernel
 // Row r (0..BN-1) of the weight tile of workgroup bx -> row of w.  Plain: n0 + r.  SwiGLU:
 // each wave's 32-column MFMA tiles alternate gate, up, gate, up ... so that the two values
@@ -197,9 +241,16 @@ __device__ inline int w_row_of(int r, int bx, int N, int epi, int& out_col) {
 // kt, slices kt+1 .. kt+STAGES-1 are on their way, with no registers and no LDS-write
 // instructions spent on them.  A lane whose piece lies outside the matrices reads from a
 // block of zeros instead, so every slice issues the same number of loads and one counter
-// wait (vmcnt) tells when a slice has landed.  Measured on MI355X: what bounds the kernel is
-// the rate at which a compute unit's L1 delivers the slices (about 20 bytes a cycle), so
-// the tile with the most products per byte that still fills the chip is chosen.
+// wait (vmcnt) tells when a slice has landed.  Two main loops: in the plain one a k-step reads
+// its fragments and multiplies; with PIPE the fragments of k-step ks+1 (also the next slice's
+// first) are read into a second set of registers before the products of k-step ks are issued.
+// Measured on MI355X (8192 x 28672 x 4096, random data): a compute unit is given its operands
+// at up to 50 bytes a cycle from L2 and reads LDS at 190, the matrix cores alone do 1.8 PFLOP/s
+// (the clock falls from 2.4 to 1.8-2.0 GHz under them); a 256x256 tile spent 115 us in its loop
+// and 21 us storing its result two bytes a lane, with nothing else on its compute unit to hide
+// that (128 KB of LDS: one workgroup at a time).  So results leave through LDS, 4 columns a lane
+// (write_tiles: 21 -> 6 us, 1.0 -> 1.14 PFLOP/s), and PIPE gives another 3-5% on all tiles but
+// 256x192.
 // Where chunk c of row r lies within the row in LDS: at c ^ swz(r).  A fragment read takes
 // one column of 32 rows; LDS serves 16 lanes of 16 bytes a cycle from 64 banks of 4 bytes, so
 // 16 consecutive rows must fall into 16 different 16-byte bank groups.  Two rows of 128 bytes
@@ -207,7 +258,7 @@ __device__ inline int w_row_of(int r, int bx, int N, int epi, int& out_col) {
 // conflicts reads zero with this, and half the active cycles with a shift by the row number.)
 template <int CH> __device__ inline int swz(int r) { static_assert(CH == 8, "rows of 8 chunks"); return (r >> 1) & 7; }
 
-template <int BM, int BN, int WARPS_M, int WARPS_N, int STAGES>
+template <int BM, int BN, int WARPS_M, int WARPS_N, int STAGES, bool PIPE = false>
 __global__ __launch_bounds__(64 * WARPS_M * WARPS_N) void k_gemm_tile_async(GemmArgs g) {
     constexpr int WAVES = WARPS_M * WARPS_N;
     constexpr int BK = 64, CH = BK / 8, RPL = 64 / CH;  // chunks of a row; rows that one load instruction covers
@@ -216,7 +267,7 @@ __global__ __launch_bounds__(64 * WARPS_M * WARPS_N) void k_gemm_tile_async(Gemm
     constexpr int ROWS = BM + BN;                       // rows of one stage: activations, then weights
     constexpr int LOADS = ROWS / RPL / WAVES;           // load instructions per wave and stage
     static_assert(ROWS % (RPL * WAVES) == 0, "stage does not divide among waves");
-    static_assert(LOADS * (STAGES - 2) < 64, "too many loads in flight for the counter");
+    static_assert(LOADS * STAGES < 64, "too many loads in flight for the counter");
     constexpr int BUF = ROWS * CH;                      // chunks per stage
     extern __shared__ uint4 lds[];                      // [STAGES][BUF]
 
@@ -292,9 +343,57 @@ __global__ __launch_bounds__(64 * WARPS_M * WARPS_N) void k_gemm_tile_async(Gemm
             for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
 
     const int nk = (k_end - k_begin + BK - 1) / BK;
+    const int lr = lane & 31, lg = lane >> 5;
+    if constexpr (PIPE) {
+        // The fragments of k-step ks+1 are read into a second set of registers before the
+        // products of k-step ks are issued, also across the edge of a slice.  A buffer is free
+        // for the slice STAGES further on as soon as every wave has left its slice (the barrier
+        // in the last k-step), and the copies begin right there: a third at once, a third in
+        // each of the next two k-steps, so that the last of them are two k-steps old when waited for.
+#pragma unroll
+        for (int st = 0; st < STAGES; ++st) ASYNC_ISSUE(st)
+        wait_vmcnt<LOADS * (STAGES - 1)>();              // slice 0 has landed
+        __builtin_amdgcn_s_barrier();
+        bf16x8 af[2][TM], wf[2][TN];
+#define READ_FRAGS(BUFI, KS, F)                                                                      \
+    {                                                                                                \
+        const uint4* A_ = lds + (BUFI) * BUF;                                                        \
+        const uint4* W_ = A_ + BM * CH;                                                              \
+        const int c_ = (KS) * 2 + lg;                                                                \
+        _Pragma("unroll") for (int i = 0; i < TM; ++i) {                                             \
+            const int r = wm0 + i * 32 + lr;                                                         \
+            af[F][i] = as_bf16x8(A_[r * CH + (c_ ^ swz<CH>(r))]);                                    \
+        }                                                                                            \
+        _Pragma("unroll") for (int j = 0; j < TN; ++j) {                                             \
+            const int r = wn0 + j * 32 + lr;                                                         \
+            wf[F][j] = as_bf16x8(W_[r * CH + (c_ ^ swz<CH>(r))]);                                    \
+        }                                                                                            \
+    }
+        READ_FRAGS(0, 0, 0)
+        for (int kt = 0; kt < nk; ++kt) {
+#pragma unroll
+            for (int ks = 0; ks < 4; ++ks) {
+                if (ks < 3) {
+                    if (ks < 2 && kt > 0) ASYNC_ISSUE_PART(kt + STAGES - 1, ks + 1, 3)
+                    READ_FRAGS(kt % STAGES, ks + 1, (ks + 1) & 1)
+                } else {
+                    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // this wave no longer reads slice kt ...
+                    wait_vmcnt<LOADS * (STAGES - 2)>();                  // ... and its share of slice kt+1 has landed
+                    __builtin_amdgcn_s_barrier();
+                    ASYNC_ISSUE_PART(kt + STAGES, 0, 3)                  // into the buffer of slice kt
+                    READ_FRAGS((kt + 1) % STAGES, 0, 0)
+                }
+#pragma unroll
+                for (int i = 0; i < TM; ++i)
+#pragma unroll
+                    for (int j = 0; j < TN; ++j)
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[ks & 1][i], wf[ks & 1][j], acc[i][j], 0, 0, 0);
+            }
+        }
+#undef READ_FRAGS
+    } else {
 #pragma unroll
     for (int st = 0; st < STAGES - 1; ++st) ASYNC_ISSUE(st)
-    const int lr = lane & 31, lg = lane >> 5;
     for (int kt = 0; kt < nk; ++kt) {
         // slice kt has landed when at most the STAGES-2 younger slices are still in flight
         wait_vmcnt<LOADS * (STAGES - 2)>();
@@ -325,14 +424,34 @@ __global__ __launch_bounds__(64 * WARPS_M * WARPS_N) void k_gemm_tile_async(Gemm
                     acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[i], wf[j], acc[i][j], 0, 0, 0);
         }
     }
+    }
 #undef ASYNC_ISSUE
 #undef ASYNC_ISSUE_PART
     wait_vmcnt<0>();                                     // the trailing loads of zeros
+
+    // where 4 columns a lane may be written, the results go through LDS, each wave through an area
+    // of its own, once no wave reads operands there any more
+    static_assert((size_t)STAGES * ROWS * CH * 16 >= (size_t)WAVES * STAGE_FLOATS * 4, "no room for the waves' output areas");
+    float* stage = reinterpret_cast<float*>(lds) + wave * STAGE_FLOATS;
+    constexpr int NTP = TN % 2 == 0 ? 2 : 1;             // tiles written together
+    if (g.vec_out) __builtin_amdgcn_s_barrier();
 
     if (g.splits > 1 || g.raw) {
         // raw sums of this K range, by weight row: the epilogue belongs to k_gemm_finish
         const int ldp = g.epi == EPI_SWIGLU ? 2 * g.N : g.N;
         float* part = g.partial + (size_t)split_ * g.M * ldp;
+        if (g.vec_out && g.epi != EPI_SWIGLU) {
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int j = 0; j < TN; j += NTP) {
+                    f32x16 t[NTP];
+#pragma unroll
+                    for (int n = 0; n < NTP; ++n) t[n] = acc[i][j + n];
+                    write_tiles<NTP>(stage, t, part, ldp, 0, m0 + wm0 + i * 32, g.M, bx * BN + wn0 + j * 32, g.N, lane);
+                }
+            return;
+        }
 #pragma unroll
         for (int i = 0; i < TM; ++i)
 #pragma unroll
@@ -349,6 +468,29 @@ __global__ __launch_bounds__(64 * WARPS_M * WARPS_N) void k_gemm_tile_async(Gemm
         return;
     }
     if (g.epi == EPI_SWIGLU) {
+        if (g.vec_out) {
+            constexpr int TO = TN / 2, NTO = TO % 2 == 0 && TO > 0 ? 2 : 1;     // output tiles of a wave's row, and how many go together
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int jo = 0; jo < TO; jo += NTO) {
+                    f32x16 t[NTO];
+                    int oc0 = 0;
+#pragma unroll
+                    for (int n = 0; n < NTO; ++n) {
+                        int oc;
+                        w_row_of<BN, WN>(wn0 + (jo + n) * 64 + lr, bx, g.N, g.epi, oc);
+                        if (n == 0) oc0 = oc - lr;
+                        const bool in = oc < g.N;
+                        const float bg = g.bias && in ? g.bias[oc] : 0.f, bu = g.bias && in ? g.bias[g.N + oc] : 0.f;
+#pragma unroll
+                        for (int e = 0; e < 16; ++e)
+                            t[n][e] = silu_fast(acc[i][(jo + n) * 2][e] + bg) * (acc[i][(jo + n) * 2 + 1][e] + bu);
+                    }
+                    write_tiles<NTO>(stage, t, g.out, g.ldo, g.out_bf16 ? 2 : 0, m0 + wm0 + i * 32, g.M, oc0, g.N, lane);
+                }
+            return;
+        }
 #pragma unroll
         for (int i = 0; i < TM; ++i)
 #pragma unroll
@@ -360,8 +502,26 @@ __global__ __launch_bounds__(64 * WARPS_M * WARPS_N) void k_gemm_tile_async(Gemm
 #pragma unroll
                 for (int e = 0; e < 16; ++e) {
                     int m = m0 + wm0 + i * 32 + (e / 4) * 8 + lg * 4 + (e % 4);
-                    if (m < g.M) store_out(g, m, oc, silu_f(acc[i][j][e] + bg) * (acc[i][j + 1][e] + bu));
+                    if (m < g.M) store_out(g, m, oc, silu_fast(acc[i][j][e] + bg) * (acc[i][j + 1][e] + bu));
                 }
+            }
+        return;
+    }
+    if (g.vec_out) {
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; j += NTP) {
+                f32x16 t[NTP];
+#pragma unroll
+                for (int n = 0; n < NTP; ++n) {
+                    const int col = bx * BN + wn0 + (j + n) * 32 + lr;
+                    const float b = g.bias && col < g.N ? g.bias[col] : 0.f;
+#pragma unroll
+                    for (int e = 0; e < 16; ++e) t[n][e] = acc[i][j + n][e] + b;
+                }
+                write_tiles<NTP>(stage, t, g.out, g.ldo, g.epi == EPI_ACCUM ? 1 : (g.out_bf16 ? 2 : 0),
+                                 m0 + wm0 + i * 32, g.M, bx * BN + wn0 + j * 32, g.N, lane);
             }
         return;
     }
@@ -453,7 +613,7 @@ __global__ __launch_bounds__(1024) void k_gemm_finish_norm(GemmArgs g) {
     }
 }
 
-template <int BM, int BN, int WM_, int WN_, int ST>
+template <int BM, int BN, int WM_, int WN_, int ST, bool PIPE = false>
 static int launch_tile_async(GemmArgs g, hipStream_t stream) {
     if (g.epi == EPI_SWIGLU && (BN / WN_ / 32) % 2) {
         xr_set_error("gemm: a %dx%d tile cannot pair gate and up columns", BM, BN);
@@ -462,7 +622,7 @@ static int launch_tile_async(GemmArgs g, hipStream_t stream) {
     size_t smem = (size_t)ST * (BM + BN) * 8 * 16;
     static bool attr_set = false;
     if (!attr_set) {
-        hipError_t e = hipFuncSetAttribute((const void*)k_gemm_tile_async<BM, BN, WM_, WN_, ST>,
+        hipError_t e = hipFuncSetAttribute((const void*)k_gemm_tile_async<BM, BN, WM_, WN_, ST, PIPE>,
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
         if (e != hipSuccess) {
             (void)hipGetLastError();             // or the next launch's check would report this refusal
@@ -491,7 +651,14 @@ static int launch_tile_async(GemmArgs g, hipStream_t stream) {
         xr_set_error("gemm: no room for the raw sums of a product whose epilogue is a kernel of its own");
         return XR_BAD_ARG;
     }
-    k_gemm_tile_async<BM, BN, WM_, WN_, ST><<<tiles * g.splits, 64 * WM_ * WN_, smem, stream>>>(g);
+    {
+        // 4 columns a lane: every row of the output (and of the raw sums) must begin 16 bytes aligned
+        const bool raw_out = g.splits > 1 || g.raw;
+        const int ld = raw_out ? (g.epi == EPI_SWIGLU ? 2 * g.N : g.N) : g.ldo;
+        const void* base = raw_out ? (const void*)g.partial : (const void*)g.out;
+        g.vec_out = g.N % 4 == 0 && ld % 4 == 0 && ((uintptr_t)base % 16) == 0 && (!raw_out || ((size_t)g.M * ld) % 4 == 0);
+    }
+    k_gemm_tile_async<BM, BN, WM_, WN_, ST, PIPE><<<tiles * g.splits, 64 * WM_ * WN_, smem, stream>>>(g);
     XR_CHECK_LAUNCH("gemm_tile_async");
     if (g.norm_whole) {
         k_gemm_finish_norm<<<(unsigned)g.M, 1024, 0, stream>>>(g);
@@ -692,18 +859,22 @@ __global__ __launch_bounds__(64 * KSW) void k_gemm_skinny(GemmArgs g) {
 }
 
 static int launch_tile_variant(int variant, const GemmArgs& g, hipStream_t stream) {
-    if (variant == 10) return launch_tile_async<128, 128, 2, 2, 3>(g, stream);
-    if (variant == 11) return launch_tile_async<128, 128, 2, 2, 4>(g, stream);
-    if (variant == 12) return launch_tile_async<256, 128, 4, 2, 3>(g, stream);
-    if (variant == 13) return launch_tile_async<256, 256, 2, 4, 2>(g, stream);
-    if (variant == 14) return launch_tile_async<256, 256, 4, 2, 2>(g, stream);
-    if (variant == 15) return launch_tile_async<256, 128, 2, 2, 3>(g, stream);
-    if (variant == 16) return launch_tile_async<128, 256, 2, 4, 3>(g, stream);
-    if (variant == 17) return launch_tile_async<128, 128, 2, 2, 2>(g, stream);
-    if (variant == 18) return launch_tile_async<256, 256, 2, 2, 2>(g, stream);
-    if (variant == 19) return launch_tile_async<256, 128, 2, 2, 2>(g, stream);
-    if (variant == 20) return launch_tile_async<128, 256, 2, 2, 2>(g, stream);
+    // (the loop that reads its fragments a k-step ahead is the faster one but for the 256x192 tile)
+    if (variant == 12) return launch_tile_async<256, 128, 4, 2, 3, true>(g, stream);
+    if (variant == 14) return launch_tile_async<256, 256, 4, 2, 2, true>(g, stream);
+    if (variant == 17) return launch_tile_async<128, 128, 2, 2, 2, true>(g, stream);
     if (variant == 26) return launch_tile_async<256, 192, 4, 2, 2>(g, stream);
+#ifdef XR_GEMM_SWEEP
+    if (variant == 10) return launch_tile_async<128, 128, 2, 2, 3>(g, stream);
+    if (variant == 13) return launch_tile_async<256, 256, 2, 4, 2>(g, stream);
+    if (variant == 16) return launch_tile_async<128, 256, 2, 4, 3>(g, stream);
+    if (variant == 18) return launch_tile_async<256, 256, 2, 2, 2>(g, stream);
+    if (variant == 42) return launch_tile_async<256, 128, 4, 2, 3>(g, stream);
+    if (variant == 44) return launch_tile_async<256, 256, 4, 2, 2>(g, stream);
+    if (variant == 47) return launch_tile_async<128, 128, 2, 2, 2>(g, stream);
+    if (variant == 53) return launch_tile_async<256, 192, 4, 2, 2, true>(g, stream);
+    if (variant == 55) return launch_tile_async<64, 128, 2, 2, 3, true>(g, stream);
+#endif
     xr_set_error("gemm: unknown variant %d", variant);
     return XR_BAD_ARG;
 }
@@ -780,7 +951,7 @@ extern "C" int xr_gemm_bf16(void* out, const void* a, const void* w, const float
     g.a = (const bf16_t*)a; g.w = (const bf16_t*)w; g.w_packed = w_packed ? 1 : 0; g.bias = bias; g.out = out;
     g.M = M; g.N = N; g.K = K; g.lda = lda; g.ldo = ldo; g.out_bf16 = out_dtype == XR_BF16; g.epi = epi;
     g.m_fast = 0; g.splits = 1; g.k_per_split = 0; g.partial = workspace; g.col0 = 0; g.col1 = N;
-    g.raw = 0; g.norm_whole = 0;
+    g.raw = 0; g.norm_whole = 0; g.vec_out = 0;
     bool want_whole_norm = false;      // a norm after a product of more than 16 rows is asked for and possible
     g.ss_in = nullptr; g.n_ss = 0; g.ss_inv_width = 0.f; g.ss_eps = 0.f;
     g.norm_w = nullptr; g.norm_w_bf16 = 0; g.xg = nullptr; g.ss_out = nullptr;
@@ -861,7 +1032,7 @@ extern "C" int xr_gemm_bf16(void* out, const void* a, const void* w, const float
             // smaller one (3 rounds + 1 of half-size tiles instead of 4).  If even the smallest
             // tile does not fill the chip, K is split as well.
             struct Cand { int variant, bm, bn; double rate; };
-            const Cand cands[4] = {{14, 256, 256, 1.0}, {26, 256, 192, 0.9}, {12, 256, 128, 0.85}, {17, 128, 128, 0.78}};
+            const Cand cands[4] = {{14, 256, 256, 1.0}, {26, 256, 192, 0.93}, {12, 256, 128, 0.90}, {17, 128, 128, 0.74}};
             auto width = [&](const Cand& c) { return sw ? c.bn / 2 : c.bn; };
             auto usable = [&](const Cand& c) { return !(sw && c.variant == 26); };
             auto count = [&](const Cand& c, int cols) { return ((M + c.bm - 1) / c.bm) * ((cols + width(c) - 1) / width(c)); };
@@ -893,7 +1064,7 @@ extern "C" int xr_gemm_bf16(void* out, const void* a, const void* w, const float
                     const double adding = ((double)(s2 + 2) * M * N * 4 / 4.5e12 + 3e-6) / unit;
                     const double saved = want_whole_norm ? 11e-6 / unit : 0.0;
                     const double t = 65536.0 * K / s2 + adding - saved;
-                    if (t < 0.97 * t_best * K) {
+                    if (t < t_best * K) {
                         g.m_fast = 1;
                         g.splits = s2;
                         if (want_whole_norm) { g.norm_whole = 1; norm->ss_out_rows = -1; }
