@@ -289,21 +289,23 @@ __global__ __launch_bounds__(64 * WARPS_M * WARPS_N) void k_gemm_tile_async(Gemm
     const int n_rows = g.epi == EPI_SWIGLU ? 2 * g.N : g.N;
     const bf16_t* zero_src = reinterpret_cast<const bf16_t*>(xr_zero_chunk);
 
-    // the pieces this lane fetches for every stage: row of the stage and column chunk
+    // The pieces this lane fetches for every stage: where each begins (or a block of zeros, for
+    // a row that does not exist) and how far on the same piece of the next slice lies.  Every
+    // slice is copied once and in order, so the pointers simply move on; only a slice that is
+    // not whole (the last, if K is no multiple of 64, and the empty ones after it that keep the
+    // count of copies in flight the same) looks at columns, lane by lane.
     const bf16_t* src[LOADS];
-    int src_c[LOADS];
-    int src_kmul[LOADS];                                          // elements to go on for one column
+    int src_step[LOADS];                                          // elements from slice to slice; 0: the row does not exist
     const size_t kblocks = (size_t)((g.K + 31) / 32);
 #pragma unroll
     for (int i = 0; i < LOADS; ++i) {
         const int row = (i * WAVES + wave) * RPL + lane / CH;     // row of the stage
-        const int slot = lane % CH;
-        const int c = slot ^ swz<CH>(row);                        // the chunk that belongs in this LDS place
-        src_c[i] = c * 8;
+        const int c = (lane % CH) ^ swz<CH>(row);                 // the chunk that belongs in this LDS place
+        const bf16_t* p = nullptr;
+        int step = BK;
         if (row < BM) {
             const int m = m0 + row;
-            src[i] = m < g.M ? g.a + (size_t)m * g.lda + c * 8 : nullptr;
-            src_kmul[i] = 1;
+            if (m < g.M) p = g.a + (size_t)m * g.lda + c * 8;
         } else {
             int oc;
             const int n = w_row_of<BN, WN>(row - BM, bx, g.N, g.epi, oc);
@@ -312,24 +314,36 @@ __global__ __launch_bounds__(64 * WARPS_M * WARPS_N) void k_gemm_tile_async(Gemm
                 // row n % 16 of group n / 16; the slice's 64 columns are 2 blocks, chunk c the
                 // (c % 4)-th of its row in block c / 4; a slice further on is 2 blocks = 1024 elements on,
                 // so one copy instruction of a wave (8 rows) reads two runs of 512 bytes
-                src[i] = ok ? g.w + (size_t)(n >> 4) * kblocks * 512 + (c >> 2) * 512 + (n & 15) * 32 + (c & 3) * 8 : nullptr;
-                src_kmul[i] = 16;
-            } else {
-                src[i] = ok ? g.w + (size_t)n * g.K + c * 8 : nullptr;
-                src_kmul[i] = 1;
+                if (ok) p = g.w + (size_t)(n >> 4) * kblocks * 512 + (c >> 2) * 512 + (n & 15) * 32 + (c & 3) * 8;
+                step = BK * 16;
+            } else if (ok) {
+                p = g.w + (size_t)n * g.K + c * 8;
             }
         }
+        src_step[i] = p ? step : 0;
+        src[i] = p ? p + (size_t)k_begin * (step / BK) : zero_src;
     }
     const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) void*)lds;
+    const uint32_t lds_wave = __builtin_amdgcn_readfirstlane(lds_base + (uint32_t)(wave * 64 * 16));
+    const int nk_whole = (k_end - k_begin) / BK;                  // slices that lie within the range entirely
 // the copies PART, PART + PARTS, .. of slice KT: spread over the k-steps of the slice before, so
 // that no wave has to push a whole slice into the memory pipeline at once
 #define ASYNC_ISSUE_PART(KT, PART, PARTS)                                                            \
     {                                                                                                \
-        const int k0_ = k_begin + (KT) * BK;                                                         \
-        const uint32_t dst_ = lds_base + (uint32_t)((((KT) % STAGES) * BUF + wave * 64) * 16);       \
-        _Pragma("unroll") for (int i = (PART); i < LOADS; i += (PARTS)) {                            \
-            const bf16_t* p_ = (src[i] && k0_ + src_c[i] < k_end) ? src[i] + (size_t)k0_ * src_kmul[i] : zero_src; \
-            lds_dma16(p_, __builtin_amdgcn_readfirstlane(dst_ + i * WAVES * 64 * 16));               \
+        const uint32_t dst_ = lds_wave + (uint32_t)(((KT) % STAGES) * BUF * 16);                     \
+        if ((KT) < nk_whole) {                                                                       \
+            _Pragma("unroll") for (int i = (PART); i < LOADS; i += (PARTS)) {                        \
+                lds_dma16(src[i], dst_ + i * WAVES * 64 * 16);                                       \
+                src[i] += src_step[i];                                                               \
+            }                                                                                        \
+        } else {                                                                                     \
+            const int k0_ = k_begin + (KT) * BK;                                                     \
+            _Pragma("unroll") for (int i = (PART); i < LOADS; i += (PARTS)) {                        \
+                const int c_ = ((lane % CH) ^ swz<CH>((i * WAVES + wave) * RPL + lane / CH)) * 8;    \
+                const bf16_t* p_ = (src_step[i] && k0_ + c_ < k_end) ? src[i] : zero_src;            \
+                lds_dma16(p_, dst_ + i * WAVES * 64 * 16);                                           \
+                src[i] += src_step[i];                                                               \
+            }                                                                                        \
         }                                                                                            \
     }
 #define ASYNC_ISSUE(KT) ASYNC_ISSUE_PART(KT, 0, 1)
