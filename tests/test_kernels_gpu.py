@@ -462,13 +462,14 @@ def test_rope_kv_write(ops, dt, H, Hk, D, rot, inter, ps, starts, q_lens):
 @pytest.mark.parametrize("H,Hk,D,rot,inter", [(4, 2, 16, 16, False), (3, 1, 48, 32, False), (6, 3, 80, 80, True),
                                                (8, 8, 128, 64, True), (5, 1, 128, 128, False), (2, 2, 32, 0, False)])
 @pytest.mark.parametrize("ps,starts,q_lens", [(16, [0, 13, 40], [9, 3, 1]), (64, [70], [1]), (8, [2, 9, 100, 7], [5, 6, 1, 4]),
-                                              (16, [3, 0], [30, 8]), (16, [5, 0, 77], [60, 20, 3])])
+                                              (16, [3, 0], [30, 8]), (16, [5, 0, 77], [60, 20, 3]),
+                                              (16, [3, 0, 8, 21], [290, 200, 70, 1]), (64, [64], [520])])
 @pytest.mark.parametrize("bias", [False, True])
 def test_projection_with_rotation_and_cache_write(ops, dt, H, Hk, D, rot, inter, ps, starts, q_lens, bias):
     """q, k and v from one product, rotated and cached.  Up to 16 bfloat16 rows the product's own
     kernel does all of it (with the weight's rows in paired order where a pair is (j, j + rot/2)),
-    up to 64 the kernel that adds the product's K ranges up;
-    more rows, or 32-bit, run the product and the rotation kernel.  Both against float64 from
+    up to 64 the kernel that adds the product's K ranges up, from 512 the tile kernel;
+    other numbers of rows, or 32-bit, run the product and the rotation kernel.  Both against float64 from
     the weights in their natural order; and the two bfloat16 ways against each other."""
     from xyntetik_runner_amd.csrc.ops import paired_order
     torch.manual_seed(H * 100 + D + ps)

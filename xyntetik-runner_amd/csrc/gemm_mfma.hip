@@ -52,6 +52,7 @@ struct RopeFuse {
     bf16_t* q_out;             // [M, H*D]
     bf16_t* k_cache;
     bf16_t* v_cache;
+    const float2* cs;          // [M][rot/2] (cosine, sine) of each row's angles, times mscale: set where the tile kernel rotates
 };
 
 struct GemmArgs {
@@ -215,6 +216,109 @@ __device__ inline void write_tiles(float* stage, const f32x16 (&t)[NT], void* ds
             float4 y = x;
             if (mode == 1) { const float4 old = *q; y.x += old.x; y.y += old.y; y.z += old.z; y.w += old.w; }
             *q = y;
+        }
+    }
+}
+
+// The cosines and sines a product of many rows needs to rotate its own result, once for all
+// its tiles: the same formulas as rope_store (/root/reference/src/model.c:3514-3532).
+__global__ __launch_bounds__(256) void k_rope_table(float2* cs, const int* positions, const float* inv_freq,
+                                                    int M, int half, float mscale) {
+    const int q = blockIdx.x * 256 + threadIdx.x;
+    if (q >= M * half) return;
+    const int m = q / half, j = q - m * half;
+    const float ang = (float)positions[m] * inv_freq[j];
+    cs[q] = make_float2(cosf(ang) * mscale, sinf(ang) * mscale);
+}
+
+// The tile kernel's way of doing what rope_store does: NT side-by-side 32x32 accumulator tiles
+// of the [query heads | key heads | value heads] product go through the wave's LDS area, and a
+// lane then has 4 consecutive columns of a row and, 8 columns away (paired order) or beside
+// them (interleaved pairs), their partners.  Queries and keys leave rotated, 4 channels a
+// store; values, cached transposed, leave 8 positions of a channel at a time where the rows
+// bring an aligned group of 8 positions of one request, else one by one.
+template <int NT>
+__device__ inline void rope_tiles(float* stage, const f32x16 (&t)[NT], const RopeFuse& rp,
+                                  int m_base, int M, int col_base, int N, int lane) {
+    constexpr int SW = 32 * NT, LD = SW + 4, CPR = SW / 4, RPI = 64 / CPR;
+    const int lr = lane & 31, lg = lane >> 5;
+#pragma unroll
+    for (int n = 0; n < NT; ++n)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) stage[((e / 4) * 8 + lg * 4 + (e % 4)) * LD + n * 32 + lr] = t[n][e];
+    const int Q = rp.H * rp.D, KV = rp.Hk * rp.D, half = rp.rot >> 1;
+    // values: the tiles hold columns of one section only where sections begin at multiples of 32 * NT;
+    // so every (8 rows, column) or (row, 4 columns) item asks for its own section
+    const int ch = lane % CPR, col = col_base + ch * 4;
+    if (col < Q + KV && col < N) {
+        const int sec = col < Q ? 0 : 1;
+        const int rel = col - (sec ? Q : 0);
+        const int hs = rel / rp.D, c = rel - hs * rp.D;
+#pragma unroll
+        for (int it = 0; it < 32 / RPI; ++it) {
+            const int row = it * RPI + lane / CPR, m = m_base + row;
+            if (m >= M) continue;
+            const float4 x = *reinterpret_cast<const float4*>(stage + row * LD + ch * 4);
+            float o[4] = {x.x, x.y, x.z, x.w};
+            int d0 = c;
+            if (c < rp.rot) {
+                const float2* cs = rp.cs + (size_t)m * half;
+                if (rp.interleaved) {
+#pragma unroll
+                    for (int e = 0; e < 4; e += 2)
+                        if (c + e < rp.rot) {
+                            const float2 f = cs[(c + e) >> 1];
+                            const float x0 = o[e], x1 = o[e + 1];
+                            o[e] = x0 * f.x - x1 * f.y;
+                            o[e + 1] = x0 * f.y + x1 * f.x;
+                        }
+                } else {
+                    const int hi = (c >> 3) & 1, j0 = (c >> 4) * 8 + (c & 7);
+                    const float4 y = *reinterpret_cast<const float4*>(stage + row * LD + (ch ^ 2) * 4);
+                    const float pv[4] = {y.x, y.y, y.z, y.w};
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        const float2 f = cs[j0 + e];
+                        const float x0 = hi ? pv[e] : o[e], x1 = hi ? o[e] : pv[e];
+                        o[e] = hi ? x0 * f.y + x1 * f.x : x0 * f.x - x1 * f.y;
+                    }
+                    d0 = j0 + hi * half;
+                }
+            }
+            const uint2 w = make_uint2(pack_bf16x2(o[0], o[1]), pack_bf16x2(o[2], o[3]));
+            if (sec == 0) {
+                *reinterpret_cast<uint2*>(rp.q_out + ((size_t)m * rp.H + hs) * rp.D + d0) = w;
+            } else {
+                const int pos = rp.positions[m];
+                const PageRef pr = page_of(rp.block_table, rp.table_stride, rp.req_of_token[m], pos, rp.page_shift, rp.page_mask);
+                *reinterpret_cast<uint2*>(rp.k_cache + (((size_t)pr.page * rp.Hk + hs) * rp.page_size + pr.off) * rp.D + d0) = w;
+            }
+        }
+    }
+    if (col_base + SW > Q + KV && KV > 0) {
+        // value columns: items are (group of 8 rows, column)
+        for (int q = lane; q < 4 * SW; q += 64) {
+            const int grp = q / SW, cc = q - grp * SW, vcol = col_base + cc;
+            const int m8 = m_base + grp * 8;
+            if (vcol < Q + KV || vcol >= N || m8 >= M) continue;
+            const int rel = vcol - Q - KV, hs = rel / rp.D, d = rel - hs * rp.D;
+            const int pos = rp.positions[m8], req = rp.req_of_token[m8];
+            const bool whole = rp.page_size >= 8 && (pos & 7) == 0 && m8 + 7 < M && rp.req_of_token[m8 + 7] == req &&
+                               rp.positions[m8 + 7] == pos + 7;
+            if (whole) {
+                const PageRef pr = page_of(rp.block_table, rp.table_stride, req, pos, rp.page_shift, rp.page_mask);
+                float v[8];
+#pragma unroll
+                for (int r = 0; r < 8; ++r) v[r] = stage[(grp * 8 + r) * LD + cc];
+                *reinterpret_cast<uint4*>(rp.v_cache + (((size_t)pr.page * rp.Hk + hs) * rp.D + d) * rp.page_size + pr.off) =
+                    make_uint4(pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3]), pack_bf16x2(v[4], v[5]), pack_bf16x2(v[6], v[7]));
+            } else {
+                for (int r = 0; r < 8 && m8 + r < M; ++r) {
+                    const int p = rp.positions[m8 + r];
+                    const PageRef pr = page_of(rp.block_table, rp.table_stride, rp.req_of_token[m8 + r], p, rp.page_shift, rp.page_mask);
+                    rp.v_cache[(((size_t)pr.page * rp.Hk + hs) * rp.D + d) * rp.page_size + pr.off] = f32_to_bf16(stage[(grp * 8 + r) * LD + cc]);
+                }
+            }
         }
     }
 }
@@ -448,7 +552,7 @@ __global__ __launch_bounds__(64 * WARPS_M * WARPS_N) void k_gemm_tile_async(Gemm
     static_assert((size_t)STAGES * ROWS * CH * 16 >= (size_t)WAVES * STAGE_FLOATS * 4, "no room for the waves' output areas");
     float* stage = reinterpret_cast<float*>(lds) + wave * STAGE_FLOATS;
     constexpr int NTP = TN % 2 == 0 ? 2 : 1;             // tiles written together
-    if (g.vec_out) __builtin_amdgcn_s_barrier();
+    if (g.vec_out || g.rope.cs) __builtin_amdgcn_s_barrier();
 
     if (g.splits > 1 || g.raw) {
         // raw sums of this K range, by weight row: the epilogue belongs to k_gemm_finish
@@ -521,7 +625,7 @@ __global__ __launch_bounds__(64 * WARPS_M * WARPS_N) void k_gemm_tile_async(Gemm
             }
         return;
     }
-    if (g.vec_out) {
+    if (g.vec_out || g.rope.cs) {
 #pragma unroll
         for (int i = 0; i < TM; ++i)
 #pragma unroll
@@ -533,6 +637,10 @@ __global__ __launch_bounds__(64 * WARPS_M * WARPS_N) void k_gemm_tile_async(Gemm
                     const float b = g.bias && col < g.N ? g.bias[col] : 0.f;
 #pragma unroll
                     for (int e = 0; e < 16; ++e) t[n][e] = acc[i][j + n][e] + b;
+                }
+                if (g.rope.cs) {
+                    rope_tiles<NTP>(stage, t, g.rope, m0 + wm0 + i * 32, g.M, bx * BN + wn0 + j * 32, g.N, lane);
+                    continue;
                 }
                 write_tiles<NTP>(stage, t, g.out, g.ldo, g.epi == EPI_ACCUM ? 1 : (g.out_bf16 ? 2 : 0),
                                  m0 + wm0 + i * 32, g.M, bx * BN + wn0 + j * 32, g.N, lane);
@@ -993,11 +1101,19 @@ extern "C" int xr_gemm_bf16(void* out, const void* a, const void* w, const float
             }
         }
     }
-    g.rope.q_out = nullptr;
+    g.rope.q_out = nullptr; g.rope.cs = nullptr;
+    // more than 64 rows: the tile kernel rotates and caches its own result, with the rows' cosines and
+    // sines from a table that a small kernel writes into the workspace first; K is then not split
+    const bool rope_direct = rope && M > 64;
     if (rope) {
-        XR_REQUIRE(M <= 64 && variant == 0 && epi == EPI_STORE && !(norm && norm->xg),
-                   "gemm: rotation and cache write are folded only into a plain product of at most 64 rows");
-        if (M > 16) {
+        XR_REQUIRE(variant == 0 && epi == EPI_STORE && !(norm && norm->xg),
+                   "gemm: rotation and cache write are folded only into a plain product whose kernel the library chooses");
+        if (rope_direct) {
+            XR_REQUIRE(workspace && (size_t)M * (rope->rot / 2 + 1) * sizeof(float2) <= workspace_bytes,
+                       "gemm: rotation after a product of %d rows needs a workspace for its table", M);
+            XR_REQUIRE(((uintptr_t)rope->q_out % 8) == 0 && ((uintptr_t)rope->k_cache % 8) == 0 && ((uintptr_t)rope->v_cache % 16) == 0,
+                       "gemm: queries and caches must be 16-byte aligned");
+        } else if (M > 16) {
             XR_REQUIRE(workspace && (size_t)M * N * 4 <= workspace_bytes, "gemm: rotation after a product of %d rows needs a workspace", M);
             g.raw = 1;
         }
@@ -1017,6 +1133,15 @@ extern "C" int xr_gemm_bf16(void* out, const void* a, const void* w, const float
         g.rope.mscale = rope->mscale; g.rope.page_shift = shift < 0 ? 0 : shift; g.rope.page_mask = rope->page_size - 1;
         g.rope.page_size = rope->page_size;
         g.rope.q_out = (bf16_t*)rope->q_out; g.rope.k_cache = (bf16_t*)rope->k_cache; g.rope.v_cache = (bf16_t*)rope->v_cache;
+        if (rope_direct) {
+            g.rope.cs = (const float2*)workspace;
+            const int half = rope->rot / 2;
+            if (half > 0) {
+                k_rope_table<<<(unsigned)(((size_t)M * half + 255) / 256), 256, 0, stream>>>((float2*)workspace, rope->positions, rope->inv_freq,
+                                                                                            M, half, rope->mscale);
+                XR_CHECK_LAUNCH("rope_table");
+            }
+        }
     }
     if (variant >= 1000) { g.m_fast = 1; variant -= 1000; }
     const bool sw = epi == EPI_SWIGLU;
@@ -1025,6 +1150,7 @@ extern "C" int xr_gemm_bf16(void* out, const void* a, const void* w, const float
     // (measured at 32 and 64 rows: 10 ranges of 32 tiles, two rounds, took 20 us where 8 take 16),
     // if the workspace has room for their sums
     auto pick_splits = [&](int tiles) {
+        if (rope_direct) return 1;
         int s = tiles >= 256 ? 1 : 256 / tiles;
         int max_s = K / 256 > 0 ? K / 256 : 1;
         s = s < 1 ? 1 : (s > max_s ? max_s : s);
@@ -1071,7 +1197,7 @@ extern "C" int xr_gemm_bf16(void* out, const void* a, const void* w, const float
             // if one was asked for).  Times here are in products of a tile at full rate; the adding
             // kernel moves (ranges + 2) x M x N x 4 bytes at about 4.5 TB/s, a tile does about
             // 4 TFLOP/s.  Measured (2048 x 4096 x 14336): 264 us against 281 us with 256x128 tiles.
-            if (!sw && workspace && count(cands[0], N) <= 128 && count(cands[0], N) >= 64) {
+            if (!sw && workspace && !rope_direct && count(cands[0], N) <= 128 && count(cands[0], N) >= 64) {
                 const int s2 = pick_splits(count(cands[0], N));
                 if (s2 >= 2) {
                     const double unit = 0.5e-12;       // seconds per product-column of a 256x256 tile's row

@@ -240,6 +240,7 @@ class Ops:
     # -- matrix product ---------------------------------------------------------
     GEMM_WORKSPACE_BYTES = 96 << 20
     FINISH_ROWS = 64        # up to here a product's epilogue may be the kernel that adds its K ranges up
+    ROPE_TILE_ROWS = 512    # from here the q/k/v product has tiles enough with K whole, and its tile kernel rotates and caches
 
     def _gemm_workspace(self, device):
         """Room for the sums of K ranges when a product with few rows is split (one buffer per process;
@@ -433,8 +434,9 @@ class Ops:
         ``w`` holds ``H`` query heads, then ``Hk`` key heads and ``Hk`` value heads (``Hk`` = 0 and
         no caches: queries alone); with ``paired`` its query and key rows are in ``paired_order``.
         Up to 16 bfloat16 rows (``h`` may be an ``UnscaledRows``) the product's kernel rotates and
-        stores its own result, up to 64 the kernel that adds the product's K ranges up does,
-        which saves a kernel and the 32-bit copy of the projections; otherwise the product and
+        stores its own result, up to 64 the kernel that adds the product's K ranges up does, from
+        512 the tile kernel (with the rows' cosines and sines from a table made first), which
+        saves a kernel and the 32-bit copy of the projections; otherwise the product and
         ``rope_kv_write`` run one after the other."""
         rows = h.data if isinstance(h, UnscaledRows) else h
         wt = w.data if isinstance(w, PackedWeight) else w
@@ -442,8 +444,8 @@ class Ops:
         if w.shape[0] != Q + 2 * KV:
             raise KernelError(f"projection has {w.shape[0]} rows, {H} query and 2 x {Hk} key/value heads of {D} need {Q + 2 * KV}")
         q = torch.empty((T, Q), dtype=rows.dtype, device=rows.device)
-        if (self.fuse_rope and T <= self.FINISH_ROWS and self._mfma_ok(rows, wt) and D % 16 == 0
-                and T * w.shape[0] * 4 <= self.GEMM_WORKSPACE_BYTES
+        if (self.fuse_rope and (T <= self.FINISH_ROWS or T >= self.ROPE_TILE_ROWS) and self._mfma_ok(rows, wt) and D % 16 == 0
+                and (T * w.shape[0] * 4 if T <= self.FINISH_ROWS else T * (rot // 2 + 1) * 8) <= self.GEMM_WORKSPACE_BYTES
                 and (Hk == 0 or (k_cache.dtype == torch.bfloat16 and v_cache.dtype == torch.bfloat16))
                 and (rot == 0 or interleaved or (paired and rot % 16 == 0))):
             self._dev(rows, wt, bias, k_cache, v_cache, positions, req_of_token, block_table, inv_freq)
