@@ -24,7 +24,7 @@ WORKLOAD = {
     "A": ([5, 17, 33, 64, 150], 16),
     "B": ([1, 9, 40, 64, 100], 24),
     "C": ([3, 31, 70], 40),
-    "D": ([200, 70, 330], 34),
+    "D": ([200, 70, 640], 34),       # (from 512 rows the q/k/v product rotates and caches its own result)
 }
 
 
@@ -86,6 +86,28 @@ def test_schedules_match_plain(models, tmp_path, which, dtype, schedule):
     out, runner = run_replay(d, dtype, steps, tmp_path, page_size)
     got = traces.collect(steps, out, cfg["vocab_size"])
     check(got, want, dtype, f"{which}/{schedule}")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_long_portions_of_several_requests_in_one_step(models, tmp_path, dtype):
+    """A step of more than 512 rows made of three requests: one that goes on at a position that
+    is no multiple of 8, one whole prompt, one decoded token between them.  The kernels that take
+    many rows at once (tile products, the product that rotates and caches its own result, 128-row
+    attention blocks) see request edges and groups of 8 positions that are not whole."""
+    d, cfg, reqs, plens, want = models["D"]
+    a, b, c = reqs["r2"], reqs["r0"], reqs["r1"]
+    steps = [
+        {"step": 0, "entries": [{"id": "r2", "tokens": a[:3], "want": [0, 1, 2]},
+                                {"id": "r1", "tokens": c[:50], "want": list(range(50))}], "end": []},
+        {"step": 1, "entries": [{"id": "r2", "tokens": a[3:333], "want": list(range(330))},
+                                {"id": "r1", "tokens": c[50:51], "want": [0]},
+                                {"id": "r0", "tokens": b, "want": list(range(len(b)))}], "end": ["r0"]},
+        {"step": 2, "entries": [{"id": "r1", "tokens": c[51:], "want": list(range(len(c) - 51))},
+                                {"id": "r2", "tokens": a[333:], "want": list(range(len(a) - 333))}], "end": ["r1", "r2"]},
+    ]
+    assert sum(len(e["tokens"]) for e in steps[1]["entries"]) >= 512
+    out, runner = run_replay(d, dtype, steps, tmp_path, 64)
+    check(traces.collect(steps, out, cfg["vocab_size"]), want, dtype, "D/long portions")
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
