@@ -104,6 +104,28 @@ def test_linear_bf16_mfma(ops, M, N, K):
                        a.double() @ w.double().T + b.double()) < 1e-5
 
 
+@pytest.mark.parametrize("M", [8, 40, 300])
+@pytest.mark.parametrize("first,width", [(0, 128), (4, 136), (3, 131), (2, 130)])
+def test_linear_into_columns_of_a_wider_matrix(ops, M, first, width):
+    """The output is a run of columns of a wider matrix: rows that begin 16 bytes aligned or not,
+    row strides that are multiples of 4 or not (the tile kernel writes 4 columns a lane only
+    where it may); what lies beside the run stays as it was."""
+    N, K = 96, 80
+    a = (torch.randn(M, K, device=DEV) * 0.5).bfloat16()
+    w = (torch.randn(N, K, device=DEV) * 0.1).bfloat16()
+    want = a.double() @ w.double().T
+    for dt, tol in ((torch.float32, 1e-5), (torch.bfloat16, 6e-3)):
+        big = torch.full((M, width), 7.0, device=DEV, dtype=dt)
+        ops.linear(a, w, out=big[:, first:first + N])
+        assert rel(big[:, first:first + N], want) < tol
+        assert (big[:, :first] == 7).all() and (big[:, first + N:] == 7).all()
+    big = torch.randn(M, width, device=DEV)
+    keep = big.clone()
+    ops.linear(a, w, out=big[:, first:first + N], accumulate=True)
+    assert rel(big[:, first:first + N], keep[:, first:first + N].double() + want) < 1e-5
+    assert torch.equal(big[:, :first], keep[:, :first]) and torch.equal(big[:, first + N:], keep[:, first + N:])
+
+
 @pytest.mark.parametrize("M", [1, 8, 16, 17, 64, 65, 300])
 @pytest.mark.parametrize("N,K", [(48, 64), (100, 72), (333, 264), (1000, 1032), (16, 8)])
 def test_linear_packed_weights_give_the_same(ops, M, N, K):
