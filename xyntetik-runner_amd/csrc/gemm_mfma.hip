@@ -1235,7 +1235,7 @@ extern "C" int xr_gemm_bf16(void* out, const void* a, const void* w, const float
             int blocks;
             if (sw) blocks = launch_skinny<1, 1, 8, 8, true, true>(g, stream);
             else if (N >= 65536) blocks = M <= 8 ? launch_skinny<1, 1, 8, 8, false, true>(g, stream) : launch_skinny<1, 2, 4, 8, false, true>(g, stream);
-            else if (N > 4096 && K <= 8192) blocks = M <= 1 ? launch_skinny<1, 1, 4, 8, false, true>(g, stream) : launch_skinny<1, 1, 4, 4, false, true>(g, stream);
+            else if (N > 4096 && K <= 8192) blocks = K > 4096 ? launch_skinny<1, 1, 4, 8, false, true>(g, stream) : launch_skinny<1, 1, 4, 4, false, true>(g, stream);
             else blocks = launch_skinny<1, 1, 8, 4, false, true>(g, stream);
             if (blocks < 0) return blocks;
             if (norm) norm->ss_out_rows = (N + 15) / 16;
