@@ -240,6 +240,13 @@ __global__ __launch_bounds__(256, 2) void k_attn_cta(AttnArgs a) {
     const bf16_t* __restrict__ vc = a.vc;
     const bf16_t* zero_src = reinterpret_cast<const bf16_t*>(xr_zero_chunk);
     const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) void*)lds;
+    // Where every lane's piece exists in every whole tile and a copy instruction brings pieces of
+    // keys only or of values only (head sizes 64, 128 and 256), a whole tile of an existing page
+    // is copied from two bases that all lanes share, each lane adding a fixed 32-bit offset.
+    constexpr bool CTA_FAST = CK_POW2 && NKC % 256 == 0 && NVC % 256 == 0 && HD % 32 == 0;
+    uint32_t fast_off[CTA_LOADS];
+#pragma unroll
+    for (int i = 0; i < CTA_LOADS; ++i) fast_off[i] = (uint32_t)src_off[i] * 2u;
 
     // page numbers of the item's keys, one per lane, 64 pages at a time
     int pages_base = kbeg >> a.page_shift;
@@ -270,11 +277,16 @@ __global__ __launch_bounds__(256, 2) void k_attn_cta(AttnArgs a) {
         const size_t pb_ = (size_t)(pg_ < 0 ? 0 : pg_) * a.Hk + kvh;                                     \
         const bf16_t* kb_ = kc + (pb_ * a.page_size + (kt_ & a.page_mask)) * HD;                         \
         const bf16_t* vb_ = vc + pb_ * HD * a.page_size + (kt_ & a.page_mask);                           \
-        const uint32_t dst_ = lds_base + (uint32_t)(((ti_ % CTA_STAGES) * STAGE_CHUNKS + wave * 64) * 16); \
-        _Pragma("unroll") for (int i = 0; i < CTA_LOADS; ++i) {                                          \
-            const bool ok_ = pg_ >= 0 && kt_ + src_key[i] < seq_len;                                     \
-            const bf16_t* p_ = ok_ ? (src_is_k[i] ? kb_ : vb_) + src_off[i] : zero_src;                  \
-            lds_dma16(p_, __builtin_amdgcn_readfirstlane(dst_ + i * 256 * 16));                          \
+        const uint32_t dst_ = __builtin_amdgcn_readfirstlane(lds_base + (uint32_t)(((ti_ % CTA_STAGES) * STAGE_CHUNKS + wave * 64) * 16)); \
+        if (CTA_FAST && pg_ >= 0 && kt_ + 32 <= seq_len) {                                               \
+            _Pragma("unroll") for (int i = 0; i < CTA_LOADS; ++i)                                        \
+                lds_dma16_base(i * 256 < NKC ? kb_ : vb_, fast_off[i], dst_ + i * 256 * 16);             \
+        } else {                                                                                         \
+            _Pragma("unroll") for (int i = 0; i < CTA_LOADS; ++i) {                                      \
+                const bool ok_ = pg_ >= 0 && kt_ + src_key[i] < seq_len;                                 \
+                const bf16_t* p_ = ok_ ? (src_is_k[i] ? kb_ : vb_) + src_off[i] : zero_src;              \
+                lds_dma16(p_, dst_ + i * 256 * 16);                                                      \
+            }                                                                                            \
         }                                                                                                \
     }
 
@@ -377,7 +389,7 @@ static_assert(STREAM_LDS_BYTES <= 160 * 1024, "the rings do not fit into LDS");
 
 __global__ __launch_bounds__(64 * STREAM_WAVES) void k_attn_stream(AttnArgs a) {
     extern __shared__ uint4 lds[];
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int kvh = blockIdx.y;
     const int* it = a.items + (size_t)blockIdx.x * ITEM_INTS;
     const int req = it[0], row0 = it[1], kbeg = it[2], kend = it[3], slot = it[4];
@@ -425,8 +437,8 @@ __global__ __launch_bounds__(64 * STREAM_WAVES) void k_attn_stream(AttnArgs a) {
     const bf16_t* __restrict__ kc = a.kc;
     const bf16_t* __restrict__ vc = a.vc;
     const bf16_t* zero_src = reinterpret_cast<const bf16_t*>(xr_zero_chunk);
-    const uint32_t ring_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) void*)lds +
-                               (uint32_t)(wave * STREAM_STAGES * W_STAGE * 16);
+    const uint32_t ring_base = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(__attribute__((address_space(3))) void*)lds +
+                                                              (uint32_t)(wave * STREAM_STAGES * W_STAGE * 16));
     const uint4* ring = lds + wave * STREAM_STAGES * W_STAGE;
 
     int pages_base = kbeg >> a.page_shift;
@@ -453,7 +465,7 @@ __global__ __launch_bounds__(64 * STREAM_WAVES) void k_attn_stream(AttnArgs a) {
             my_page = bt[in ? pi : 0];                                                                   \
             my_page = in ? my_page : -1;                                                                 \
         }                                                                                                \
-        const uint32_t dst_ = ring_base + (uint32_t)((j_ % STREAM_STAGES) * W_STAGE * 16);               \
+        const uint32_t dst_ = __builtin_amdgcn_readfirstlane(ring_base + (uint32_t)((j_ % STREAM_STAGES) * W_STAGE * 16)); \
         if (a.page_size >= 32) {                                                                         \
             int pg_ = -1;                                                                                \
             if (live_) pg_ = __builtin_amdgcn_readlane(my_page, __builtin_amdgcn_readfirstlane((kt_ >> a.page_shift) - pages_base)); \
@@ -464,7 +476,7 @@ __global__ __launch_bounds__(64 * STREAM_WAVES) void k_attn_stream(AttnArgs a) {
             _Pragma("unroll") for (int i = 0; i < W_LOADS; ++i) {                                        \
                 const bool ok_ = pg_ >= 0 && kt_ + src_key[i] < seq_len;                                 \
                 const bf16_t* p_ = ok_ ? (src_is_k[i] ? kb_ + src_key[i] * HD : vb_ + src_key[i]) + src_off[i] : zero_src; \
-                lds_dma16(p_, __builtin_amdgcn_readfirstlane(dst_ + i * 64 * 16));                       \
+                lds_dma16(p_, dst_ + i * 64 * 16);                                                       \
             }                                                                                            \
         } else {                                                                                         \
             _Pragma("unroll") for (int i = 0; i < W_LOADS; ++i) {                                        \
@@ -476,7 +488,7 @@ __global__ __launch_bounds__(64 * STREAM_WAVES) void k_attn_stream(AttnArgs a) {
                 const int ko_ = key_ & a.page_mask;                                                      \
                 const bf16_t* p_ = src_is_k[i] ? kc + (pb_ * a.page_size + ko_) * HD + src_off[i]        \
                                                : vc + pb_ * HD * a.page_size + src_off[i] + ko_;         \
-                lds_dma16(ok_ ? p_ : zero_src, __builtin_amdgcn_readfirstlane(dst_ + i * 64 * 16));      \
+                lds_dma16(ok_ ? p_ : zero_src, dst_ + i * 64 * 16);                                      \
             }                                                                                            \
         }                                                                                                \
     }
