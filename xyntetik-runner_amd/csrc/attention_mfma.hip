@@ -73,15 +73,21 @@ __device__ inline uint4 keep_if(bool ok, uint4 v) {     // zero unless ok, word 
 }
 __device__ inline uint32_t pack2(float lo, float hi) { return pack_bf16x2(lo, hi); }
 
-// One tile's softmax step for the lane's row: p[] from s[], the running maximum m and sum l,
-// and the rescaling of the output accumulators when the maximum moved.
+// One tile's softmax step for the lane's row: p[] from s[], the running reference m and sum l,
+// and the rescaling of the output accumulators when the reference moved.  The reference is a
+// maximum seen so far, and follows the true maximum only when that has risen by more than
+// MAX_SLACK (in units of log2): any reference gives the same quotient sum(p v) / sum(p), terms up
+// to 2^8 are no strain on 32-bit sums or on bfloat16 P, and the 64 multiplications a lane owes
+// its output when any row of the wave moves its reference become rare (before, nearly every tile
+// of a few thousand keys paid them).
+#define MAX_SLACK 8.0f
 #define ATTN_SOFTMAX_STEP(KT, KEND)                                                                  \
         if ((KT) + 32 <= (KEND) && (KT) + 31 <= pos_min && (KT) >= lo_max) {                             \
             float mt = fmaxf(fmaxf(s[0], s[1]), fmaxf(s[2], s[3]));                                      \
 _Pragma("unroll")                                                                                        \
             for (int e = 4; e < 16; e += 4) mt = fmaxf(mt, fmaxf(fmaxf(s[e], s[e + 1]), fmaxf(s[e + 2], s[e + 3]))); \
             mt = fmaxf(mt, __shfl_xor(mt, 32, 64));                                                      \
-            const float mn = fmaxf(m, mt * c2);                                                          \
+            const float mn = mt * c2 > m + MAX_SLACK ? mt * c2 : m;                                      \
             corr = __builtin_amdgcn_exp2f(m - mn);                                                       \
             float rs = 0.f;                                                                              \
 _Pragma("unroll")                                                                                        \
@@ -102,7 +108,7 @@ _Pragma("unroll")                                                               
                 mt = fmaxf(mt, p[e]);                                                                    \
             }                                                                                            \
             mt = fmaxf(mt, __shfl_xor(mt, 32, 64));                                                      \
-            const float mn = fmaxf(m, mt);                                                               \
+            const float mn = mt > m + MAX_SLACK ? mt : m;                                                \
             const float mu = mn == -INFINITY ? 0.f : mn;                                                 \
             corr = __builtin_amdgcn_exp2f(m - mu);                                                       \
             float rs = 0.f;                                                                              \
