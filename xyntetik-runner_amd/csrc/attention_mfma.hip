@@ -648,18 +648,36 @@ __global__ __launch_bounds__(256) void k_attn_merge(MergeArgs a) {
         const float* ml = a.part_ml + (((size_t)s0 * a.Hk + kvh) * ROWS + r) * 2;
         const float* po = a.part_o + (((size_t)s0 * a.Hk + kvh) * ROWS + r) * HD + d4;
         const size_t ml_step = (size_t)stride * a.Hk * ROWS * 2, po_step = (size_t)stride * a.Hk * ROWS * HD;
+        // 16 slots at a time, all their loads on their way before the first is used (a thread that
+        // took the maxima first and then the outputs, four loads at a time, waited out eight memory
+        // latencies for the 14 slots of a lone request: 8 us, as long as the attention itself)
+        constexpr int MS = 16;
         float mx = -INFINITY;
-#pragma unroll 4
-        for (int s = 0; s < ns; ++s) mx = fmaxf(mx, ml[s * ml_step]);
         float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
         float wsum = 0.f;
-#pragma unroll 4
-        for (int s = 0; s < ns; ++s) {
-            const float2 v2 = *reinterpret_cast<const float2*>(ml + s * ml_step);
-            const float w = v2.y > 0.f ? v2.y * __builtin_amdgcn_exp2f(v2.x - mx) : 0.f;
-            const float4 v = *reinterpret_cast<const float4*>(po + s * po_step);
-            acc.x += w * v.x; acc.y += w * v.y; acc.z += w * v.z; acc.w += w * v.w;
-            wsum += w;
+        for (int sb = 0; sb < ns; sb += MS) {
+            float2 mlv[MS];
+            float4 pv[MS];
+#pragma unroll
+            for (int u = 0; u < MS; ++u) {
+                const int sc = sb + u < ns ? sb + u : sb;
+                mlv[u] = *reinterpret_cast<const float2*>(ml + sc * ml_step);
+                pv[u] = *reinterpret_cast<const float4*>(po + sc * po_step);
+            }
+            float cm = mx;
+#pragma unroll
+            for (int u = 0; u < MS; ++u)
+                if (sb + u < ns) cm = fmaxf(cm, mlv[u].x);
+            const float resc = mx == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(mx - cm);   // (1 while there is one group only)
+            acc.x *= resc; acc.y *= resc; acc.z *= resc; acc.w *= resc;
+            wsum *= resc;
+            mx = cm;
+#pragma unroll
+            for (int u = 0; u < MS; ++u) {
+                const float w = (sb + u < ns && mlv[u].y > 0.f) ? mlv[u].y * __builtin_amdgcn_exp2f(mlv[u].x - mx) : 0.f;
+                acc.x += w * pv[u].x; acc.y += w * pv[u].y; acc.z += w * pv[u].z; acc.w += w * pv[u].w;
+                wsum += w;
+            }
         }
         const float inv = wsum > 0.f ? 1.0f / wsum : 0.f;
         bf16_t* op = a.out + ((size_t)(q0 + tok) * a.H + kvh * G + hg) * HD + d4;
