@@ -751,7 +751,7 @@ def test_attention_plan_covers_every_key_once():
                 if len(parts) > 1:
                     for w in range(waves):              # every 32-row block that exists is merged from its slots
                         if row0 + 32 * w < n * G:
-                            assert (b, row0 + 32 * w, parts[0][2] + w, len(parts), waves) in jobs
+                            assert (b, row0 + 32 * w, parts[0][2] + w, len(parts), waves, sum(q_lens[:b]), q_lens[b]) in jobs
                     used += [p[2] + w for p in parts for w in range(waves)]
         # a row belongs to one kind of item only
         assert not {(b, r // 128) for b, r, *_ in cta_items} & {(b, r // 128) for b, r, *_ in items}

@@ -42,7 +42,7 @@ static_assert(HD % 16 == 0 && HD >= 16 && HD <= 256, "head size must be a multip
 
 #define ITEM_INTS 8                   // req, row0, k_begin, k_end, slot (-1: final), q0, q_len, start
 #define ROWS 32
-#define JOB_INTS 5                    // req, row0, first slot, slots, distance between slots
+#define JOB_INTS 7                    // req, row0, first slot, slots, distance between slots, q0, q_len (as in the items)
 
 struct AttnArgs {
     const bf16_t* q;        // [T, H, HD]
@@ -622,7 +622,7 @@ __global__ __launch_bounds__(64 * STREAM_WAVES) void k_attn_stream(AttnArgs a) {
     }
 }
 
-// One merge job: {req, row0, first_slot, n_slots, slot_stride}.  Slot s holds the normalised output of
+// One merge job: {req, row0, first_slot, n_slots, slot_stride, q0, q_len}.  Slot s holds the normalised output of
 // its keys with their maximum m_s (in units of log2) and sum l_s; the whole is
 // sum_s w_s O_s / sum_s w_s with w_s = l_s * 2^(m_s - max m).
 struct MergeArgs {
@@ -636,10 +636,10 @@ struct MergeArgs {
 
 __global__ __launch_bounds__(256) void k_attn_merge(MergeArgs a) {
     const int* job = a.jobs + (size_t)blockIdx.x * JOB_INTS;
-    const int req = job[0], row0 = job[1], s0 = job[2], ns = job[3], stride = job[4];
+    const int row0 = job[1], s0 = job[2], ns = job[3], stride = job[4];
     const int kvh = blockIdx.y;
     const int G = a.H / a.Hk;
-    const int q0 = a.cu_q[req], q_len = a.cu_q[req + 1] - q0;
+    const int q0 = job[5], q_len = job[6];          // (with the job: one dependent read less before the partial results)
     const int n_rows = (q_len * G - row0) < ROWS ? (q_len * G - row0) : ROWS;      // rows of this block that exist
     for (int idx = threadIdx.x; idx < n_rows * (HD / 4); idx += 256) {
         const int r = idx / (HD / 4), d4 = (idx % (HD / 4)) * 4;

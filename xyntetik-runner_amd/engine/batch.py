@@ -30,8 +30,8 @@ class AttentionPlan:
     ``n_cta_items`` are blocks of 128 rows that a workgroup takes together (its wave w the rows
     from ``row0 + 32 w``, with partial slot ``slot + w``), the other ``n_items`` blocks of 32
     rows, one wave each.
-    ``jobs [m, 5]``: request, first row of 32, first slot, number of slots to merge and the
-    distance between them.
+    ``jobs [m, 7]``: request, first row of 32, first slot, number of slots to merge, the
+    distance between them, the request's first row in the step and its number of tokens.
     """
     items: torch.Tensor
     n_items: int
@@ -128,7 +128,7 @@ def plan_attention(starts, q_lens, group_size: int, window: Optional[int], n_kv_
             rows = q_lens[b] * group_size
             for w in range(ATTN_CTA_ROWS // ATTN_ROWS):
                 if row0 + w * ATTN_ROWS < rows:
-                    jobs.append((b, row0 + w * ATTN_ROWS, first + w, n_parts, ATTN_CTA_ROWS // ATTN_ROWS))
+                    jobs.append((b, row0 + w * ATTN_ROWS, first + w, n_parts, ATTN_CTA_ROWS // ATTN_ROWS, q0s[b], q_lens[b]))
 
     budget = max(1, ATTN_STREAM_SLOTS // n_kv_heads)       # items that run at a time
     for b, row0, lo, hi, tiles in blocks:
@@ -144,7 +144,7 @@ def plan_attention(starts, q_lens, group_size: int, window: Optional[int], n_kv_
             items.append((b, row0, k, e, slot, q0s[b], q_lens[b], starts[b]))
             slot += 1
             k = e
-        jobs.append((b, row0, first, slot - first, 1))
+        jobs.append((b, row0, first, slot - first, 1, q0s[b], q_lens[b]))
     return cta_items, items, jobs, slot
 
 

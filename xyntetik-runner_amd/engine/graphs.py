@@ -72,7 +72,7 @@ class StaticDecodeContext:
 
     def _alloc(self) -> None:
         B, S = self.B, self.S
-        n_plan = len(self._plan_keys) * (B * S * 8 + B * 5)
+        n_plan = len(self._plan_keys) * (B * S * 8 + B * 7)
         offs = np.concatenate([[0], np.cumsum(self._sizes)]).astype(np.int64)
         total = int(offs[-1]) + n_plan
         self._offs = offs
@@ -93,10 +93,10 @@ class StaticDecodeContext:
         for k in self._plan_keys:
             self._plan_off[k] = base
             items = d[base:base + B * S * 8]
-            jobs = d[base + B * S * 8:base + B * S * 8 + B * 5]
+            jobs = d[base + B * S * 8:base + B * S * 8 + B * 7]
             self._plans[k] = AttentionPlan(items, B * S, jobs if S > 1 else None, B if S > 1 else 0,
                                            B * S if S > 1 else 0)
-            base += B * S * 8 + B * 5
+            base += B * S * 8 + B * 7
 
     def block_table(self, group: int) -> torch.Tensor:
         return self._tables[group]
@@ -174,7 +174,7 @@ class StaticDecodeContext:
         group_size, window, _ = key
         B, S = self.B, self.S
         items = h[base:base + B * S * 8].reshape(B, S, 8)
-        jobs = h[base + B * S * 8:base + B * S * 8 + B * 5].reshape(B, 5)
+        jobs = h[base + B * S * 8:base + B * S * 8 + B * 7].reshape(B, 7)
         hi = starts.astype(np.int64) + 1                          # keys [lo, hi)
         lo = np.zeros(B, dtype=np.int64)
         if window:
@@ -201,6 +201,8 @@ class StaticDecodeContext:
         jobs[:, 2] = np.arange(B) * S
         jobs[:, 3] = S
         jobs[:, 4] = 1
+        jobs[:, 5] = np.arange(B)
+        jobs[:, 6] = 1
 
 
 class DecodeGraphs:
