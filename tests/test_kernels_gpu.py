@@ -654,6 +654,8 @@ ATTN_WORKGROUP_CASES = [
     (2, 2, 16, 32, None, [5], [70], 1),
     (5, 1, 64, 128, 33, [1000, 3], [90, 40], 4),       # five heads a group: rows of a token straddle waves
     (3, 3, 48, 32, 9, [60], [200], None),              # a window shorter than a tile
+    (4, 2, 128, 32, None, [37, 0], [200, 96], None),   # a tile a page: whole tiles come from bases all lanes share
+    (4, 4, 64, 32, 50, [300, 31], [100, 70], 2),       # the same with a window and key ranges
 ]
 
 
