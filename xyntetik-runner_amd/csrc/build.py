@@ -40,7 +40,7 @@ UNITS: Dict[str, dict] = {
     },
 }
 ATTN_SOURCES = ["errors.hip", "attention_mfma.hip"]
-HEADERS = ["common.h", "async_copy.h"]
+HEADERS = ["common.h", "async_copy.h", "no_alloc.h"]
 
 
 class BuildError(RuntimeError):

@@ -15,6 +15,9 @@
 // point, added with integer atomics, so the result does not depend on the order in
 // which lanes arrive.
 #include "common.h"
+#include "no_alloc.h"
+
+#include <mutex>
 
 #define SM_THREADS 1024
 #define SM_FIX 1099511627776.0   // 2^40
@@ -266,7 +269,7 @@ __global__ __launch_bounds__(SM_THREADS) void k_sample(SampleArgs a) {
     if (threadIdx.x == 0) a.out[r] = (int)(pick & 0xFFFFFFull);
 }
 
-extern "C" int xr_sample(int* out, float* logits, int W, int V, int ld, const float* temp, const int* top_k,
+static int sample_launch(int* out, float* logits, int W, int V, int ld, const float* temp, const int* top_k,
                          const float* top_p, const float* min_p, const float* repeat_penalty,
                          const float* draw, const int* recent, const int* n_recent, int recent_cap,
                          const int* exempt, int n_exempt, float* greedy_ws, hipStream_t stream) {
@@ -287,4 +290,57 @@ extern "C" int xr_sample(int* out, float* logits, int W, int V, int ld, const fl
     k_sample<<<W, SM_THREADS, 0, stream>>>(a);
     XR_CHECK_LAUNCH("sample");
     return XR_OK;
+}
+
+extern "C" int xr_sample(int* out, float* logits, int W, int V, int ld, const float* temp, const int* top_k,
+                         const float* top_p, const float* min_p, const float* repeat_penalty,
+                         const float* draw, const int* recent, const int* n_recent, int recent_cap,
+                         const int* exempt, int n_exempt, float* greedy_ws, hipStream_t stream) {
+    return sample_launch(out, logits, W, V, ld, temp, top_k, top_p, min_p, repeat_penalty, draw, recent, n_recent,
+                         recent_cap, exempt, n_exempt, greedy_ws, stream);
+}
+
+// ------------------------------------------------------------------------------ no allocation
+// The same pick with the first pass's work area in an array of the library's own (no_alloc.h).
+// In host code the array's name is only a handle: its device address is asked for once per
+// device and kept, and the kernels get that address as they get the caller's work area above.
+#define XR_MAX_DEVICES 64
+static __device__ __align__(256) float scratch[(size_t)XR_SAMPLE_STATIC_MAX_ROWS * GREEDY_SPLITS * 2];
+static float* scratch_ptr[XR_MAX_DEVICES];       // the array's address on each device, once resolved
+static std::mutex scratch_lock;
+
+static int scratch_on_current_device(float** ptr) {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) (void)hipGetLastError();
+    XR_REQUIRE(e == hipSuccess, "sample_static: no current device: %s", hipGetErrorString(e));
+    XR_REQUIRE(dev >= 0 && dev < XR_MAX_DEVICES, "sample_static: device %d is beyond the %d this library keeps an address for", dev, XR_MAX_DEVICES);
+    std::lock_guard<std::mutex> hold(scratch_lock);
+    if (!scratch_ptr[dev]) {
+        void* p = nullptr;
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess) (void)hipGetLastError();
+        XR_REQUIRE(e == hipSuccess && p, "sample_static: the work area's address on device %d: %s", dev, hipGetErrorString(e));
+        scratch_ptr[dev] = (float*)p;
+    }
+    *ptr = scratch_ptr[dev];
+    return XR_OK;
+}
+
+extern "C" int xr_sample_static_init() {
+    float* p = nullptr;
+    return scratch_on_current_device(&p);
+}
+
+extern "C" int xr_sample_static(int* out, float* logits, int W, int V, int ld, const float* temp, const int* top_k,
+                                const float* top_p, const float* min_p, const float* repeat_penalty,
+                                const float* draw, const int* recent, const int* n_recent, int recent_cap,
+                                const int* exempt, int n_exempt, hipStream_t stream) {
+    XR_REQUIRE(W <= XR_SAMPLE_STATIC_MAX_ROWS, "sample_static: %d rows, the library's work area holds %d (use xr_sample with a work area of the caller's)",
+               W, XR_SAMPLE_STATIC_MAX_ROWS);
+    float* ws = nullptr;
+    const int rc = scratch_on_current_device(&ws);
+    if (rc != XR_OK) return rc;
+    return sample_launch(out, logits, W, V, ld, temp, top_k, top_p, min_p, repeat_penalty, draw, recent, n_recent,
+                         recent_cap, exempt, n_exempt, ws, stream);
 }
