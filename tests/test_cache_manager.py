@@ -133,3 +133,34 @@ def test_random_orders_keep_every_invariant(seed):
         m.release(rid)
     m.check()
     assert all(m.free_pages(g) == m.pages_per_group for g in range(len(groups))) and m.slots.n_free == 4
+
+
+def test_trim_gives_back_what_a_step_reserved_and_did_not_run():
+    m = CacheManager([FULL, WIN], page_size=4, pages_per_group=8, n_slots=2)
+    m.admit("a")
+    m.reserve("a", 6); m.advance("a", 6)
+    free = [m.free_pages(0), m.free_pages(1)]
+    m.reserve("a", 19)                 # three more pages in each group; then the step fails
+    assert m.free_pages(0) == free[0] - 3
+    m.trim("a")
+    assert [m.free_pages(0), m.free_pages(1)] == free and m.get("a").n_tokens == 6
+    assert m.pages_needed_new(9) == [3, 3]
+    m.check()
+    m.reserve("a", 7); m.advance("a", 7)
+    m.check()
+
+
+def test_a_reader_may_not_look_further_back_than_the_cache_it_reads_keeps():
+    """An entry of the run order that reads another entry's cache with a wider window, or with
+    none, would look up pages that the owner's window has given back."""
+    import torch
+    from xyntetik_runner_amd.cache import CacheStorage
+    dev = torch.device("cpu")
+    own, narrow, wide, full = KVSpec(1, 16, 8), KVSpec(1, 16, 4), KVSpec(1, 16, 12), KVSpec(1, 16, None)
+    ok = CacheStorage([own, narrow, own], [None] * 3, [None, 0, 0], 4, 3, 2, torch.float32, dev)
+    assert [lc.owns for lc in ok.layers] == [True, False, False] and ok.layers[1].k is ok.layers[0].k
+    for reader in (wide, full):
+        with pytest.raises(ValueError, match="keeps only the last 8 keys"):
+            CacheStorage([own, reader], [None] * 2, [None, 0], 4, 3, 2, torch.float32, dev)
+    # an owner that keeps every key serves any reader
+    CacheStorage([full, narrow, full], [None] * 3, [None, 0, 0], 4, 3, 2, torch.float32, dev)

@@ -177,9 +177,21 @@ def test_out_of_pages_is_an_error_that_changes_nothing(models):
     toks = reqs["r3"]
     runner.step([StepEntry("a", toks[:40], [])])
     free = runner.manager.free_pages()
+    slots = runner.manager.slots.n_free
     with pytest.raises(OutOfPages):
         runner.step([StepEntry("a", toks[40:60], []), StepEntry("b", toks[:30], [])])
     assert runner.manager.free_pages() == free and runner.length("a") == 40
+    # the request the failed step would have started is not live and holds no state slot
+    assert not runner.has("b") and runner.manager.slots.n_free == slots
+    # nor does a step leave anything behind that asks for more state slots than there are
+    with pytest.raises(OutOfPages):
+        runner.step([StepEntry("c", toks[:2], []), StepEntry("d", toks[:2], [])])
+    assert not runner.has("c") and not runner.has("d") and runner.manager.slots.n_free == slots
+    # or whose wanted places lie outside its tokens
+    with pytest.raises(ValueError):
+        runner.step([StepEntry("c", toks[:2], [2])])
+    assert not runner.has("c") and runner.manager.free_pages() == free
+    runner.manager.check()
     got = runner.step([StepEntry("a", toks[40:64], list(range(24)))]).cpu().numpy()
     mx, mean = logit_error(got, want["r3"][40:64])
     assert mx <= TOL["float32"][0]

@@ -114,6 +114,23 @@ class CacheManager:
     def pages_needed(self, req_id: Hashable, new_len: int) -> List[int]:
         return self._new_pages_needed(self.requests[req_id], new_len)
 
+    def pages_needed_new(self, new_len: int) -> List[int]:
+        """Pages per group that a request not yet admitted needs for its first ``new_len`` tokens
+        (all of them: a window gives pages back only once the tokens are cached)."""
+        return [self.pages_for(new_len)] * len(self.groups)
+
+    def trim(self, req_id: Hashable) -> None:
+        """Give back the pages reserved beyond the tokens the request holds (for a step that
+        reserved and then did not run)."""
+        rc = self.requests[req_id]
+        keep = self.pages_for(rc.n_tokens)
+        for gi, g in enumerate(self.groups):
+            table = rc.tables[gi]
+            while len(table) > keep:
+                page = table.pop()
+                if page >= 0:
+                    g.pool.give(page)
+
     def reserve(self, req_id: Hashable, new_len: int) -> None:
         """Make positions ``[n_tokens, new_len)`` writable in every group, or raise and change nothing."""
         rc = self.requests[req_id]

@@ -45,6 +45,11 @@ class CacheStorage:
                     if (okv.num_kv_heads, okv.head_dim) != (kv.num_kv_heads, kv.head_dim):
                         raise ValueError(f"run order entry {i} reads the cache of entry {owner}, "
                                          f"whose heads or head size differ")
+                    # the owner's window decides which pages exist: a reader that looks further
+                    # back would look up pages that were given back
+                    if okv.window is not None and (kv.window is None or kv.window > okv.window):
+                        raise ValueError(f"run order entry {i} (window {kv.window}) reads the cache of entry {owner}, "
+                                         f"which keeps only the last {okv.window} keys")
                 self.layers.append(LayerCache(src.group, page_size, False, src.k, src.v, None))
                 continue
             group, k, v = -1, None, None

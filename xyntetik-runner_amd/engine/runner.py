@@ -98,26 +98,53 @@ class ModelRunner:
             return None
         if token_source is not None and not self.takes_token_source(entries):
             raise ValueError("tokens on the device are taken only by a recorded decode step")
+        mgr = self.manager
         seen = set()
         for e in entries:
             if e.req_id in seen:
                 raise ValueError(f"request {e.req_id!r} appears twice in one step")
             seen.add(e.req_id)
-            if not self.has(e.req_id):
-                self.start(e.req_id)
-        mgr = self.manager
+            for w in e.want:
+                if not (0 <= w < len(e.tokens)):
+                    raise ValueError(f"request {e.req_id!r}: wanted place {w} is outside its {len(e.tokens)} tokens")
+        # Everything the step needs is counted before anything is taken: a state slot for every
+        # request that is new, pages for all entries.  If it does not fit the step raises and
+        # nothing has changed: no request admitted, no slot or page held.
+        new = [e for e in entries if not self.has(e.req_id)]
+        if len(new) > mgr.slots.n_free:
+            raise OutOfPages(f"this step starts {len(new)} requests, {mgr.slots.n_free} of {mgr.slots.size} state slots are free")
+        need = [0] * len(mgr.groups)
+        for e in entries:
+            if self.has(e.req_id):
+                per = mgr.pages_needed(e.req_id, mgr.get(e.req_id).n_tokens + len(e.tokens))
+            else:
+                per = mgr.pages_needed_new(len(e.tokens))
+            need = [a + b for a, b in zip(need, per)]
+        for gi, g in enumerate(mgr.groups):
+            if need[gi] > g.pool.n_free:
+                raise OutOfPages(f"this step needs {need[gi]} new pages in group {gi}, {g.pool.n_free} of {g.pool.size} are free")
+        for e in new:
+            self.start(e.req_id)
         rcs = [mgr.get(e.req_id) for e in entries]
-        # reserve for all or for none
-        spare = None
+        try:
+            for e, rc in zip(entries, rcs):
+                mgr.reserve(e.req_id, rc.n_tokens + len(e.tokens))
+            out = self._run(entries, rcs, token_source)
+        except BaseException:
+            # a step that failed leaves no request behind that it started and no page it reserved
+            started = {e.req_id for e in new}
+            for e in entries:
+                if e.req_id in started:
+                    mgr.release(e.req_id)
+                else:
+                    mgr.trim(e.req_id)
+            raise
         for e, rc in zip(entries, rcs):
-            need = mgr.pages_needed(e.req_id, rc.n_tokens + len(e.tokens))
-            if any(need):
-                spare = [s + n for s, n in zip(spare, need)] if spare else list(need)
-        for gi, g in enumerate(mgr.groups if spare else ()):
-            if spare[gi] > g.pool.n_free:
-                raise OutOfPages(f"this step needs {spare[gi]} new pages in group {gi}, {g.pool.n_free} of {g.pool.size} are free")
-        for e, rc in zip(entries, rcs):
-            mgr.reserve(e.req_id, rc.n_tokens + len(e.tokens))
+            mgr.advance(e.req_id, rc.n_tokens + len(e.tokens))
+        return out
+
+    def _run(self, entries, rcs, token_source) -> Optional[torch.Tensor]:
+        mgr = self.manager
         if self.graphs is not None and self.graphs.applies(entries):
             out = self._step_graph(entries, rcs, token_source)
         else:
@@ -125,8 +152,6 @@ class ModelRunner:
             self._zero_fresh_state(ctx)
             x = self.model.forward(ctx, self.storage.layers)
             out = self.model.logits(ctx, x, ctx.want_rows) if ctx.n_want else None
-        for e, rc in zip(entries, rcs):
-            mgr.advance(e.req_id, rc.n_tokens + len(e.tokens))
         return out
 
     def takes_token_source(self, entries: Sequence[StepEntry]) -> bool:

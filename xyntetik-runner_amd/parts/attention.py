@@ -20,6 +20,8 @@ import torch
 
 from .base import KVSpec, Mixer, ParamSpec, make_part, register_mixer
 
+MAX_HEAD_DIM = 256      # the attention and rotation kernels keep a head's channels in registers up to this size
+
 
 class PagedAttention(Mixer):
     takes_unscaled_rows = True
@@ -33,6 +35,9 @@ class PagedAttention(Mixer):
             raise ValueError(f"{num_heads} query heads are not a multiple of {num_kv_heads} key/value heads")
         if window is not None and window < 1:
             raise ValueError(f"attention window {window} must be at least 1")
+        if not (1 <= int(head_dim) <= MAX_HEAD_DIM):
+            # refused when the model is built, not at its first step
+            raise ValueError(f"attention head size {head_dim} is outside what the attention kernels take (1 to {MAX_HEAD_DIM})")
         self.hidden_size, self.num_heads = int(hidden_size), int(num_heads)
         self.num_kv_heads, self.head_dim = int(num_kv_heads), int(head_dim)
         self.window = int(window) if window is not None else None

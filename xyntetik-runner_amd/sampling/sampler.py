@@ -17,7 +17,7 @@ from .params import RECENT_WINDOW, SamplerState
 class Sampler:
     def __init__(self, ops, device, exempt_ids: Sequence[int] = ()):
         self.ops, self.device = ops, device
-        ex = list(exempt_ids)[:12]
+        ex = [int(t) for t in exempt_ids]          # (the kernel walks the list, however long)
         self.exempt = torch.tensor(ex, dtype=torch.int32, device=device) if ex else None
 
     @staticmethod
