@@ -132,5 +132,22 @@ def test_no_size_stands_in_code():
     for k in ("hidden_size", "num_heads", "num_kv_heads", "head_dim"):
         assert pa[k] != pb[k]
     assert sa.layers[0].feed_forward.params["intermediate_size"] != sb.layers[0].feed_forward.params["intermediate_size"]
-    assert sa.layers[0].mixer_norm.params["eps"] != sb.layers[0].mixer_norm.params["eps"]
+    assert sa.layers[0].norms["mixer_norm"].params["eps"] != sb.layers[0].norms["mixer_norm"].params["eps"]
     assert sa.vocab_size != sb.vocab_size and len(sa.layers) != len(sb.layers)
+
+
+def test_sizes_the_kernels_do_not_take_are_refused_when_the_model_is_built():
+    """A head size beyond what the attention and rotation kernels take is an error at load,
+    not at the first step (the reference refuses bad geometry at load too,
+    /root/reference/src/model.c:2295-2329)."""
+    from xyntetik_runner_amd.engine.model import Model
+    raw = dict(TINY_A, head_dim=272, num_attention_heads=2, num_key_value_heads=1)
+    arch, cfg = config_from_dict(raw)
+    with pytest.raises(ValueError, match="head size 272"):
+        Model(arch.build_spec(cfg))
+    Model(config_from_dict(dict(raw, head_dim=256))[0].build_spec(config_from_dict(dict(raw, head_dim=256))[1]))
+    # an activation the gated feed-forward's kernels do not have is named with the ones they have
+    from xyntetik_runner_amd.config import PartSpec
+    from xyntetik_runner_amd.parts import make_part
+    with pytest.raises(ValueError, match="silu"):
+        make_part("feed_forward", PartSpec("gated_mlp", {"hidden_size": 8, "intermediate_size": 16, "activation": "gelu"}))

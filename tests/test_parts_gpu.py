@@ -161,10 +161,15 @@ def test_embedding_head_and_block(rt_for, dt):
         head = make_part("head", PartSpec("linear", {"vocab_size": V, "hidden_size": E, "tied": tied}))
         assert (head.param_specs() == {}) == tied
         hw = bf(rng.normal(size=(V, E)))
-        head.bind({} if tied else {"weight": torch.tensor(hw, dtype=torch.float32).to(DT[dt]).to(DEV)}, rt, tied_to=emb.weight)
+        head.bind({} if tied else {"weight": torch.tensor(hw, dtype=torch.float32).to(DT[dt]).to(DEV)}, rt, tied_to=emb)
         h = bf(rng.normal(size=(3, E)))
         got = head.forward(Ctx(rt.ops), torch.tensor(h, dtype=torch.float32).to(DT[dt]).to(DEV))
         assert got.dtype == torch.float32 and rel(got, h @ (table if tied else hw).T) < 1e-5
+        if tied:
+            # one table for both: the head's, in the order its product reads it, from which the
+            # embedding gathers the same rows as before
+            assert emb.weight is head.weight
+            assert rel(emb.forward(Ctx(rt.ops), ids), table[[5, 0, 76, 0]]) == 0
 
     # the pre-norm arrangement with stand-in parts: x += 2*norm(x) then x += 3*norm(x)
     class N:
@@ -174,9 +179,13 @@ def test_embedding_head_and_block(rt_for, dt):
         def forward_add(self, ctx, cache, h, res): res += h.float()
     class F:
         def forward_add(self, ctx, h, res): res += h.float()
-    blk = make_block("prenorm", N(2.0), M(), N(3.0), F())
+    blk = make_block("prenorm", M(), F(), {"mixer_norm": N(2.0), "feed_forward_norm": N(3.0)})
     x = torch.ones(2, 4, device=DEV)
     blk.forward(Ctx(rt.ops), None, x)
     assert torch.equal(x, torch.full((2, 4), 12.0, device=DEV))      # 1 + 2 = 3; 3 + 9 = 12
     with pytest.raises(ValueError):
-        make_block("no-such-arrangement", None, None, None, None)
+        make_block("no-such-arrangement", None, None, {})
+    with pytest.raises(ValueError, match="feed_forward_norm"):     # the arrangement names its norms
+        make_block("prenorm", M(), F(), {"mixer_norm": N(2.0)})
+    with pytest.raises(ValueError, match="feed-forward"):
+        make_block("prenorm", M(), None, {"mixer_norm": N(2.0), "feed_forward_norm": N(3.0)})

@@ -72,8 +72,9 @@ def register_toy():
         mixers = [attn("layers.0.attn.", window=c["window"]),
                   PartSpec("toy_ema", {"hidden_size": E, "state_size": c["ema_size"], "decay": c["ema_decay"]}, prefix="layers.1.ema."),
                   attn("layers.2.attn.", window=c["window"], kv_shared=True)]
-        layers = [LayerSpec(mixer=m, feed_forward=mlp(f"layers.{i}.mlp."), mixer_norm=norm(f"layers.{i}.norm1."),
-                            feed_forward_norm=norm(f"layers.{i}.norm2.")) for i, m in enumerate(mixers)]
+        layers = [LayerSpec(mixer=m, feed_forward=mlp(f"layers.{i}.mlp."),
+                            norms={"mixer_norm": norm(f"layers.{i}.norm1."), "feed_forward_norm": norm(f"layers.{i}.norm2.")})
+                  for i, m in enumerate(mixers)]
         return ModelSpec(
             architecture="ToyForCausalLM", hidden_size=E, vocab_size=c["vocab_size"], max_position=c["max_position_embeddings"],
             embedding=PartSpec("token_embedding", {"vocab_size": c["vocab_size"], "hidden_size": E}, prefix="embed."),
@@ -215,3 +216,105 @@ def test_unknown_part_kind_is_a_clear_error():
     with pytest.raises(ValueError) as e:
         make_part("mixer", PartSpec("no_such_mixer", {}))
     assert "no_such_mixer" in str(e.value) and "paged_attention" in str(e.value)
+
+
+# ----------------------------------------------------------------------------- windows through captured decode steps
+TOYW_CONFIG = {
+    "architectures": ["ToyWindowForCausalLM"], "hidden_size": 64, "num_attention_heads": 4, "num_key_value_heads": 2,
+    "head_dim": 32, "intermediate_size": 96, "vocab_size": 131, "window": 40, "rms_norm_eps": 1e-5,
+    "rope_theta": 10000.0, "max_position_embeddings": 512,
+}
+
+
+def register_toy_window():
+    """Two stateless attention layers, the first with a window of 40 keys, the second with all
+    keys: two cache groups, and decode steps that a HIP graph can record."""
+    from xyntetik_runner_amd.config import ExecStep, Fields, LayerSpec, ModelSpec, PartSpec, register_architecture
+
+    def parse(raw):
+        f = Fields(raw)
+        return {k: (f.number(k) if isinstance(TOYW_CONFIG[k], float) else f.integer(k, lo=1, hi=1 << 20))
+                for k in TOYW_CONFIG if k != "architectures"}
+
+    def build(c):
+        E = c["hidden_size"]
+        norm = lambda p: PartSpec("rmsnorm", {"size": E, "eps": c["rms_norm_eps"]}, prefix=p)
+        rot = PartSpec("rotary", {"head_dim": c["head_dim"], "theta": c["rope_theta"]})
+        attn = lambda p, **kw: PartSpec("paged_attention", dict(
+            hidden_size=E, num_heads=c["num_attention_heads"], num_kv_heads=c["num_key_value_heads"],
+            head_dim=c["head_dim"], position=rot, **kw), prefix=p)
+        mlp = lambda p: PartSpec("gated_mlp", {"hidden_size": E, "intermediate_size": c["intermediate_size"]}, prefix=p)
+        layers = [LayerSpec(mixer=attn(f"layers.{i}.attn.", window=win), feed_forward=mlp(f"layers.{i}.mlp."),
+                            norms={"mixer_norm": norm(f"layers.{i}.norm1."), "feed_forward_norm": norm(f"layers.{i}.norm2.")})
+                  for i, win in enumerate([c["window"], None])]
+        return ModelSpec(
+            architecture="ToyWindowForCausalLM", hidden_size=E, vocab_size=c["vocab_size"],
+            max_position=c["max_position_embeddings"],
+            embedding=PartSpec("token_embedding", {"vocab_size": c["vocab_size"], "hidden_size": E}, prefix="embed."),
+            layers=layers, order=[ExecStep(0), ExecStep(1)], final_norm=norm("norm."),
+            head=PartSpec("linear", {"vocab_size": c["vocab_size"], "hidden_size": E, "tied": False}, prefix="head."))
+
+    register_architecture("ToyWindowForCausalLM", parse, build, replace=True)
+
+
+def plain_toy_window(cfg, w, tokens):
+    E, H, Hk, D = cfg["hidden_size"], cfg["num_attention_heads"], cfg["num_key_value_heads"], cfg["head_dim"]
+    T = len(tokens)
+    inv = P.rope_inv_freq(D, cfg["rope_theta"])
+    pos = np.arange(T)
+    x = w["embed.weight"][tokens].copy()
+    for i, win in enumerate([cfg["window"], None]):
+        p = f"layers.{i}."
+        h = P.rmsnorm(x, w[p + "norm1.weight"], cfg["rms_norm_eps"])
+        q = P.rope((h @ w[p + "attn.q_proj.weight"].T).reshape(T, H, D), pos, inv)
+        k = P.rope((h @ w[p + "attn.k_proj.weight"].T).reshape(T, Hk, D), pos, inv)
+        v = (h @ w[p + "attn.v_proj.weight"].T).reshape(T, Hk, D)
+        x = x + P.attention(q, k, v, 1 / math.sqrt(D), win).reshape(T, H * D) @ w[p + "attn.o_proj.weight"].T
+        h = P.rmsnorm(x, w[p + "norm2.weight"], cfg["rms_norm_eps"])
+        x = x + P.mlp(h, w[p + "mlp.gate_proj.weight"], w[p + "mlp.up_proj.weight"], w[p + "mlp.down_proj.weight"])
+    return P.rmsnorm(x, w["norm.weight"], cfg["rms_norm_eps"]) @ w["head.weight"].T
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_windowed_decoding_through_captured_steps(tmp_path, dtype):
+    """Two requests decode far past the window through recorded graphs (bfloat16: the MFMA
+    attention, pages of 16): the windowed group's block tables are rewritten every step as pages
+    are given back (their entries become -1), the other group's only grow.  Every page starts
+    as NaN, so a read of a page that was given back, or beyond a request's length, shows."""
+    from xyntetik_runner_amd.config import unregister_architecture
+    from xyntetik_runner_amd.engine import ModelRunner, StepEntry
+    from xyntetik_runner_amd.weights import write_random_model
+    register_toy_window()
+    try:
+        d = write_random_model(TOYW_CONFIG, str(tmp_path / "toyw"), seed=6, std=0.08, norm_jitter=0.1)
+        cfg, w = P.load_folder(d)
+        runner = ModelRunner.from_folder(d, dtype=dtype, max_tokens=512, page_size=16, max_requests=2)
+        assert runner.graphs.usable and [g.spec.window for g in runner.manager.groups] == [40, None]
+        for lc in runner.storage.layers:
+            lc.k.fill_(float("nan")); lc.v.fill_(float("nan"))
+        reqs = {"a": prompt_ids(200, cfg["vocab_size"], 41), "b": prompt_ids(170, cfg["vocab_size"], 42)}
+        want = {k: plain_toy_window(cfg, w, v) for k, v in reqs.items()}
+        n0 = {"a": 30, "b": 7}
+        got = {k: [] for k in reqs}
+        out = runner.step([StepEntry(k, reqs[k][:n0[k]], list(range(n0[k]))) for k in reqs]).cpu().numpy()
+        got["a"].append(out[:30]); got["b"].append(out[30:])
+        fewest = 99
+        for i in range(160):
+            entries = [StepEntry(k, [reqs[k][n0[k] + i]], [0]) for k in reqs]
+            out = runner.step(entries).cpu().numpy()
+            for r, k in enumerate(reqs):
+                got[k].append(out[r:r + 1])
+            runner.manager.check()
+            tabs = runner.manager.get("a").tables
+            fewest = min(fewest, sum(p >= 0 for p in tabs[0]))
+            assert sum(p >= 0 for p in tabs[0]) <= 40 // 16 + 2 and all(p >= 0 for p in tabs[1])
+        assert runner.graphs.replays >= 150 and fewest <= 4
+        assert -1 in runner.manager.get("a").tables[0]           # pages were given back while it decoded
+        tol = (2e-5, 2e-6) if dtype == "float32" else (2e-2, 3e-3)
+        for k in reqs:
+            rows = np.concatenate(got[k])
+            assert np.isfinite(rows).all()
+            mx, mean = logit_error(rows, want[k][:len(rows)])
+            assert mx <= tol[0] and mean <= tol[1], (k, mx, mean)
+    finally:
+        unregister_architecture("ToyWindowForCausalLM")

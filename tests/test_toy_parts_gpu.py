@@ -1,8 +1,9 @@
 """More generality with toy parts defined here only: a feed-forward that routes every token to
-one of several experts, and a position encoding that is no rotation.  Both are registered
-from this file, named by a toy architecture's spec in one layer beside the framework's own
-parts in the other, and replayed through the framework's step function, cache and trace
-program in every way of cutting the work.  They stand for no model of anyone's.
+one of several experts, a position encoding that is no rotation, an arrangement with a third
+norm (after the mixer) and one without a feed-forward.  All are registered from this file,
+named by a toy architecture's spec beside the framework's own parts, and replayed through the
+framework's step function, cache and trace program in every way of cutting the work.  They
+stand for no model of anyone's.
 """
 import io
 import math
@@ -33,8 +34,28 @@ def wave_table(positions, head_dim, base):
 
 def register_toy2():
     from xyntetik_runner_amd.config import ExecStep, Fields, LayerSpec, ModelSpec, PartSpec, register_architecture
-    from xyntetik_runner_amd.parts import (FeedForward, ParamSpec, PositionEncoding, register_feed_forward,
-                                           register_position)
+    from xyntetik_runner_amd.parts import (Block, FeedForward, ParamSpec, PositionEncoding, register_block,
+                                           register_feed_forward, register_position)
+
+    class SandwichBlock(Block):
+        """x += post(mixer(pre(x))); x += feed_forward(norm(x)): three norms, named by the layer's spec."""
+        norm_names = ("mixer_norm", "mixer_post_norm", "feed_forward_norm")
+
+        def forward(self, ctx, cache, x):
+            n = self.norms
+            y = self.mixer.forward(ctx, cache, n["mixer_norm"].forward(ctx, x))
+            if y.dtype != torch.float32:
+                y = ctx.ops.convert(y, torch.float32)
+            ctx.ops.add_(x, n["mixer_post_norm"].forward(ctx, y))
+            self.feed_forward.forward_add(ctx, n["feed_forward_norm"].forward(ctx, x), x)
+
+    class MixerOnlyBlock(Block):
+        """x += mixer(norm(x)) and nothing else: a layer without a feed-forward."""
+        norm_names = ("mixer_norm",)
+        needs_feed_forward = False
+
+        def forward(self, ctx, cache, x):
+            self.mixer.forward_add(ctx, cache, self.norms["mixer_norm"].forward(ctx, x), x)
 
     class WavePosition(PositionEncoding):
         """q and k get a position-dependent vector added (the same for every head)."""
@@ -108,18 +129,23 @@ def register_toy2():
             LayerSpec(mixer=attn("layers.0.attn.", wave),
                       feed_forward=PartSpec("toy_routed", {"hidden_size": E, "expert_size": c["expert_size"],
                                                            "num_experts": c["num_experts"]}, prefix="layers.0.moe."),
-                      mixer_norm=norm("layers.0.norm1."), feed_forward_norm=norm("layers.0.norm2.")),
+                      norms={"mixer_norm": norm("layers.0.norm1."), "feed_forward_norm": norm("layers.0.norm2.")}),
             LayerSpec(mixer=attn("layers.1.attn.", rot),
                       feed_forward=PartSpec("gated_mlp", {"hidden_size": E, "intermediate_size": c["intermediate_size"]},
                                             prefix="layers.1.mlp."),
-                      mixer_norm=norm("layers.1.norm1."), feed_forward_norm=norm("layers.1.norm2.")),
+                      norms={"mixer_norm": norm("layers.1.norm1."), "mixer_post_norm": norm("layers.1.norm_post."),
+                             "feed_forward_norm": norm("layers.1.norm2.")}, block="toy_sandwich"),
+            LayerSpec(mixer=attn("layers.2.attn.", rot), norms={"mixer_norm": norm("layers.2.norm1.")},
+                      block="toy_mixer_only"),
         ]
         return ModelSpec(
             architecture="Toy2ForCausalLM", hidden_size=E, vocab_size=c["vocab_size"], max_position=c["max_position_embeddings"],
             embedding=PartSpec("token_embedding", {"vocab_size": c["vocab_size"], "hidden_size": E}, prefix="embed."),
-            layers=layers, order=[ExecStep(0), ExecStep(1)], final_norm=norm("norm."),
+            layers=layers, order=[ExecStep(0), ExecStep(1), ExecStep(2)], final_norm=norm("norm."),
             head=PartSpec("linear", {"vocab_size": c["vocab_size"], "hidden_size": E, "tied": False}, prefix="head."))
 
+    register_block("toy_sandwich", SandwichBlock, replace=True)
+    register_block("toy_mixer_only", MixerOnlyBlock, replace=True)
     register_position("toy_wave", WavePosition, replace=True)
     register_feed_forward("toy_routed", RoutedMLP, replace=True)
     register_architecture("Toy2ForCausalLM", parse, build, replace=True)
@@ -130,7 +156,7 @@ def plain_toy2(cfg, w, tokens):
     T, F = len(tokens), cfg["expert_size"]
     pos = np.arange(T)
     x = w["embed.weight"][tokens].copy()
-    for i in range(2):
+    for i in range(3):
         p = f"layers.{i}."
         h = P.rmsnorm(x, w[p + "norm1.weight"], cfg["rms_norm_eps"])
         q = (h @ w[p + "attn.q_proj.weight"].T).reshape(T, H, D)
@@ -142,7 +168,12 @@ def plain_toy2(cfg, w, tokens):
         else:
             inv = P.rope_inv_freq(D, cfg["rope_theta"])
             q, k = P.rope(q, pos, inv), P.rope(k, pos, inv)
-        x = x + P.attention(q, k, v, 1 / math.sqrt(D)).reshape(T, H * D) @ w[p + "attn.o_proj.weight"].T
+        a = P.attention(q, k, v, 1 / math.sqrt(D)).reshape(T, H * D) @ w[p + "attn.o_proj.weight"].T
+        if i == 1:                       # the arrangement with a norm after the mixer
+            a = P.rmsnorm(a, w[p + "norm_post.weight"], cfg["rms_norm_eps"])
+        x = x + a
+        if i == 2:                       # the arrangement without a feed-forward
+            continue
         h = P.rmsnorm(x, w[p + "norm2.weight"], cfg["rms_norm_eps"])
         if i == 0:
             prob = np.stack([P.softmax(row) for row in h @ w[p + "moe.router.weight"].T])
@@ -171,6 +202,8 @@ def toy2(tmp_path_factory):
     unregister_architecture("Toy2ForCausalLM")
     unregister("position", "toy_wave")
     unregister("feed_forward", "toy_routed")
+    unregister("block", "toy_sandwich")
+    unregister("block", "toy_mixer_only")
 
 
 def test_the_router_uses_every_expert(toy2):

@@ -27,10 +27,11 @@ def build_llama_spec(cfg: LlamaConfig) -> ModelSpec:
             feed_forward=PartSpec("gated_mlp", {
                 "hidden_size": cfg.hidden_size, "intermediate_size": cfg.intermediate_size,
                 "activation": cfg.hidden_act, "bias": cfg.mlp_bias}, prefix=p + "mlp."),
-            mixer_norm=PartSpec("rmsnorm", {"size": cfg.hidden_size, "eps": cfg.rms_norm_eps},
-                                prefix=p + "input_layernorm."),
-            feed_forward_norm=PartSpec("rmsnorm", {"size": cfg.hidden_size, "eps": cfg.rms_norm_eps},
-                                       prefix=p + "post_attention_layernorm."),
+            norms={
+                "mixer_norm": PartSpec("rmsnorm", {"size": cfg.hidden_size, "eps": cfg.rms_norm_eps},
+                                       prefix=p + "input_layernorm."),
+                "feed_forward_norm": PartSpec("rmsnorm", {"size": cfg.hidden_size, "eps": cfg.rms_norm_eps},
+                                              prefix=p + "post_attention_layernorm.")},
             block="prenorm"))
     return ModelSpec(
         architecture=cfg.architecture,

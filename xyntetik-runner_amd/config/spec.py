@@ -13,7 +13,7 @@ which layers are windowed, which layer owns the cache rows a layer reads
 from __future__ import annotations
 
 from dataclasses import dataclass, field
-from typing import Any, Dict, List, Optional
+from typing import Any, Dict, List, Mapping, Optional
 
 
 @dataclass(frozen=True)
@@ -31,13 +31,15 @@ class PartSpec:
 class LayerSpec:
     """One layer's parts.
 
-    ``block`` names the arrangement (how norms, mixer, feed-forward and the
-    residual sums follow each other).
+    ``block`` names the arrangement (how norms, mixer, feed-forward and the residual sums
+    follow each other); ``norms`` holds the norms that arrangement has, under the names it
+    gives them ("prenorm": ``mixer_norm`` and ``feed_forward_norm``; an arrangement with a
+    third norm simply names three).  An arrangement may do without a mixer or without a
+    feed-forward.
     """
-    mixer: PartSpec
-    feed_forward: PartSpec
-    mixer_norm: PartSpec
-    feed_forward_norm: PartSpec
+    mixer: Optional[PartSpec] = None
+    feed_forward: Optional[PartSpec] = None
+    norms: Mapping[str, PartSpec] = field(default_factory=dict)
     block: str = "prenorm"
 
 

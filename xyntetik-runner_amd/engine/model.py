@@ -23,8 +23,10 @@ class Model:
         self.blocks: List[Block] = []
         for ls in spec.layers:
             self.blocks.append(make_block(
-                ls.block, make_part("norm", ls.mixer_norm), make_part("mixer", ls.mixer),
-                make_part("norm", ls.feed_forward_norm), make_part("feed_forward", ls.feed_forward)))
+                ls.block,
+                make_part("mixer", ls.mixer) if ls.mixer is not None else None,
+                make_part("feed_forward", ls.feed_forward) if ls.feed_forward is not None else None,
+                {name: make_part("norm", ps) for name, ps in ls.norms.items()}))
         self.final_norm = make_part("norm", spec.final_norm)
         self.head = make_part("head", spec.head)
         self.rt: Optional[Runtime] = None
@@ -33,10 +35,12 @@ class Model:
     def _named_parts(self):
         yield self.spec.embedding.prefix, self.embedding
         for ls, blk in zip(self.spec.layers, self.blocks):
-            yield ls.mixer_norm.prefix, blk.mixer_norm
-            yield ls.mixer.prefix, blk.mixer
-            yield ls.feed_forward_norm.prefix, blk.feed_forward_norm
-            yield ls.feed_forward.prefix, blk.feed_forward
+            for name, ps in ls.norms.items():
+                yield ps.prefix, blk.norms[name]
+            if ls.mixer is not None:
+                yield ls.mixer.prefix, blk.mixer
+            if ls.feed_forward is not None:
+                yield ls.feed_forward.prefix, blk.feed_forward
         yield self.spec.final_norm.prefix, self.final_norm
         yield self.spec.head.prefix, self.head
 
@@ -64,7 +68,7 @@ class Model:
         for prefix, part in self._named_parts():
             mine = {rel: tensors.pop(prefix + rel) for rel in part.param_specs() if prefix + rel in tensors}
             if part is self.head:
-                part.bind(mine, rt, tied_to=getattr(self.embedding, "weight", None))
+                part.bind(mine, rt, tied_to=self.embedding)
             else:
                 part.bind(mine, rt)
 
@@ -74,8 +78,8 @@ class Model:
         kv, st, of = [], [], []
         for step in self.spec.order:
             mixer = self.blocks[step.layer].mixer
-            kv.append(mixer.kv_spec())
-            st.append(mixer.state_spec() if step.cache_of is None else None)
+            kv.append(mixer.kv_spec() if mixer is not None else None)
+            st.append(mixer.state_spec() if mixer is not None and step.cache_of is None else None)
             of.append(step.cache_of)
         return kv, st, of
 

@@ -20,7 +20,8 @@ Families and what each must offer:
   residual stream (the default calls ``forward``; a part with a fused epilogue
   overrides it).
 * ``FeedForward``: ``forward(ctx, h) -> y`` and ``forward_add(ctx, h, residual)``.
-* ``Block``: the arrangement; ``forward(ctx, cache, x)`` updates ``x`` in place.
+* ``Block``: the arrangement; it names its norms (``norm_names``), may do without a mixer or a
+  feed-forward, and ``forward(ctx, cache, x)`` updates ``x`` in place.
 
 Optional, for fewer kernels when a few tokens are decoded: a mixer or feed-forward
 may override ``forward_add_norm(..., residual, norm, defer)``, which adds into the
@@ -29,7 +30,7 @@ both (``Ops.linear_add_rmsnorm``).  With ``defer`` the result may be an
 ``UnscaledRows`` (the rows still lack the division by their root mean square, which
 the next product applies to its own result); a caller sets ``defer`` only if the part
 that reads the result has ``takes_unscaled_rows`` set, which says that it hands ``h``
-to ``Ops.linear`` or ``Ops.linear_swiglu`` and reads nothing else of it than its
+to ``Ops.linear`` or ``Ops.linear_gated`` and reads nothing else of it than its
 ``shape``, ``dtype`` and ``device``.  A block with ``chained`` set takes the result of
 its first norm from the block before it and makes the next block's
 (``entry_norm()``); every default does the plain thing.
@@ -149,7 +150,7 @@ class FeedForward(Part):
     def forward(self, ctx, h: torch.Tensor) -> torch.Tensor:
         raise NotImplementedError
 
-    #: True if ``h`` may be an ``UnscaledRows`` (it only goes into ``Ops.linear`` or ``Ops.linear_swiglu``)
+    #: True if ``h`` may be an ``UnscaledRows`` (it only goes into ``Ops.linear`` or ``Ops.linear_gated``)
     takes_unscaled_rows = False
 
     def forward_add(self, ctx, h: torch.Tensor, residual: torch.Tensor) -> None:
@@ -162,17 +163,32 @@ class FeedForward(Part):
 
 
 class Block:
-    """An arrangement of two norms, a mixer and a feed-forward around the residual stream."""
+    """An arrangement of a layer's parts around the residual stream: a mixer, a feed-forward
+    (an arrangement may do without either) and the norms it names in ``norm_names``."""
 
-    def __init__(self, mixer_norm: Norm, mixer: Mixer, feed_forward_norm: Norm, feed_forward: FeedForward):
-        self.mixer_norm = mixer_norm
-        self.mixer = mixer
-        self.feed_forward_norm = feed_forward_norm
-        self.feed_forward = feed_forward
+    #: the norms this arrangement has, by the names a ``LayerSpec`` gives them
+    norm_names: Tuple[str, ...] = ()
+    needs_mixer = True
+    needs_feed_forward = True
+
+    def __init__(self, mixer: Optional[Mixer], feed_forward: Optional[FeedForward], norms: Dict[str, Norm]):
+        kind = type(self).__name__
+        if (mixer is None) == self.needs_mixer or (feed_forward is None) == self.needs_feed_forward:
+            raise ValueError(f"{kind}: this arrangement has {'a' if self.needs_mixer else 'no'} mixer and "
+                             f"{'a' if self.needs_feed_forward else 'no'} feed-forward")
+        if set(norms) != set(self.norm_names):
+            raise ValueError(f"{kind}: this arrangement has the norms {sorted(self.norm_names)}, "
+                             f"the layer names {sorted(norms)}")
+        self.mixer, self.feed_forward, self.norms = mixer, feed_forward, dict(norms)
 
     def parts(self):
-        return {"mixer_norm": self.mixer_norm, "mixer": self.mixer,
-                "feed_forward_norm": self.feed_forward_norm, "feed_forward": self.feed_forward}
+        """Every part of the layer by name."""
+        out = dict(self.norms)
+        if self.mixer is not None:
+            out["mixer"] = self.mixer
+        if self.feed_forward is not None:
+            out["feed_forward"] = self.feed_forward
+        return out
 
     #: True if ``forward`` also takes ``h`` (the result of this block's first norm, made by the
     #: block before) and ``after`` (the next block's ``entry_norm()``), and returns the next
@@ -254,8 +270,9 @@ def make_part(family: str, spec) -> Any:
     return reg[spec.kind](**spec.params)
 
 
-def make_block(kind: str, mixer_norm, mixer, feed_forward_norm, feed_forward) -> Block:
+def make_block(kind: str, mixer, feed_forward, norms) -> Block:
+    """The arrangement ``kind`` around the given parts (``norms``: name -> norm)."""
     reg = _REGISTRIES["block"]
     if kind not in reg:
         raise ValueError(f"no block arrangement {kind!r}; registered: {sorted(reg)}")
-    return reg[kind](mixer_norm, mixer, feed_forward_norm, feed_forward)
+    return reg[kind](mixer, feed_forward, norms)

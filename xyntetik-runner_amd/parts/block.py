@@ -15,6 +15,15 @@ def _takes_unscaled(part) -> bool:
 
 class PreNormBlock(Block):
     chained = True
+    norm_names = ("mixer_norm", "feed_forward_norm")
+
+    @property
+    def mixer_norm(self):
+        return self.norms["mixer_norm"]
+
+    @property
+    def feed_forward_norm(self):
+        return self.norms["feed_forward_norm"]
 
     def entry_norm(self):
         return self.mixer_norm, _takes_unscaled(self.mixer)

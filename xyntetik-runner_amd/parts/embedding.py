@@ -21,6 +21,13 @@ class TokenEmbedding(Part):
         self.rt = rt
         self.weight = tensors[self.weight_name]
 
+    def share_table(self, table) -> None:
+        """Gather from ``table`` from now on: the same values in another layout (a tied output
+        head's packed copy), so that the model keeps the table once."""
+        if tuple(table.shape) != (self.vocab_size, self.hidden_size):
+            raise ValueError(f"a table of {tuple(table.shape)} cannot stand for one of {(self.vocab_size, self.hidden_size)}")
+        self.weight = table
+
     def forward(self, ctx, token_ids):
         return self.rt.ops.embedding(self.weight, token_ids, self.scale)
 

@@ -22,13 +22,17 @@ class LinearHead(Part):
         return {self.weight_name: ParamSpec((self.vocab_size, self.hidden_size), role="matrix")}
 
     def bind(self, tensors, rt, tied_to=None) -> None:
+        """``tied_to``: the embedding part whose table a tied head uses."""
         self.rt = rt
-        weight = tied_to if self.tied else tensors[self.weight_name]
+        weight = getattr(tied_to, "weight", None) if self.tied else tensors[self.weight_name]
         if weight is None:
             raise ValueError("a tied head needs the embedding table")
-        # in the kernels' own order where they have one (a tied head then keeps a copy of its own:
-        # the embedding gathers rows from the table as it is stored)
+        # In the kernels' own order where they have one.  A tied head shares one buffer with the
+        # embedding (/root/reference/src/model.c:2354 aliases the pointer): where the table is
+        # packed for the head's product, the embedding gathers its rows from the packed table too.
         self.weight = rt.ops.pack_weight(weight)
+        if self.tied and self.weight is not weight and hasattr(tied_to, "share_table"):
+            tied_to.share_table(self.weight)
 
     def forward(self, ctx, h):
         return self.rt.ops.linear(h, self.weight, out_dtype=torch.float32)
