@@ -27,7 +27,7 @@ def rel(got, want):
 
 
 # ------------------------------------------------------------------ small kernels
-@pytest.mark.parametrize("V,E", [(100, 72), (333, 4100)])
+@pytest.mark.parametrize("V,E", [(100, 72), (333, 4100), (77, 4104)])
 @pytest.mark.parametrize("dt", ["float32", "bfloat16"])
 def test_embedding(ops, V, E, dt):
     table = torch.randn(V, E, device=DEV).to(DT[dt])
@@ -36,6 +36,10 @@ def test_embedding(ops, V, E, dt):
     want = table.float()[torch.tensor([0, V - 1, 5, 0, 0, 17], device=DEV)]       # out of range reads row 0
     assert got.dtype == torch.float32 and torch.equal(got, want)
     assert torch.equal(ops.embedding(table, ids, scale=2.0), want * 2)
+    if dt == "bfloat16":            # the same rows from the table in the matrix kernels' packed order
+        packed = ops.pack_weight(table)
+        assert (packed is not table) == (E % 8 == 0)            # (a width that is no multiple of 8 is not packed)
+        assert torch.equal(ops.embedding(packed, ids, scale=1.0), want)
 
 
 @pytest.mark.parametrize("E", [8, 100, 4096, 5000])
@@ -102,6 +106,30 @@ def test_linear_bf16_mfma(ops, M, N, K):
         for variant in (12, 1014, 17, 26):               # tile shapes the dispatch may pick for other sizes
             assert rel(ops.linear(a, w, bias=b, out_dtype=torch.float32, variant=variant),
                        a.double() @ w.double().T + b.double()) < 1e-5
+
+
+@pytest.mark.parametrize("M", [8, 40, 300])
+def test_gated_product_with_gates_far_from_zero(ops, M):
+    """Gate values of -200 and +200 through the fused epilogues: the weight-streaming kernel's
+    (8 rows), the kernel's that adds up K ranges (40 rows) and the tile kernel's, which uses the
+    hardware's 2^x and reciprocal (300 rows).  act(-200) * up is 0 and no NaN
+    (/root/reference/src/model.c:4442-4452), act(200) is 200."""
+    from xyntetik_runner_amd.csrc.ops import PackedWeight
+    K, F = 64, 96
+    a = torch.ones(M, K, device=DEV).bfloat16()
+    wg = torch.empty(F, K, device=DEV)
+    wg[:F // 2] = -200.0 / K
+    wg[F // 2:] = 200.0 / K
+    w2 = torch.cat([wg, torch.randn(F, K, device=DEV) * 0.1]).bfloat16()
+    up = a.double() @ w2[F:].double().T
+    for w in (w2, ops.pack_weight(w2, gated=True)):
+        got = ops.linear_gated(a, w, activation="silu").float()
+        assert torch.isfinite(got).all()
+        assert (got[:, :F // 2] == 0).all()
+        assert rel(got[:, F // 2:], 200.0 * up[:, F // 2:]) < 6e-3
+    assert isinstance(ops.pack_weight(w2, gated=True), PackedWeight)
+    with pytest.raises(Exception, match="not built into the kernels"):
+        ops.linear_gated(a, w2, activation="no-such-activation")
 
 
 @pytest.mark.parametrize("M", [8, 40, 300])
@@ -587,6 +615,8 @@ ATTN_CASES = [
     (5, 1, 80, 32, None, [300, 10], [1, 3]),       # decoding with a head size that is no power of two
     (4, 2, 256, 16, 600, [700, 3], [1, 2]),        # the largest head, small pages, a window that has given pages back
     (6, 2, 48, 64, None, [5000], [1]),             # more than 64 pages: the page numbers are fetched again on the way
+    (64, 8, 128, 64, None, [900, 0, 130], [1, 70, 3]),   # 8 query heads a key/value head: 4 tokens x 8 heads in a 32-row block
+    (32, 32, 128, 64, None, [700, 0, 64], [1, 150, 2]),  # one query head a key/value head, 32 of them: 32 tokens in a block
 ]
 
 

@@ -18,12 +18,29 @@ __global__ void k_embedding(float* __restrict__ out, const TW* __restrict__ tabl
     for (int i = threadIdx.x; i < E; i += blockDim.x) o[i] = ld<TW>(row, i) * scale;
 }
 
+// The same from a bfloat16 table in the matrix kernels' packed order (blocks of 16 rows x 32
+// columns, 1 KB each, [row group][column block][row][column]): a model that ties its output
+// head to the embedding then keeps the table once, in the order the head's product reads it.
+__global__ void k_embedding_packed(float* __restrict__ out, const bf16_t* __restrict__ table,
+                                   const int* __restrict__ ids, int E, int V, float scale) {
+    int t = blockIdx.x;
+    int id = ids[t];
+    if (id < 0 || id >= V) id = 0;
+    const size_t kblocks = (size_t)((E + 31) / 32);
+    const bf16_t* grp = table + (size_t)(id >> 4) * kblocks * 512 + (id & 15) * 32;
+    float* o = out + (size_t)t * E;
+    for (int i = threadIdx.x; i < E; i += blockDim.x) o[i] = bf16_to_f32(grp[(size_t)(i >> 5) * 512 + (i & 31)]) * scale;
+}
+
 extern "C" int xr_embedding(float* out, const void* table, const int* ids, int T, int E, int V,
-                            float scale, int table_dtype, hipStream_t stream) {
+                            float scale, int table_dtype, int packed, hipStream_t stream) {
     XR_REQUIRE(T >= 0 && E > 0 && V > 0, "embedding: bad sizes T=%d E=%d V=%d", T, E, V);
     XR_REQUIRE(table_dtype == XR_F32 || table_dtype == XR_BF16, "embedding: bad dtype %d", table_dtype);
+    XR_REQUIRE(!packed || table_dtype == XR_BF16, "embedding: a packed table is bfloat16");
     if (T == 0) return XR_OK;
-    if (table_dtype == XR_F32)
+    if (packed)
+        k_embedding_packed<<<T, 256, 0, stream>>>(out, (const bf16_t*)table, ids, E, V, scale);
+    else if (table_dtype == XR_F32)
         k_embedding<float><<<T, 256, 0, stream>>>(out, (const float*)table, ids, E, V, scale);
     else
         k_embedding<bf16_t><<<T, 256, 0, stream>>>(out, (const bf16_t*)table, ids, E, V, scale);
@@ -304,29 +321,30 @@ extern "C" int xr_rope_kv_write(const float* q_in, const float* k_in, const floa
     return XR_OK;
 }
 
-// ---------------------------------------------------------------- SiLU gate
-// h = silu(g) * u, silu(g) = g / (1 + exp(-g)) (/root/reference/src/model.c:4451-4452,
+// ---------------------------------------------------------------- gate
+// h = act(g) * u; act = SiLU: g / (1 + exp(-g)) (/root/reference/src/model.c:4451-4452,
 // /root/reference/src/kernels.cu:2868-2874).  gu row = [gate(F) | up(F)].
 template <typename TI, typename TO>
-__global__ void k_silu_mul(TO* __restrict__ out, const TI* __restrict__ gu, int F, int ld_gu, size_t n) {
+__global__ void k_gate_mul(TO* __restrict__ out, const TI* __restrict__ gu, int F, int ld_gu, size_t n, int act) {
     size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= n) return;
     size_t t = i / F;
     int c = (int)(i - t * F);
     float g = ld<TI>(gu, t * ld_gu + c);
     float u = ld<TI>(gu, t * ld_gu + F + c);
-    st<TO>(out, i, (g / (1.0f + expf(-g))) * u);
+    st<TO>(out, i, gate_act<false>(act, g) * u);
 }
 
-extern "C" int xr_silu_mul(void* out, const void* gu, int T, int F, int ld_gu, int dtype, hipStream_t stream) {
-    XR_REQUIRE(T >= 0 && F > 0 && ld_gu >= 2 * F, "silu_mul: bad sizes T=%d F=%d ld=%d", T, F, ld_gu);
+extern "C" int xr_gate_mul(void* out, const void* gu, int T, int F, int ld_gu, int dtype, int act, hipStream_t stream) {
+    XR_REQUIRE(T >= 0 && F > 0 && ld_gu >= 2 * F, "gate_mul: bad sizes T=%d F=%d ld=%d", T, F, ld_gu);
+    XR_REQUIRE(act >= 0 && act < XR_ACT_COUNT, "gate_mul: unknown activation code %d", act);
     size_t n = (size_t)T * F;
     if (n == 0) return XR_OK;
     unsigned blocks = (unsigned)((n + 255) / 256);
-    if (dtype == XR_F32) k_silu_mul<float, float><<<blocks, 256, 0, stream>>>((float*)out, (const float*)gu, F, ld_gu, n);
-    else if (dtype == XR_BF16) k_silu_mul<bf16_t, bf16_t><<<blocks, 256, 0, stream>>>((bf16_t*)out, (const bf16_t*)gu, F, ld_gu, n);
-    else { xr_set_error("silu_mul: bad dtype %d", dtype); return XR_BAD_ARG; }
-    XR_CHECK_LAUNCH("silu_mul");
+    if (dtype == XR_F32) k_gate_mul<float, float><<<blocks, 256, 0, stream>>>((float*)out, (const float*)gu, F, ld_gu, n, act);
+    else if (dtype == XR_BF16) k_gate_mul<bf16_t, bf16_t><<<blocks, 256, 0, stream>>>((bf16_t*)out, (const bf16_t*)gu, F, ld_gu, n, act);
+    else { xr_set_error("gate_mul: bad dtype %d", dtype); return XR_BAD_ARG; }
+    XR_CHECK_LAUNCH("gate_mul");
     return XR_OK;
 }
 

@@ -75,6 +75,24 @@ __host__ __device__ inline uint32_t pack_bf16x2(float lo, float hi) {
 }
 #endif
 
+// Activations of a gated feed-forward, act(gate) * up, by the code the Python side passes.
+// Another activation is another code and another case below; every kernel that applies the
+// gate (the products' epilogues and k_gate_mul) takes the code as an argument.
+#define XR_ACT_SILU 0
+#define XR_ACT_COUNT 1
+#if defined(__HIP_DEVICE_COMPILE__)
+// FAST: with the hardware's 2^x and reciprocal (1 ulp each)
+template <bool FAST> __device__ inline float gate_act(int act, float g) {
+    switch (act) {
+    default:    // XR_ACT_SILU: g / (1 + exp(-g)) (/root/reference/src/model.c:4451-4452)
+        return FAST ? g * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(g * -1.44269504f))
+                    : g / (1.0f + expf(-g));
+    }
+}
+#else
+template <bool FAST> __host__ __device__ inline float gate_act(int, float g) { return g; }   // the host pass only parses the callers
+#endif
+
 template <typename T> __device__ inline float ld(const T* p, size_t i);
 template <> __device__ inline float ld<float>(const float* p, size_t i) { return p[i]; }
 template <> __device__ inline float ld<bf16_t>(const bf16_t* p, size_t i) { return bf16_to_f32(p[i]); }

@@ -33,7 +33,7 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 
 #define EPI_STORE 0
 #define EPI_ACCUM 1
-#define EPI_SWIGLU 2
+#define EPI_GATED 2     // w = [gate rows; up rows]: act(gate) * up, act = GemmArgs.act
 
 // Rotation and cache write in the epilogue of the skinny kernel (on: q_out not null).  The
 // product's columns are [query heads | key heads | value heads], each head D wide; what would
@@ -64,6 +64,7 @@ struct GemmArgs {
     int M, N, K, lda, ldo;
     int out_bf16;      // storage of out
     int epi;
+    int act;           // the gate's activation (XR_ACT_*), with EPI_GATED
     int m_fast;        // tile order of the asynchronous kernel: 1 = consecutive workgroups share a weight tile
     int splits;        // > 1: K is cut into this many ranges, each workgroup writes raw sums to `partial`
     int k_per_split;   // columns per range (a multiple of 64)
@@ -132,13 +133,6 @@ __device__ inline bf16x8 as_bf16x8(uint4 v) {
 __device__ inline uint4 keep_if(bool ok, uint4 v) {
     return make_uint4(ok ? v.x : 0u, ok ? v.y : 0u, ok ? v.z : 0u, ok ? v.w : 0u);
 }
-__device__ inline float silu_f(float g) { return g / (1.0f + expf(-g)); }
-// the same with the hardware's 2^x and reciprocal (1 ulp each), for the tile kernel, where a lane
-// has 64 of them to do while nothing else runs on its compute unit
-__device__ inline float silu_fast(float g) {
-    return g * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(g * -1.44269504f));
-}
-
 __device__ inline void store_out(const GemmArgs& g, int m, int n, float v) {
     size_t o = (size_t)m * g.ldo + n;
     if (g.epi == EPI_ACCUM) {
@@ -329,7 +323,7 @@ __device__ inline void rope_tiles(float* stage, const f32x16 (&t)[NT], const Rop
 // of one output column meet in the same lane and register.
 template <int BN, int WN>
 __device__ inline int w_row_of(int r, int bx, int N, int epi, int& out_col) {
-    if (epi != EPI_SWIGLU) {
+    if (epi != EPI_GATED) {
         out_col = bx * BN + r;
         return out_col;
     }
@@ -382,7 +376,7 @@ __global__ __launch_bounds__(64 * WARPS_M * WARPS_N) void k_gemm_tile_async(Gemm
     // in its L2 while the weight tile of the moment is fetched once from memory for all.
     const int tiles_m = (g.M + BM - 1) / BM;
     constexpr int BN_OUT_S = BN / 2;
-    const int bn_out = g.epi == EPI_SWIGLU ? BN_OUT_S : BN;
+    const int bn_out = g.epi == EPI_GATED ? BN_OUT_S : BN;
     const int tiles_n = (g.col1 - g.col0 + bn_out - 1) / bn_out;
     const int tile_ = (int)(blockIdx.x / g.splits), split_ = (int)(blockIdx.x % g.splits);
     const int bm_ = g.m_fast ? tile_ % tiles_m : tile_ / tiles_n;
@@ -390,7 +384,7 @@ __global__ __launch_bounds__(64 * WARPS_M * WARPS_N) void k_gemm_tile_async(Gemm
     const int k_begin = split_ * g.k_per_split;
     const int k_end = (k_begin + g.k_per_split) < g.K ? (k_begin + g.k_per_split) : g.K;
     const int m0 = bm_ * BM;
-    const int n_rows = g.epi == EPI_SWIGLU ? 2 * g.N : g.N;
+    const int n_rows = g.epi == EPI_GATED ? 2 * g.N : g.N;
     const bf16_t* zero_src = reinterpret_cast<const bf16_t*>(xr_zero_chunk);
 
     // The pieces this lane fetches for every stage: where each begins (or a block of zeros, for
@@ -556,9 +550,9 @@ __global__ __launch_bounds__(64 * WARPS_M * WARPS_N) void k_gemm_tile_async(Gemm
 
     if (g.splits > 1 || g.raw) {
         // raw sums of this K range, by weight row: the epilogue belongs to k_gemm_finish
-        const int ldp = g.epi == EPI_SWIGLU ? 2 * g.N : g.N;
+        const int ldp = g.epi == EPI_GATED ? 2 * g.N : g.N;
         float* part = g.partial + (size_t)split_ * g.M * ldp;
-        if (g.vec_out && g.epi != EPI_SWIGLU) {
+        if (g.vec_out && g.epi != EPI_GATED) {
 #pragma unroll
             for (int i = 0; i < TM; ++i)
 #pragma unroll
@@ -585,7 +579,7 @@ __global__ __launch_bounds__(64 * WARPS_M * WARPS_N) void k_gemm_tile_async(Gemm
             }
         return;
     }
-    if (g.epi == EPI_SWIGLU) {
+    if (g.epi == EPI_GATED) {
         if (g.vec_out) {
             constexpr int TO = TN / 2, NTO = TO % 2 == 0 && TO > 0 ? 2 : 1;     // output tiles of a wave's row, and how many go together
 #pragma unroll
@@ -603,7 +597,7 @@ __global__ __launch_bounds__(64 * WARPS_M * WARPS_N) void k_gemm_tile_async(Gemm
                         const float bg = g.bias && in ? g.bias[oc] : 0.f, bu = g.bias && in ? g.bias[g.N + oc] : 0.f;
 #pragma unroll
                         for (int e = 0; e < 16; ++e)
-                            t[n][e] = silu_fast(acc[i][(jo + n) * 2][e] + bg) * (acc[i][(jo + n) * 2 + 1][e] + bu);
+                            t[n][e] = gate_act<true>(g.act, acc[i][(jo + n) * 2][e] + bg) * (acc[i][(jo + n) * 2 + 1][e] + bu);
                     }
                     write_tiles<NTO>(stage, t, g.out, g.ldo, g.out_bf16 ? 2 : 0, m0 + wm0 + i * 32, g.M, oc0, g.N, lane);
                 }
@@ -620,7 +614,7 @@ __global__ __launch_bounds__(64 * WARPS_M * WARPS_N) void k_gemm_tile_async(Gemm
 #pragma unroll
                 for (int e = 0; e < 16; ++e) {
                     int m = m0 + wm0 + i * 32 + (e / 4) * 8 + lg * 4 + (e % 4);
-                    if (m < g.M) store_out(g, m, oc, silu_fast(acc[i][j][e] + bg) * (acc[i][j + 1][e] + bu));
+                    if (m < g.M) store_out(g, m, oc, gate_act<true>(g.act, acc[i][j][e] + bg) * (acc[i][j + 1][e] + bu));
                 }
             }
         return;
@@ -664,7 +658,7 @@ __global__ __launch_bounds__(64 * WARPS_M * WARPS_N) void k_gemm_tile_async(Gemm
 
 // Sums the K ranges of a split product in a fixed order and applies the epilogue.
 __global__ __launch_bounds__(256) void k_gemm_finish(GemmArgs g) {
-    const int ldp = g.epi == EPI_SWIGLU ? 2 * g.N : g.N;
+    const int ldp = g.epi == EPI_GATED ? 2 * g.N : g.N;
     const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
     const bool ok = idx < (size_t)g.M * g.N;
     if (!ok && !g.rope.q_out) return;
@@ -678,10 +672,10 @@ __global__ __launch_bounds__(256) void k_gemm_finish(GemmArgs g) {
         const float val = v + (g.bias ? g.bias[n] : 0.f);
         const float partner = __shfl_xor(val, g.rope.interleaved ? 1 : 8);
         if (ok) rope_store(g.rope, m, n, val, partner);
-    } else if (g.epi == EPI_SWIGLU) {
+    } else if (g.epi == EPI_GATED) {
         for (int s = 0; s < g.splits; ++s) u += p[s * step + g.N];
         const float bg = g.bias ? g.bias[n] : 0.f, bu = g.bias ? g.bias[g.N + n] : 0.f;
-        store_out(g, m, n, silu_f(v + bg) * (u + bu));
+        store_out(g, m, n, gate_act<false>(g.act, v + bg) * (u + bu));
     } else {
         store_out(g, m, n, v + (g.bias ? g.bias[n] : 0.f));
     }
@@ -737,7 +731,7 @@ __global__ __launch_bounds__(1024) void k_gemm_finish_norm(GemmArgs g) {
 
 template <int BM, int BN, int WM_, int WN_, int ST, bool PIPE = false>
 static int launch_tile_async(GemmArgs g, hipStream_t stream) {
-    if (g.epi == EPI_SWIGLU && (BN / WN_ / 32) % 2) {
+    if (g.epi == EPI_GATED && (BN / WN_ / 32) % 2) {
         xr_set_error("gemm: a %dx%d tile cannot pair gate and up columns", BM, BN);
         return XR_BAD_ARG;
     }
@@ -753,7 +747,7 @@ static int launch_tile_async(GemmArgs g, hipStream_t stream) {
         }
         attr_set = true;
     }
-    int n_out_tile = g.epi == EPI_SWIGLU ? BN / 2 : BN;
+    int n_out_tile = g.epi == EPI_GATED ? BN / 2 : BN;
     if (g.col1 <= 0 || g.col1 > g.N) g.col1 = g.N;
     if (g.col0 < 0 || g.col0 % n_out_tile || g.col0 >= g.col1 || (g.col1 < g.N && g.col1 % n_out_tile)) {
         xr_set_error("gemm: columns %d..%d do not start at a %d-column tile", g.col0, g.col1, n_out_tile);
@@ -776,7 +770,7 @@ static int launch_tile_async(GemmArgs g, hipStream_t stream) {
     {
         // 4 columns a lane: every row of the output (and of the raw sums) must begin 16 bytes aligned
         const bool raw_out = g.splits > 1 || g.raw;
-        const int ld = raw_out ? (g.epi == EPI_SWIGLU ? 2 * g.N : g.N) : g.ldo;
+        const int ld = raw_out ? (g.epi == EPI_GATED ? 2 * g.N : g.N) : g.ldo;
         const void* base = raw_out ? (const void*)g.partial : (const void*)g.out;
         g.vec_out = g.N % 4 == 0 && ld % 4 == 0 && ((uintptr_t)base % 16) == 0 && (!raw_out || ((size_t)g.M * ld) % 4 == 0);
     }
@@ -951,7 +945,7 @@ __global__ __launch_bounds__(64 * KSW) void k_gemm_skinny(GemmArgs g) {
         if (SWIGLU) {
             if (ok) {
                 float bg = g.bias ? g.bias[nn] : 0.f, bu = g.bias ? g.bias[g.N + nn] : 0.f;
-                store_out(g, tok, nn, silu_f(v[0] + bg) * (v[NWT - 1] + bu));
+                store_out(g, tok, nn, gate_act<false>(g.act, v[0] + bg) * (v[NWT - 1] + bu));
             }
         } else if (g.rope.q_out) {
             // rotated and cached (the partner of a pair is 8 lanes away, or 1)
@@ -986,17 +980,6 @@ static int launch_tile_variant(int variant, const GemmArgs& g, hipStream_t strea
     if (variant == 14) return launch_tile_async<256, 256, 4, 2, 2, true>(g, stream);
     if (variant == 17) return launch_tile_async<128, 128, 2, 2, 2, true>(g, stream);
     if (variant == 26) return launch_tile_async<256, 192, 4, 2, 2>(g, stream);
-#ifdef XR_GEMM_SWEEP
-    if (variant == 10) return launch_tile_async<128, 128, 2, 2, 3>(g, stream);
-    if (variant == 13) return launch_tile_async<256, 256, 2, 4, 2>(g, stream);
-    if (variant == 16) return launch_tile_async<128, 256, 2, 4, 3>(g, stream);
-    if (variant == 18) return launch_tile_async<256, 256, 2, 2, 2>(g, stream);
-    if (variant == 42) return launch_tile_async<256, 128, 4, 2, 3>(g, stream);
-    if (variant == 44) return launch_tile_async<256, 256, 4, 2, 2>(g, stream);
-    if (variant == 47) return launch_tile_async<128, 128, 2, 2, 2>(g, stream);
-    if (variant == 53) return launch_tile_async<256, 192, 4, 2, 2, true>(g, stream);
-    if (variant == 55) return launch_tile_async<64, 128, 2, 2, 3, true>(g, stream);
-#endif
     xr_set_error("gemm: unknown variant %d", variant);
     return XR_BAD_ARG;
 }
@@ -1052,26 +1035,27 @@ extern "C" int xr_pack_weight(void* dst, const void* src, int N, int K, hipStrea
     return XR_OK;
 }
 
-// epi: 0 store, 1 add into float out, 2 SwiGLU (w has 2N rows: gate rows then up rows).
+// epi: 0 store, 1 add into float out, 2 gated (w has 2N rows: gate rows then up rows; act: XR_ACT_*).
 // variant: 0 = choose by shape; 1 = skinny; 10..20 = tile shapes; 30, 31 = few rows with K split;
 //          +1000 = row tiles of one weight tile follow each other.
 // w_packed: the weights are in k_pack_weight's order.
 // workspace (may be null): room for split products, workspace_bytes long; without it K is not split.
 extern "C" int xr_gemm_bf16(void* out, const void* a, const void* w, const float* bias, int M, int N, int K,
-                            int lda, int ldo, int out_dtype, int epi, int variant, int w_packed, float* workspace,
+                            int lda, int ldo, int out_dtype, int epi, int act, int variant, int w_packed, float* workspace,
                             size_t workspace_bytes, XrGemmNorm* norm, const XrGemmRope* rope, hipStream_t stream) {
     XR_REQUIRE(M >= 0 && N > 0 && K > 0, "gemm: bad sizes M=%d N=%d K=%d", M, N, K);
     XR_REQUIRE(lda >= K && ldo >= N, "gemm: row strides lda=%d ldo=%d are shorter than K=%d N=%d", lda, ldo, K, N);
     XR_REQUIRE(K % 8 == 0 && lda % 8 == 0, "gemm: the MFMA kernels need K (%d) and the row stride (%d) to be multiples of 8", K, lda);
     XR_REQUIRE(((uintptr_t)a % 16) == 0 && ((uintptr_t)w % 16) == 0, "gemm: operands must be 16-byte aligned");
     XR_REQUIRE(epi >= 0 && epi <= 2, "gemm: unknown epilogue %d", epi);
-    XR_REQUIRE(!(w_packed && epi == EPI_SWIGLU && N % 16), "gemm: packed gate and up rows need a width that is a multiple of 16, got %d", N);
+    XR_REQUIRE(epi != EPI_GATED || (act >= 0 && act < XR_ACT_COUNT), "gemm: unknown activation code %d", act);
+    XR_REQUIRE(!(w_packed && epi == EPI_GATED && N % 16), "gemm: packed gate and up rows need a width that is a multiple of 16, got %d", N);
     XR_REQUIRE(epi != EPI_ACCUM || out_dtype == XR_F32, "gemm: accumulation needs a 32-bit output");
     XR_REQUIRE(out_dtype == XR_F32 || out_dtype == XR_BF16, "gemm: bad output dtype %d", out_dtype);
     if (M == 0) return XR_OK;
     GemmArgs g;
     g.a = (const bf16_t*)a; g.w = (const bf16_t*)w; g.w_packed = w_packed ? 1 : 0; g.bias = bias; g.out = out;
-    g.M = M; g.N = N; g.K = K; g.lda = lda; g.ldo = ldo; g.out_bf16 = out_dtype == XR_BF16; g.epi = epi;
+    g.M = M; g.N = N; g.K = K; g.lda = lda; g.ldo = ldo; g.out_bf16 = out_dtype == XR_BF16; g.epi = epi; g.act = act;
     g.m_fast = 0; g.splits = 1; g.k_per_split = 0; g.partial = workspace; g.col0 = 0; g.col1 = N;
     g.raw = 0; g.norm_whole = 0; g.vec_out = 0;
     bool want_whole_norm = false;      // a norm after a product of more than 16 rows is asked for and possible
@@ -1144,8 +1128,8 @@ extern "C" int xr_gemm_bf16(void* out, const void* a, const void* w, const float
         }
     }
     if (variant >= 1000) { g.m_fast = 1; variant -= 1000; }
-    const bool sw = epi == EPI_SWIGLU;
-    const int w_rows = epi == EPI_SWIGLU ? 2 * N : N;
+    const bool sw = epi == EPI_GATED;
+    const int w_rows = epi == EPI_GATED ? 2 * N : N;
     // K ranges so that the workgroups make one round on the 256 compute units and no more
     // (measured at 32 and 64 rows: 10 ranges of 32 tiles, two rounds, took 20 us where 8 take 16),
     // if the workspace has room for their sums
@@ -1244,20 +1228,6 @@ extern "C" int xr_gemm_bf16(void* out, const void* a, const void* w, const float
         if (M <= 32) return rc_of(sw ? launch_skinny<2, 1, 16, 8, true>(g, stream) : launch_skinny<2, 1, 16, 8, false>(g, stream));
         return rc_of(sw ? launch_skinny<4, 2, 8, 4, true>(g, stream) : launch_skinny<4, 2, 8, 4, false>(g, stream));
     }
-#ifdef XR_GEMM_SWEEP
-#define SK(id, MT, RT, KSW, U, NT) if (variant == id) return rc_of(sw ? launch_skinny<MT, RT, KSW, U, true, NT>(g, stream) : launch_skinny<MT, RT, KSW, U, false, NT>(g, stream));
-    SK(100, 1, 1, 16, 8, false) SK(101, 1, 1, 8, 8, false) SK(102, 1, 1, 8, 16, false) SK(103, 1, 1, 4, 16, false)
-    SK(104, 1, 1, 4, 8, false) SK(105, 1, 2, 8, 8, false) SK(106, 1, 2, 4, 8, false) SK(107, 1, 1, 16, 4, false)
-    SK(108, 1, 1, 16, 8, true) SK(109, 1, 1, 8, 8, true) SK(110, 1, 1, 8, 16, true) SK(111, 1, 2, 8, 8, true)
-    SK(112, 1, 2, 16, 4, false) SK(113, 1, 4, 4, 4, false) SK(114, 1, 1, 2, 16, false) SK(115, 1, 2, 4, 8, true)
-    SK(140, 4, 2, 8, 4, false) SK(141, 4, 1, 8, 4, false) SK(142, 4, 1, 16, 4, false) SK(143, 4, 2, 4, 4, false)
-    SK(144, 4, 4, 4, 2, false) SK(145, 4, 2, 8, 4, true) SK(146, 4, 1, 8, 8, false) SK(147, 4, 2, 8, 2, false)
-    SK(148, 4, 4, 4, 4, false) SK(149, 4, 4, 8, 2, false)
-    SK(116, 1, 1, 4, 32, false) SK(117, 1, 1, 8, 4, false) SK(118, 1, 2, 8, 4, false) SK(119, 1, 2, 4, 16, false)
-    SK(120, 1, 1, 2, 32, false) SK(121, 1, 4, 4, 8, false) SK(122, 1, 2, 2, 16, false) SK(123, 1, 1, 16, 16, false)
-    SK(124, 1, 4, 8, 4, false) SK(125, 1, 2, 16, 8, false) SK(126, 1, 4, 2, 8, false)
-#undef SK
-#endif
     if (variant == 30 || variant == 31) {       // few rows: 32 or 64 of them against 128 weight rows, K split
         const int bn_out = sw ? 64 : 128;
         g.splits = pick_splits((N + bn_out - 1) / bn_out);

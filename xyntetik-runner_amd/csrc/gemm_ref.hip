@@ -3,11 +3,17 @@
 // Weights are [n_out][n_in] row-major as the reference keeps them
 // (/root/reference/src/model.c:193-205); each output is a sum over k in ascending
 // order, whatever the batch, so a row's result does not depend on its neighbours.
+// The sum has two levels: runs of RBK * RB_FOLD = 128 columns are summed by FMA, and the runs'
+// sums are added up with a compensated (Kahan) sum.  One running 32-bit sum over the 14,336
+// columns of a wide feed-forward loses about 1e-5 of the result to rounding, which at such
+// widths is as much as a real fault may be; summed this way a product is about ten times closer
+// to the exact one, so the 32-bit path can be held to the tolerance that small models are.
 #include "common.h"
 
 #define RBM 64
 #define RBN 64
 #define RBK 16
+#define RB_FOLD 8
 
 template <typename TI, typename TO, bool ACC>
 __global__ __launch_bounds__(256) void k_gemm_ref(TO* __restrict__ out, const TI* __restrict__ a,
@@ -17,13 +23,23 @@ __global__ __launch_bounds__(256) void k_gemm_ref(TO* __restrict__ out, const TI
     __shared__ float Ws[RBK][RBN + 4];
     int m0 = blockIdx.y * RBM, n0 = blockIdx.x * RBN;
     int tx = threadIdx.x & 15, ty = threadIdx.x >> 4;
-    float acc[4][4];
+    float acc[4][4], tot[4][4], lost[4][4];      // the run's sum, the sum of the runs, what that sum has lost
 #pragma unroll
     for (int i = 0; i < 4; ++i)
 #pragma unroll
-        for (int j = 0; j < 4; ++j) acc[i][j] = 0.f;
+        for (int j = 0; j < 4; ++j) acc[i][j] = tot[i][j] = lost[i][j] = 0.f;
+#define FOLD_RUN()                                                   \
+    _Pragma("unroll") for (int i = 0; i < 4; ++i)                    \
+        _Pragma("unroll") for (int j = 0; j < 4; ++j) {              \
+            const float y = acc[i][j] - lost[i][j];                  \
+            const float t = tot[i][j] + y;                           \
+            lost[i][j] = (t - tot[i][j]) - y;                        \
+            tot[i][j] = t;                                           \
+            acc[i][j] = 0.f;                                         \
+        }
 
-    for (int k0 = 0; k0 < K; k0 += RBK) {
+    int slice = 0;
+    for (int k0 = 0; k0 < K; k0 += RBK, ++slice) {
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
             int idx = threadIdx.x + e * 256;
@@ -46,7 +62,10 @@ __global__ __launch_bounds__(256) void k_gemm_ref(TO* __restrict__ out, const TI
                 for (int j = 0; j < 4; ++j) acc[i][j] = fmaf(av[i], wv[j], acc[i][j]);
         }
         __syncthreads();
+        if (slice % RB_FOLD == RB_FOLD - 1) { FOLD_RUN() }
     }
+    FOLD_RUN()
+#undef FOLD_RUN
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
         int gm = m0 + ty * 4 + i;
@@ -55,7 +74,7 @@ __global__ __launch_bounds__(256) void k_gemm_ref(TO* __restrict__ out, const TI
         for (int j = 0; j < 4; ++j) {
             int gn = n0 + tx * 4 + j;
             if (gn >= N) continue;
-            float v = acc[i][j];
+            float v = tot[i][j];
             if (bias) v += bias[gn];
             size_t o = (size_t)gm * ldo + gn;
             if (ACC) v += ld<TO>(out, o);

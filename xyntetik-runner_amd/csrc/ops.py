@@ -18,10 +18,19 @@ from . import build as _build
 
 XR_F32, XR_BF16 = 0, 1
 _CODE = {torch.float32: XR_F32, torch.bfloat16: XR_BF16}
+# activations of a gated feed-forward, by the code the kernels know them under (XR_ACT_* of common.h)
+GATE_ACTIVATIONS = {"silu": 0}
 
 
 class KernelError(RuntimeError):
     pass
+
+
+def activation_code(name: str) -> int:
+    try:
+        return GATE_ACTIVATIONS[name]
+    except KeyError:
+        raise KernelError(f"gate activation {name!r} is not built into the kernels (known: {sorted(GATE_ACTIVATIONS)})") from None
 
 
 def dtype_code(dt: torch.dtype) -> int:
@@ -34,15 +43,15 @@ def dtype_code(dt: torch.dtype) -> int:
 _p, _i, _f, _sz, _u32 = C.c_void_p, C.c_int, C.c_float, C.c_size_t, C.c_uint32
 
 _PROTOS = {
-    "xr_embedding": [_p, _p, _p, _i, _i, _i, _f, _i, _p],
+    "xr_embedding": [_p, _p, _p, _i, _i, _i, _f, _i, _i, _p],
     "xr_rmsnorm": [_p, _p, _p, _p, _i, _i, _i, _f, _i, _i, _p],
     "xr_rope_kv_write": [_p, _p, _p, _i, _p, _p, _p, _p, _p, _p, _i, _p, _i, _i, _i, _i, _i, _i, _f, _i, _i, _i, _p],
-    "xr_silu_mul": [_p, _p, _i, _i, _i, _i, _p],
+    "xr_gate_mul": [_p, _p, _i, _i, _i, _i, _i, _p],
     "xr_add": [_p, _p, _sz, _i, _p],
     "xr_fill_rows": [_p, _p, _i, _sz, _u32, _p],
     "xr_convert": [_p, _p, _sz, _i, _i, _p],
     "xr_gemm_ref": [_p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _p],
-    "xr_gemm_bf16": [_p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _i, _p, _sz, _p, _p, _p],
+    "xr_gemm_bf16": [_p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _p, _sz, _p, _p, _p],
     "xr_pack_weight": [_p, _p, _i, _i, _p],
     "xr_attention_ref": [_p, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _f, _i, _i, _p],
     "xr_sample": [_p, _p, _i, _i, _i, _p, _p, _p, _p, _p, _p, _p, _p, _i, _p, _i, _p, _p],
@@ -61,7 +70,7 @@ class PackedWeight:
     """A bfloat16 weight matrix ``[rows, cols]`` in the order the MFMA kernels read it: blocks of
     16 rows x 32 columns, 1 KB each (``data[row group, column block, row, column]``), rows and
     columns padded with zeros.  Made by
-    ``Ops.pack_weight``; ``Ops.linear`` and ``Ops.linear_swiglu`` take it in place of the matrix."""
+    ``Ops.pack_weight``; ``Ops.linear`` and ``Ops.linear_gated`` take it in place of the matrix."""
 
     def __init__(self, data: torch.Tensor, rows: int, cols: int):
         self.data, self.rows, self.cols = data, rows, cols
@@ -85,7 +94,7 @@ class UnscaledRows:
     row (row t's sum is ``sumsq[:, t].sum()``), so the norm's row t is
     ``data[t] * rsqrt(sumsq[:, t].sum() / E + eps)``.  As that factor is one number a row, a
     product ``rows @ w^T`` may apply it to its result instead: ``Ops.linear`` and
-    ``Ops.linear_swiglu`` take this in place of the rows.  Made by ``Ops.linear_add_rmsnorm``."""
+    ``Ops.linear_gated`` take this in place of the rows.  Made by ``Ops.linear_add_rmsnorm``."""
 
     MAX_ROWS = 16
 
@@ -172,14 +181,16 @@ class Ops:
             raise KernelError(f"{what} must be contiguous")
 
     # -- element-wise and row-wise ----------------------------------------------
-    def embedding(self, table: torch.Tensor, ids: torch.Tensor, scale: float = 1.0) -> torch.Tensor:
-        """``out[t] = table[ids[t]] * scale`` as 32-bit rows."""
-        self._dev(table, ids)
-        self._contig(table, "embedding table")
+    def embedding(self, table, ids: torch.Tensor, scale: float = 1.0) -> torch.Tensor:
+        """``out[t] = table[ids[t]] * scale`` as 32-bit rows; ``table`` is a matrix or a ``PackedWeight``."""
+        packed = isinstance(table, PackedWeight)
+        data = table.data if packed else table
+        self._dev(data, ids)
+        self._contig(data, "embedding table")
         T, (V, E) = ids.numel(), table.shape
-        out = torch.empty((T, E), dtype=torch.float32, device=table.device)
-        self.lib.check(self.lib.xr_embedding(out.data_ptr(), table.data_ptr(), ids.data_ptr(), T, E, V,
-                                             float(scale), dtype_code(table.dtype), _stream()))
+        out = torch.empty((T, E), dtype=torch.float32, device=data.device)
+        self.lib.check(self.lib.xr_embedding(out.data_ptr(), data.data_ptr(), ids.data_ptr(), T, E, V,
+                                             float(scale), dtype_code(data.dtype), 1 if packed else 0, _stream()))
         return out
 
     def rmsnorm(self, x: torch.Tensor, w: Optional[torch.Tensor], eps: float, out_dtype: torch.dtype,
@@ -198,17 +209,21 @@ class Ops:
                                            dtype_code(w.dtype) if w is not None else XR_F32, _stream()))
         return out
 
-    def silu_mul(self, gu: torch.Tensor) -> torch.Tensor:
-        """``silu(gu[:, :F]) * gu[:, F:]``."""
+    def gate_mul(self, gu: torch.Tensor, activation: str = "silu") -> torch.Tensor:
+        """``act(gu[:, :F]) * gu[:, F:]``."""
         self._dev(gu)
         T, F2 = gu.shape
         F = F2 // 2
         if gu.stride(1) != 1 or F2 % 2:
-            raise KernelError("silu_mul input must be [rows, 2F] with unit column stride")
+            raise KernelError("gate_mul input must be [rows, 2F] with unit column stride")
         out = torch.empty((T, F), dtype=gu.dtype, device=gu.device)
-        self.lib.check(self.lib.xr_silu_mul(out.data_ptr(), gu.data_ptr(), T, F, gu.stride(0),
-                                            dtype_code(gu.dtype), _stream()))
+        self.lib.check(self.lib.xr_gate_mul(out.data_ptr(), gu.data_ptr(), T, F, gu.stride(0),
+                                            dtype_code(gu.dtype), activation_code(activation), _stream()))
         return out
+
+    def silu_mul(self, gu: torch.Tensor) -> torch.Tensor:
+        """``silu(gu[:, :F]) * gu[:, F:]``."""
+        return self.gate_mul(gu, "silu")
 
     def add_(self, x: torch.Tensor, y: torch.Tensor) -> None:
         """``x += y`` with 32-bit ``x``."""
@@ -256,7 +271,7 @@ class Ops:
                 and a.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0)
 
     def pack_weight(self, w: torch.Tensor, gated: bool = False):
-        """``w`` for use as the weight of ``linear`` (``gated``: of ``linear_swiglu``): packed for
+        """``w`` for use as the weight of ``linear`` (``gated``: of ``linear_gated``): packed for
         the MFMA kernels where they will serve it (bfloat16, a width that is a multiple of 8, for
         gate and up rows a height that is a multiple of 32), else ``w`` itself."""
         if not (self.use_mfma and w.dtype == torch.bfloat16 and w.dim() == 2 and w.shape[1] % 8 == 0):
@@ -303,7 +318,7 @@ class Ops:
         if self._mfma_ok(a, wt):
             self.lib.check(self.lib.xr_gemm_bf16(out.data_ptr(), a.data_ptr(), wt.data_ptr(), _ptr(bias), M, N, K,
                                                  a.stride(0), out.stride(0), dtype_code(out.dtype),
-                                                 1 if accumulate else 0, variant, 1 if packed else 0,
+                                                 1 if accumulate else 0, 0, variant, 1 if packed else 0,
                                                  *self._gemm_workspace(a.device),
                                                  C.addressof(norm) if norm is not None else None, None, _stream()))
             return out
@@ -333,7 +348,7 @@ class Ops:
         """``residual += a @ w^T (+ bias)``, then the RMSNorm of the updated rows.
 
         With ``defer`` the caller says that what reads the result is a ``linear`` or
-        ``linear_swiglu``: for at most 16 bfloat16 rows the product's kernel then also writes the
+        ``linear_gated``: for at most 16 bfloat16 rows the product's kernel then also writes the
         weighted rows and their partial sums of squares, and an ``UnscaledRows`` comes back, whose
         scale the next product applies.  From 17 to 64 rows the kernel that adds up the product's K
         ranges takes whole rows and writes the finished norm.  In every other case the norm's own
@@ -367,35 +382,41 @@ class Ops:
         self.linear(a, w, bias=bias, out=residual, accumulate=True)
         return self.rmsnorm(residual, norm_weight, eps, out_dtype)
 
-    def linear_swiglu(self, a: torch.Tensor, w, bias: Optional[torch.Tensor] = None,
-                      variant: int = 0) -> torch.Tensor:
-        """``silu(a @ w[:F]^T) * (a @ w[F:]^T)`` for ``w [2F, K]`` = gate rows then up rows
-        (a matrix, or a ``PackedWeight`` made with ``gated=True``)."""
+    def linear_gated(self, a: torch.Tensor, w, bias: Optional[torch.Tensor] = None, activation: str = "silu",
+                     variant: int = 0) -> torch.Tensor:
+        """``act(a @ w[:F]^T) * (a @ w[F:]^T)`` for ``w [2F, K]`` = gate rows then up rows
+        (a matrix, or a ``PackedWeight`` made with ``gated=True``); ``activation`` is one of
+        ``GATE_ACTIVATIONS``."""
+        act = activation_code(activation)
         packed = isinstance(w, PackedWeight)
         wt = w.data if packed else w
         norm, a = self._norm_before(a, None)
         F = w.shape[0] // 2
         if w.shape[0] % 2:
-            raise KernelError("linear_swiglu: the weight must have an even number of rows")
+            raise KernelError("linear_gated: the weight must have an even number of rows")
         if self._mfma_ok(a, wt):
             self._dev(a, wt, bias)
-            self._contig(wt, "linear_swiglu weight")
+            self._contig(wt, "linear_gated weight")
             M, K = a.shape
             if K != w.shape[1] or a.stride(1) != 1:
-                raise KernelError(f"linear_swiglu: shapes {tuple(a.shape)} x {tuple(w.shape)}^T do not fit")
+                raise KernelError(f"linear_gated: shapes {tuple(a.shape)} x {tuple(w.shape)}^T do not fit")
             if bias is not None and (bias.dtype != torch.float32 or bias.numel() != 2 * F):
-                raise KernelError("linear_swiglu: bias must be float32 [2F]")
+                raise KernelError("linear_gated: bias must be float32 [2F]")
             out = torch.empty((M, F), dtype=a.dtype, device=a.device)
             self.lib.check(self.lib.xr_gemm_bf16(out.data_ptr(), a.data_ptr(), wt.data_ptr(), _ptr(bias), M, F, K,
-                                                 a.stride(0), F, dtype_code(out.dtype), 2, variant,
+                                                 a.stride(0), F, dtype_code(out.dtype), 2, act, variant,
                                                  1 if packed else 0, *self._gemm_workspace(a.device),
                                                  C.addressof(norm) if norm is not None else None, None, _stream()))
             return out
         if norm is not None:
-            raise KernelError("linear_swiglu: rows that still lack their norm's scale need the MFMA kernels")
+            raise KernelError("linear_gated: rows that still lack their norm's scale need the MFMA kernels")
         if packed:
-            raise KernelError("linear_swiglu: a packed weight needs bfloat16 rows that are 16-byte aligned")
-        return self.silu_mul(self.linear(a, w, bias=bias))
+            raise KernelError("linear_gated: a packed weight needs bfloat16 rows that are 16-byte aligned")
+        return self.gate_mul(self.linear(a, w, bias=bias), activation)
+
+    def linear_swiglu(self, a: torch.Tensor, w, bias: Optional[torch.Tensor] = None, variant: int = 0) -> torch.Tensor:
+        """``linear_gated`` with the SiLU gate."""
+        return self.linear_gated(a, w, bias=bias, activation="silu", variant=variant)
 
     # -- attention --------------------------------------------------------------
     def rope_kv_write(self, q_in, k_in, v_in, q_out, k_cache, v_cache, positions, req_of_token,
@@ -462,7 +483,7 @@ class Ops:
             rp.interleaved, rp.mscale, rp.page_size = 1 if interleaved else 0, float(mscale), page_size
             rp.q_out, rp.k_cache, rp.v_cache = q.data_ptr(), _ptr(k_cache) if Hk else None, _ptr(v_cache) if Hk else None
             self.lib.check(self.lib.xr_gemm_bf16(None, rows.data_ptr(), wt.data_ptr(), _ptr(bias), T, w.shape[0],
-                                                 rows.shape[1], rows.stride(0), w.shape[0], XR_F32, 0, 0,
+                                                 rows.shape[1], rows.stride(0), w.shape[0], XR_F32, 0, 0, 0,
                                                  1 if isinstance(w, PackedWeight) else 0,
                                                  *self._gemm_workspace(rows.device),
                                                  C.addressof(norm) if norm is not None else None,

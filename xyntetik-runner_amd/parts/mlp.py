@@ -1,4 +1,4 @@
-"""Gated feed-forward: ``down(act(gate(h)) * up(h))`` with act = SiLU
+"""Gated feed-forward: ``down(act(gate(h)) * up(h))``; act = SiLU is the one activation built
 (/root/reference/src/model.c:6399-6407, ``gated_act`` :4451-4452).
 
 ``gate`` and ``up`` are kept as one ``[2F, E]`` matrix so that one product makes both;
@@ -19,8 +19,11 @@ class GatedMLP(FeedForward):
 
     def __init__(self, hidden_size: int, intermediate_size: int, activation: str = "silu", bias: bool = False,
                  gate_name: str = "gate_proj", up_name: str = "up_proj", down_name: str = "down_proj"):
-        if activation != "silu":
-            raise ValueError(f"gated feed-forward: activation {activation!r} is not supported (silu)")
+        from ..csrc.ops import GATE_ACTIVATIONS
+        if activation not in GATE_ACTIVATIONS:
+            raise ValueError(f"gated feed-forward: activation {activation!r} is not built into the kernels "
+                             f"(known: {sorted(GATE_ACTIVATIONS)})")
+        self.activation = activation
         self.hidden_size, self.intermediate_size = int(hidden_size), int(intermediate_size)
         self.bias = bool(bias)
         self.names = (gate_name, up_name, down_name)
@@ -49,7 +52,7 @@ class GatedMLP(FeedForward):
             self.b_down = tensors[f"{d}.bias"].float().contiguous()
 
     def _hidden(self, ctx, h):
-        return self.rt.ops.linear_swiglu(h, self.w_gate_up, bias=self.b_gate_up)
+        return self.rt.ops.linear_gated(h, self.w_gate_up, bias=self.b_gate_up, activation=self.activation)
 
     def forward(self, ctx, h):
         return self.rt.ops.linear(self._hidden(ctx, h), self.w_down, bias=self.b_down)
