@@ -156,8 +156,12 @@ def measure_prefill(runner, cfg, T, repeats, seed):
         torch.cuda.synchronize()
         t0 = time.perf_counter()
         out = runner.step([StepEntry(("prefill", r), toks, [T - 1])])
-        out.cpu()
+        last = out.cpu()
         dt = time.perf_counter() - t0
+        # the reference's rule for a run that computed nothing: all-zero logits fail
+        # (/root/reference/tests/test_gpu_identity.c:190-201); so do logits that are not finite
+        if not bool(torch.isfinite(last).all()) or float(last.abs().max()) == 0.0 or float(last.std()) == 0.0:
+            raise RuntimeError("prefill: the logits of the prompt's last position are not finite, all zero or all equal")
         runner.finish(("prefill", r))
         if r > 0:
             best = dt if best is None else min(best, dt)

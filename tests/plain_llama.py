@@ -48,6 +48,52 @@ def load_folder(model_dir):
     return cfg, read_safetensors(os.path.join(model_dir, "model.safetensors"))
 
 
+class TensorsOnDemand:
+    """name -> float64 array like ``read_safetensors``, but every tensor is read from the file
+    and widened when it is asked for and kept nowhere: for a model whose widened weights
+    should not all stand in memory at once (one product's matrix at a time)."""
+
+    def __init__(self, path):
+        self.path = path
+        with open(path, "rb") as f:
+            (n,) = struct.unpack("<Q", f.read(8))
+            self.header = {k: v for k, v in json.loads(f.read(n).decode("utf-8")).items() if k != "__metadata__"}
+        self.base = 8 + n
+
+    def __contains__(self, name):
+        return name in self.header
+
+    def __iter__(self):
+        return iter(self.header)
+
+    def get(self, name, default=None):
+        return self[name] if name in self.header else default
+
+    def __getitem__(self, name):
+        info = self.header[name]
+        b, e = info["data_offsets"]
+        with open(self.path, "rb") as f:
+            f.seek(self.base + b)
+            raw = f.read(e - b)
+        dt = info["dtype"]
+        if dt == "BF16":
+            arr = (np.frombuffer(raw, dtype="<u2").astype(np.uint32) << 16).view(np.float32).astype(np.float64)
+        elif dt == "F32":
+            arr = np.frombuffer(raw, dtype="<f4").astype(np.float64)
+        elif dt == "F16":
+            arr = np.frombuffer(raw, dtype="<f2").astype(np.float64)
+        else:
+            raise ValueError(f"{name}: dtype {dt}")
+        return arr.reshape(info["shape"])
+
+
+def open_folder(model_dir):
+    """As ``load_folder`` with the tensors read on demand."""
+    with open(os.path.join(model_dir, "config.json")) as f:
+        cfg = json.load(f)
+    return cfg, TensorsOnDemand(os.path.join(model_dir, "model.safetensors"))
+
+
 # ----------------------------------------------------------------------------- parts
 def rmsnorm(x, w, eps):
     """y = x * (1/sqrt(mean(x^2) + eps)) * w: eps inside the root, added to the mean.
@@ -88,6 +134,14 @@ def rope_inv_freq(rot_dim, theta, scaling=None):
     return out
 
 
+def rope_angle(position, inv_freq_j):
+    """a = pos * inv_freq[j] the way the reference forms it: the table holds floats
+    (/root/reference/src/model.c:286-289) and ``float a = pos * fr[j]`` is a float product (:3520).
+    At position 2,048 that product differs from the exact one by up to 1.2e-4 rad for the fastest
+    pair, which belongs to the model as it is defined; cosine and sine are then taken exactly."""
+    return float(np.float32(position) * np.float32(inv_freq_j))
+
+
 def rope(x, positions, inv_freq, interleaved=False):
     """Rotate pair j of every head by a = pos * inv_freq[j]:
     (x0, x1) -> (x0 cos a - x1 sin a, x0 sin a + x1 cos a).  Un-permuted checkpoints pair
@@ -98,12 +152,24 @@ def rope(x, positions, inv_freq, interleaved=False):
     y = x.copy()
     for t in range(T):
         for j in range(half):
-            a = positions[t] * inv_freq[j]
+            a = rope_angle(positions[t], inv_freq[j])
             c, s = math.cos(a), math.sin(a)
             i0, i1 = (2 * j, 2 * j + 1) if interleaved else (j, j + half)
             x0, x1 = x[t, :, i0].copy(), x[t, :, i1].copy()
             y[t, :, i0] = x0 * c - x1 * s
             y[t, :, i1] = x0 * s + x1 * c
+    return y
+
+
+def rope_all_at_once(x, positions, inv_freq):
+    """``rope`` for pairs (j, j + rot/2) with whole arrays in place of its loops (for long sequences)."""
+    half = len(inv_freq)
+    a = (np.asarray(positions, dtype=np.float32)[:, None] * np.asarray(inv_freq, dtype=np.float32)[None, :]).astype(np.float64)
+    c, s = np.cos(a)[:, None, :], np.sin(a)[:, None, :]
+    y = x.copy()
+    x0, x1 = x[:, :, :half], x[:, :, half:2 * half]
+    y[:, :, :half] = x0 * c - x1 * s
+    y[:, :, half:2 * half] = x0 * s + x1 * c
     return y
 
 
@@ -133,6 +199,26 @@ def attention(q, k, v, scale, window=None):
     return out
 
 
+def attention_all_at_once(q, k, v, scale, window=None):
+    """``attention`` with one score matrix per head in place of its loops (for long sequences):
+    softmax over the keys a position may see of (q k^T) * scale, times v."""
+    T, H, D = q.shape
+    Hk = k.shape[1]
+    mul = H // Hk
+    pos = np.arange(T)
+    seen = pos[None, :] <= pos[:, None]
+    if window:
+        seen &= pos[None, :] > pos[:, None] - window
+    out = np.zeros((T, H, D))
+    for h in range(H):
+        kvh = h // mul
+        s = (q[:, h, :] @ k[:, kvh, :].T) * scale
+        s = np.where(seen, s, -np.inf)
+        e = np.exp(s - s.max(axis=1, keepdims=True))
+        out[:, h, :] = (e / e.sum(axis=1, keepdims=True)) @ v[:, kvh, :]
+    return out
+
+
 def silu(g):
     """g / (1 + exp(-g)).  /root/reference/src/model.c:4451-4452"""
     return g / (1.0 + np.exp(-g))
@@ -146,10 +232,14 @@ def mlp(h, wg, wu, wd, bg=None, bu=None, bd=None):
 
 
 # ----------------------------------------------------------------------------- the model
-def forward(cfg, w, tokens, return_hidden=False):
-    """Logits [T, V] of one whole sequence.  Order per layer: norm, q/k/v, rotation of q
-    and k, attention over positions <= own, output projection, add, norm, feed-forward,
-    add; then final norm and head.  /root/reference/src/model.c:6148-6483"""
+def forward(cfg, w, tokens, return_hidden=False, rows=None, all_at_once=False):
+    """Logits [T, V] of one whole sequence (of the positions ``rows`` only, if given).  Order
+    per layer: norm, q/k/v, rotation of q and k, attention over positions <= own, output
+    projection, add, norm, feed-forward, add; then final norm and head.
+    /root/reference/src/model.c:6148-6483.  ``all_at_once``: rotation and attention by their
+    whole-array forms (a long sequence would take the loops minutes)."""
+    rope_fn = rope_all_at_once if all_at_once else rope
+    attention_fn = attention_all_at_once if all_at_once else attention
     E = cfg["hidden_size"]
     H = cfg["num_attention_heads"]
     Hk = cfg.get("num_key_value_heads") or H
@@ -174,9 +264,9 @@ def forward(cfg, w, tokens, return_hidden=False):
             q = q + w[p + "self_attn.q_proj.bias"]
             k = k + w[p + "self_attn.k_proj.bias"]
             v = v + w[p + "self_attn.v_proj.bias"]
-        q = rope(q.reshape(T, H, D), pos, inv_freq)
-        k = rope(k.reshape(T, Hk, D), pos, inv_freq)
-        o = attention(q, k, v.reshape(T, Hk, D), scale).reshape(T, H * D)
+        q = rope_fn(q.reshape(T, H, D), pos, inv_freq)
+        k = rope_fn(k.reshape(T, Hk, D), pos, inv_freq)
+        o = attention_fn(q, k, v.reshape(T, Hk, D), scale).reshape(T, H * D)
         a = o @ w[p + "self_attn.o_proj.weight"].T
         if cfg.get("attention_bias"):
             a = a + w[p + "self_attn.o_proj.bias"]
@@ -188,6 +278,8 @@ def forward(cfg, w, tokens, return_hidden=False):
                     w.get(p + "mlp.down_proj.bias") if mb else None)   # /root/reference/src/model.c:6421-6423
     if return_hidden:
         return x
+    if rows is not None:
+        x = x[list(rows)]
     h = rmsnorm(x, w["model.norm.weight"], eps)      # /root/reference/src/model.c:6479
     head = w["model.embed_tokens.weight"] if cfg.get("tie_word_embeddings") else w["lm_head.weight"]
     return h @ head.T                                # /root/reference/src/model.c:6481, tied :2353-2366

@@ -42,7 +42,11 @@ def test_rope_identity_norm_composition_and_relative_positions():
     q, k = rng.normal(size=(1, 1, 8)), rng.normal(size=(1, 1, 8))
     d1 = np.dot(P.rope(q, [9], inv)[0, 0], P.rope(k, [4], inv)[0, 0])
     d2 = np.dot(P.rope(q, [105], inv)[0, 0], P.rope(k, [100], inv)[0, 0])
-    assert math.isclose(d1, d2, rel_tol=1e-9)                          # only the distance counts
+    # only the distance counts: as far as a float angle goes (the reference's `float a = pos * fr[j]`
+    # rounds position 105 times the frequency to 24 bits, about 4e-6 rad); a wrong pairing or
+    # sign changes the product by its own size
+    assert math.isclose(d1, d2, rel_tol=2e-6)
+    assert P.rope_angle(2048, np.float64(1) / 3) == float(np.float32(2048) * np.float32(1 / 3))
     d3 = np.dot(P.rope(q, [4], inv)[0, 0], P.rope(k, [9], inv)[0, 0])
     assert not math.isclose(d1, d3, rel_tol=1e-3)                      # and its sign matters
 
@@ -51,7 +55,7 @@ def test_rope_rotation_direction_and_pairing():
     # one pair, angle pi/2 at position 1: (1, 0) -> (0, 1); a wrong sign gives (0, -1)
     inv = np.array([math.pi / 2])
     x = np.array([[[1.0, 0.0]]])
-    assert np.allclose(P.rope(x, [1], inv)[0, 0], [0.0, 1.0], atol=1e-12)
+    assert np.allclose(P.rope(x, [1], inv)[0, 0], [0.0, 1.0], atol=1e-7)         # (the angle is a float: pi/2 to 24 bits)
     # half-split on un-permuted rows == adjacent pairs on rows permuted as [0, D/2, 1, D/2+1, ...]
     # (the converter's relation, /root/reference/src/model.c:1464-1466)
     D = 8
@@ -80,6 +84,59 @@ def test_llama3_scaling_bands():
     assert np.allclose(P.rope_inv_freq(32, 500000.0, dict(sc, factor=1.0)), base)   # factor 1 = identity
     assert np.allclose(P.rope_inv_freq(16, 1000.0, {"rope_type": "linear", "factor": 4.0}),
                        P.rope_inv_freq(16, 1000.0) / 4.0)
+
+
+def _plain_table(rot, theta, scaling=None):
+    return np.asarray(P.rope_inv_freq(rot, theta, scaling), dtype=np.float64)
+
+
+def _engine_table(rot, theta, scaling=None):
+    from xyntetik_runner_amd.parts.rotary import rotary_inv_freq
+    return rotary_inv_freq(rot, theta, scaling).numpy().astype(np.float64)
+
+
+@pytest.mark.parametrize("table", [_plain_table, _engine_table], ids=["plain", "engine"])
+def test_llama3_scaling_is_continuous_monotone_and_linear_in_frequency(table):
+    """What fixes the interpolation between the two bands beside its text
+    (hook: /root/reference/src/model.c:291-297, where the reference divides by the factors a file
+    brings): the scaled/unscaled ratio is 1 below wavelength orig/high and 1/factor above
+    orig/low, so a rule that joins them must meet both values at the band's edges, fall
+    monotonically between them, and, being linear in orig/wavelength, give the mean of the two
+    values where orig/wavelength is the mean of low and high.  Swapping the two weights of the
+    interpolation jumps by the factor at both edges; interpolating in wavelength instead of
+    frequency misses the midpoint."""
+    sc = {"rope_type": "llama3", "factor": 8.0, "low_freq_factor": 1.0, "high_freq_factor": 4.0,
+          "original_max_position_embeddings": 8192}
+    orig, low, high, factor = 8192.0, 1.0, 4.0, 8.0
+
+    def ratio(wavelength):
+        # a table of two entries whose second has exactly this wavelength: theta^(-1/2) = 2 pi / wavelength
+        theta = (wavelength / (2.0 * math.pi)) ** 2
+        return table(4, theta, sc)[1] / table(4, theta)[1]
+
+    for edge, value in ((orig / high, 1.0), (orig / low, 1.0 / factor)):
+        below, above = ratio(edge * (1 - 1e-9)), ratio(edge * (1 + 1e-9))
+        assert abs(below - value) < 1e-6 and abs(above - value) < 1e-6, (edge, below, above)
+    sweep = [ratio(w) for w in np.geomspace(orig / high / 2, orig / low * 2, 300)]
+    assert all(a >= b - 1e-12 for a, b in zip(sweep, sweep[1:])) and sweep[0] == 1.0 and abs(sweep[-1] - 1 / factor) < 1e-15
+    for share in (0.25, 0.5, 0.75):         # orig/wavelength = low + share * (high - low)
+        w = orig / (low + share * (high - low))
+        assert abs(ratio(w) - ((1 - share) / factor + share)) < 1e-9, share
+    # the benchmark model's table (head size 128, base 5e5) has several entries inside the band
+    base, got = table(128, 500000.0), table(128, 500000.0, sc)
+    wl = 2 * math.pi / base
+    mid = (wl > orig / high) & (wl < orig / low)
+    assert mid.sum() >= 5
+    r = got / base
+    assert np.all(np.diff(r) <= 1e-12) and np.all((r[mid] < 1.0) & (r[mid] > 1.0 / factor))
+    s = (orig / wl[mid] - low) / (high - low)
+    assert np.allclose(r[mid], (1 - s) / factor + s, rtol=1e-9)
+
+
+def test_plain_and_engine_tables_agree():
+    for rot, theta, sc in ((32, 500000.0, TINY_B["rope_scaling"]), (128, 500000.0, dict(TINY_B["rope_scaling"], original_max_position_embeddings=8192)),
+                           (16, 10000.0, None), (48, 1000.0, {"rope_type": "linear", "factor": 2.0})):
+        assert np.allclose(_plain_table(rot, theta, sc), _engine_table(rot, theta, sc), rtol=1e-12)
 
 
 # ------------------------------------------------------------------ attention
@@ -190,3 +247,26 @@ def test_layer_norms_sit_before_the_parts(model_a):
     assert np.allclose(P.forward(cfg, w1, toks), P.forward(cfg, w2, toks))
     w3 = dict(w); w3["model.layers.0.input_layernorm.weight"] = w["model.layers.0.input_layernorm.weight"] * 3.0
     assert not np.allclose(P.forward(cfg, w, toks), P.forward(cfg, w3, toks))
+
+
+# ------------------------------------------------------------------ the forms for long sequences
+def test_whole_array_forms_equal_the_loops(tmp_path):
+    """``rope_all_at_once`` and ``attention_all_at_once`` (used where the loops would take
+    minutes) against the loops they stand for, with and without a window, grouped heads; and a
+    model read tensor by tensor against the same model read whole."""
+    T, H, Hk, D = 23, 6, 2, 16
+    q, k, v = rng.normal(size=(T, H, D)), rng.normal(size=(T, Hk, D)), rng.normal(size=(T, Hk, D))
+    pos = np.arange(T) + 3
+    for rot in (D, 8):
+        inv = P.rope_inv_freq(rot, 300.0)
+        assert np.allclose(P.rope_all_at_once(q, pos, inv), P.rope(q, pos, inv), rtol=1e-13, atol=1e-15)
+    for window in (None, 5):
+        assert np.allclose(P.attention_all_at_once(q, k, v, 0.3, window), P.attention(q, k, v, 0.3, window), rtol=1e-12)
+    d = make_model("B", str(tmp_path / "m"))
+    cfg, w = P.load_folder(d)
+    cfg2, lazy = P.open_folder(d)
+    assert cfg2 == cfg and sorted(lazy) == sorted(w) and all(np.array_equal(lazy[n], w[n]) for n in w)
+    toks = prompt_ids(40, cfg["vocab_size"], 3)
+    want = P.forward(cfg, w, toks)
+    got = P.forward(cfg, lazy, toks, rows=[0, 17, 39], all_at_once=True)
+    assert np.allclose(got, want[[0, 17, 39]], rtol=1e-10, atol=1e-12)

@@ -60,14 +60,17 @@ def random_state(expected: Mapping[str, ParamSpec], seed: int, std: float = 0.02
 
 def write_random_model(config: Mapping[str, Any], out_dir: str, seed: int, std: float = 0.02,
                        norm_jitter: float = 0.0, dtype: str = "bfloat16",
-                       vector_dtype: Optional[str] = None) -> str:
-    """Write ``out_dir/config.json`` and ``out_dir/model.safetensors`` for ``config`` (a config.json dict)."""
+                       vector_dtype: Optional[str] = None, device: Optional[torch.device] = None) -> str:
+    """Write ``out_dir/config.json`` and ``out_dir/model.safetensors`` for ``config`` (a config.json dict).
+    ``device``: where the values are drawn (a large model is drawn much faster on the GPU; the
+    values depend on the device's generator, the file is what counts)."""
     from ..config import config_from_dict
     from ..engine.model import Model
     arch, typed = config_from_dict(config)
     spec = arch.build_spec(typed)
     expected = Model.expected_tensors(spec)
-    state = random_state(expected, seed, std=std, jitter=norm_jitter, dtype=dtype, vector_dtype=vector_dtype)
+    state = random_state(expected, seed, std=std, jitter=norm_jitter, dtype=dtype, vector_dtype=vector_dtype,
+                         device=torch.device(device) if device is not None else None)
     os.makedirs(out_dir, exist_ok=True)
     cfg = dict(config)
     cfg.setdefault("torch_dtype", dtype)
