@@ -294,6 +294,6 @@ def test_command_line(folders):
     b = subprocess.run(cmd, capture_output=True, timeout=120)
     assert a.returncode == 0 and a.stdout == b.stdout and a.stdout.startswith(b"hi\n")
     bad = subprocess.run(cmd[:-2] + ["-s", "0"], capture_output=True, text=True, timeout=120)
-    assert bad.returncode == 1 and "not a usable seed" in bad.stderr
+    assert bad.returncode == 1 and "seed 0 cannot be used" in bad.stderr
     long = subprocess.run(cmd[:4] + ["--ids", ",".join(["1"] * 200), "-c", "100"], capture_output=True, text=True, timeout=120)
     assert long.returncode == 1 and "does not fit a context of 100" in long.stderr

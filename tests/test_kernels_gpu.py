@@ -42,6 +42,14 @@ def test_embedding(ops, V, E, dt):
         assert torch.equal(ops.embedding(packed, ids, scale=1.0), want)
 
 
+@pytest.mark.parametrize("n_words,blocks", [(4, 1), (1 << 20, 64), (12345 * 4, 2048), (3 * (1 << 20) + 4, 7)])
+def test_stream_read_reads_every_word_once(ops, n_words, blocks):
+    """The memory yardstick's kernel: the XOR it leaves is the XOR of all words of the buffer."""
+    buf = torch.randint(-2 ** 31, 2 ** 31 - 1, (n_words,), dtype=torch.int32, device=DEV)
+    got = ops.stream_read(buf, blocks).cpu().numpy().view(np.uint32)
+    assert np.bitwise_xor.reduce(got) == np.bitwise_xor.reduce(buf.cpu().numpy().view(np.uint32))
+
+
 @pytest.mark.parametrize("E", [8, 100, 4096, 5000])
 @pytest.mark.parametrize("out", ["float32", "bfloat16"])
 @pytest.mark.parametrize("wdt", ["float32", "bfloat16"])

@@ -33,26 +33,26 @@ VERSION_LINE = "runner (xyntetik-runner_amd) {v}"
 USAGE = """usage: runner -m MODEL_DIR [options]
 
 options:
-  -m PATH        model folder (config.json + model.safetensors)
-  -p TEXT        prompt (one-shot completion; \\n etc. are unescaped)
-  -f FILE        read prompt from file (appended after -p text)
-  --ids LIST     prompt as comma-separated token ids; output is printed as ids
-  -n N           max tokens to generate (default 256, -1 = until EOS)
-  -c N           context length (default: min(model max, 4096))
-  -b N           prompt batch size: tokens per step (default 512)
-  -s N           RNG seed (default: time; 0 is refused)
-  --temp F       temperature (0 = greedy: returns the model's argmax
-                 with no repeat penalty applied) (default 0)
-  --top-k N      top-k (0 = off)
-  --top-p F      top-p
-  --min-p F      min-p vs the top candidate (0 = off)
-  --repeat-penalty F  penalty on recently emitted tokens (1 = off)
-  --no-bos       do not add BOS token
-  --ignore-eos   keep generating past end-of-text tokens
+  -m PATH        the model: a folder holding config.json and model.safetensors
+  -p TEXT        the prompt to complete; backslash escapes such as \\n are expanded
+  -f FILE        take the prompt from FILE (it follows the -p text if both are given)
+  --ids LIST     the prompt as token ids separated by commas; the answer is printed as ids too
+  -n N           how many tokens to generate at most (default 256; -1: stop only at an end token)
+  -c N           context length in tokens (default: the model's own limit, capped at 4096)
+  -b N           how many prompt tokens one step may take (default 512)
+  -s N           seed of the sampler's generator (default: from the clock; 0 is refused)
+  --temp F       sampling temperature (default 0 = always the most likely token,
+                 and then no repeat penalty either)
+  --top-k N      sample among the N most likely tokens only (0: no limit)
+  --top-p F      sample from the smallest set of tokens whose probabilities reach F
+  --min-p F      drop tokens less likely than F times the most likely one (0: keep all)
+  --repeat-penalty F  make tokens of the recent window less likely by factor F (1: off)
+  --no-bos       do not put the begin-of-sequence token before the prompt
+  --ignore-eos   go on generating when an end token comes
   --dtype T      bfloat16 (default) or float32
-  --bench-json   run a small decode benchmark and print JSON metrics
-  --version      print the runner version and exit
-  -v             verbose model info
+  --bench-json   time a short generation and print the figures as JSON
+  --version      print the version and leave
+  -v             print the model's sizes while loading
 """
 
 
@@ -164,8 +164,8 @@ def main(argv: Optional[List[str]] = None) -> int:
         sys.stderr.write(USAGE)
         return 1
     if o["seed"] is not None and o["seed"] == 0:
-        sys.stderr.write("error: -s 0 is not a usable seed — the sampler's RNG state 0 is a fixed point. "
-                         "Use any other value.\n")
+        sys.stderr.write("error: seed 0 cannot be used (-s 0): the sampler's generator never leaves state 0. "
+                         "Any other seed will do.\n")
         return 1
     from .config import ConfigError, load_config
     from .weights import SafetensorsError, WeightError

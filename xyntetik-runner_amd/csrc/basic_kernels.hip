@@ -402,3 +402,42 @@ extern "C" int xr_convert(void* out, const void* in, size_t n, int in_dtype, int
     XR_CHECK_LAUNCH("convert");
     return XR_OK;
 }
+
+// ---------------------------------------------------------------- memory yardstick
+// What the memory system delivers to a kernel that does nothing but read: every workgroup
+// streams a range of its own with 16-byte loads marked as streaming, eight of them in flight
+// a lane, and leaves the XOR of its words (so the loads cannot be dropped, and a test can
+// check that every word was read once).  The benchmark reports a decode step's bytes per second
+// as a fraction of this figure beside the fraction of the nominal peak.
+typedef uint32_t xr_u32x4 __attribute__((ext_vector_type(4)));
+__global__ __launch_bounds__(256) void k_stream_read(const xr_u32x4* __restrict__ src, size_t n16, uint32_t* __restrict__ sink) {
+    const size_t per = (n16 + gridDim.x - 1) / gridDim.x;
+    const size_t begin = (size_t)blockIdx.x * per;
+    const size_t end = begin + per < n16 ? begin + per : n16;
+    xr_u32x4 acc = {0u, 0u, 0u, 0u};
+    size_t i = begin + threadIdx.x;
+    for (; i + 7 * 256 < end; i += 8 * 256) {
+        xr_u32x4 v[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) v[u] = __builtin_nontemporal_load(src + i + u * 256);
+#pragma unroll
+        for (int u = 0; u < 8; ++u) acc ^= v[u];
+    }
+    for (; i < end; i += 256) acc ^= __builtin_nontemporal_load(src + i);
+    uint32_t x = acc.x ^ acc.y ^ acc.z ^ acc.w;
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) x ^= __shfl_xor(x, o, 64);
+    __shared__ uint32_t part[4];
+    if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = x;
+    __syncthreads();
+    if (threadIdx.x == 0) sink[blockIdx.x] = part[0] ^ part[1] ^ part[2] ^ part[3];
+}
+
+// sink: [blocks] words; the XOR of all of them is the XOR of the buffer's 32-bit words.
+extern "C" int xr_stream_read(const void* src, size_t bytes, uint32_t* sink, int blocks, hipStream_t stream) {
+    XR_REQUIRE(src && sink && blocks > 0 && blocks <= 65535, "stream_read: bad operands (%d workgroups)", blocks);
+    XR_REQUIRE(bytes % 16 == 0 && ((uintptr_t)src % 16) == 0, "stream_read: the buffer must be a multiple of 16 bytes long and aligned so");
+    k_stream_read<<<blocks, 256, 0, stream>>>((const xr_u32x4*)src, bytes / 16, sink);
+    XR_CHECK_LAUNCH("stream_read");
+    return XR_OK;
+}

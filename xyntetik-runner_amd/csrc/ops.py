@@ -50,6 +50,7 @@ _PROTOS = {
     "xr_add": [_p, _p, _sz, _i, _p],
     "xr_fill_rows": [_p, _p, _i, _sz, _u32, _p],
     "xr_convert": [_p, _p, _sz, _i, _i, _p],
+    "xr_stream_read": [_p, _sz, _p, _i, _p],
     "xr_gemm_ref": [_p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _p],
     "xr_gemm_bf16": [_p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _p, _sz, _p, _p, _p],
     "xr_pack_weight": [_p, _p, _i, _i, _p],
@@ -251,6 +252,17 @@ class Ops:
         self.lib.check(self.lib.xr_convert(out.data_ptr(), x.data_ptr(), x.numel(), dtype_code(x.dtype),
                                            dtype_code(dtype), _stream()))
         return out
+
+    def stream_read(self, buf: torch.Tensor, blocks: int = 2048) -> torch.Tensor:
+        """Read ``buf`` once, every workgroup a range of its own (the yardstick for what a kernel
+        that only reads gets from memory); returns ``[blocks]`` int32 whose XOR is the XOR of the
+        buffer's 32-bit words."""
+        self._dev(buf)
+        self._contig(buf, "stream_read buffer")
+        sink = torch.empty((blocks,), dtype=torch.int32, device=buf.device)
+        self.lib.check(self.lib.xr_stream_read(buf.data_ptr(), buf.numel() * buf.element_size(), sink.data_ptr(),
+                                               blocks, _stream()))
+        return sink
 
     # -- matrix product ---------------------------------------------------------
     GEMM_WORKSPACE_BYTES = 96 << 20
