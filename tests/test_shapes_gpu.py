@@ -1,4 +1,4 @@
-"""The benchmark model's layer sizes, end to end against the plain implementation.
+"""The benchmark models' layer sizes, end to end against the plain implementation.
 
 Two of its 32 layers at their real widths (hidden 4096, 32 query and 8 key/value heads of 128,
 feed-forward 14336, vocabulary 128256, llama3 rotary scaling with an original context of 8192),
@@ -42,17 +42,24 @@ DECODED = 24
 LONG_ROWS = [0, 1, 2, 63, 64, 127, 128, 255, 256, 1023, 1024, 2046, 2047]
 
 
-@pytest.fixture(scope="module")
-def shape_8b(tmp_path_factory):
+def make_case(config, folder, seed, prompts, decoded, long_rows):
+    """A random model of ``config`` in ``folder``, requests ``prompts`` (name -> prompt length) with
+    ``decoded`` given tokens each, and the plain logits at the compared places: ``long_rows`` and the
+    decoded tokens of the request "long", every place of the others."""
     from xyntetik_runner_amd.weights import write_random_model
-    d = write_random_model(SHAPE_8B_2_OF_32_LAYERS, str(tmp_path_factory.mktemp("shape8b")), seed=8, device="cuda:0")
+    d = write_random_model(config, folder, seed=seed, device="cuda:0")
     cfg, w = P.open_folder(d)                       # a matrix is widened when its product comes, not before
     V = cfg["vocab_size"]
-    reqs = {name: prompt_ids(n + DECODED, V, 500 + i) for i, (name, n) in enumerate(PROMPT.items())}
-    rows = {"long": LONG_ROWS + list(range(PROMPT["long"], PROMPT["long"] + DECODED)),
-            "mid": list(range(PROMPT["mid"] + DECODED)), "short": list(range(PROMPT["short"] + DECODED))}
+    reqs = {name: prompt_ids(n + decoded, V, 500 + i) for i, (name, n) in enumerate(prompts.items())}
+    rows = {name: (long_rows + list(range(n, n + decoded)) if name == "long" else list(range(n + decoded)))
+            for name, n in prompts.items()}
     want = {name: P.forward(cfg, w, reqs[name], rows=rows[name], all_at_once=True) for name in reqs}
     return d, cfg, reqs, rows, want
+
+
+@pytest.fixture(scope="module")
+def shape_8b(tmp_path_factory):
+    return make_case(SHAPE_8B_2_OF_32_LAYERS, str(tmp_path_factory.mktemp("shape8b")), 8, PROMPT, DECODED, LONG_ROWS)
 
 
 def run_steps(d, dtype, steps):
@@ -126,3 +133,50 @@ def test_8b_widths_2_of_32_layers_mixed(shape_8b, dtype):
     assert [sum(len(t) for _, t, _ in st) for st in steps[:5]] == [49, 1026, 602, 386, 42]
     got, runner = run_steps(d, dtype, steps)
     compare(got, want, dtype, "mixed")
+
+
+# ----------------------------------------------------------------------------- the other two shapes
+# Llama-2-7B's widths: one query head a key/value head (32 of them), a feed-forward of 11,008, a
+# vocabulary of 32,000, no rotary scaling.  Llama-3.1-70B's: 8 query heads a key/value head (4 tokens
+# fill an attention block of 32 rows), a width of 8,192, a feed-forward of 28,672.
+OTHER_SHAPES = {
+    "7b_widths_2_of_32_layers": dict(SHAPE_8B_2_OF_32_LAYERS, num_key_value_heads=32, intermediate_size=11008,
+                                     vocab_size=32000, rope_theta=10000.0, rope_scaling=None,
+                                     max_position_embeddings=4096),
+    "70b_widths_1_of_80_layers": dict(SHAPE_8B_2_OF_32_LAYERS, num_hidden_layers=1, hidden_size=8192,
+                                      num_attention_heads=64, intermediate_size=28672),
+}
+OTHER_PROMPT = {"long": 640, "short": 21}
+OTHER_DECODED = 12
+OTHER_LONG_ROWS = [0, 1, 63, 64, 127, 128, 511, 512, 575, 576, 639]
+
+
+@pytest.fixture(scope="module", params=list(OTHER_SHAPES))
+def other_shape(request, tmp_path_factory):
+    case = make_case(OTHER_SHAPES[request.param], str(tmp_path_factory.mktemp(request.param)), 9, OTHER_PROMPT,
+                     OTHER_DECODED, OTHER_LONG_ROWS)
+    yield (request.param,) + case
+    import shutil
+    shutil.rmtree(case[0], ignore_errors=True)          # (a model file of several GB)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_other_benchmark_widths(other_shape, dtype):
+    """The short request's prompt alone (21 rows), then a step of 577 rows (a 576-row portion of the
+    long prompt beside a decoded token), one of 65 (the portion's rest and a decoded token), then
+    decoded tokens of both."""
+    name, d, cfg, reqs, rows, want = other_shape
+    L, S = reqs["long"], reqs["short"]
+    pl, ps = OTHER_PROMPT["long"], OTHER_PROMPT["short"]
+    steps = [
+        [("short", S[:ps], list(range(ps)))],
+        [("long", L[:576], [r for r in rows["long"] if r < 576]), ("short", [S[ps]], [0])],
+        [("short", [S[ps + 1]], [0]), ("long", L[576:pl], [r - 576 for r in rows["long"] if 576 <= r < pl])],
+    ]
+    for i in range(OTHER_DECODED):
+        entries = [("long", [L[pl + i]], [0])]
+        if i + 2 < OTHER_DECODED:
+            entries.append(("short", [S[ps + 2 + i]], [0]))
+        steps.append(entries)
+    got, runner = run_steps(d, dtype, steps)
+    compare(got, want, dtype, name)
