@@ -151,3 +151,23 @@ def test_sizes_the_kernels_do_not_take_are_refused_when_the_model_is_built():
     from xyntetik_runner_amd.parts import make_part
     with pytest.raises(ValueError, match="silu"):
         make_part("feed_forward", PartSpec("gated_mlp", {"hidden_size": 8, "intermediate_size": 16, "activation": "gelu"}))
+
+
+def test_a_layer_brings_exactly_the_parts_its_arrangement_names():
+    """The arrangement names its norms and says whether it has a mixer and a feed-forward; a layer
+    spec that brings other norms, or lacks a part, is refused when the model is built."""
+    from xyntetik_runner_amd.config import LayerSpec, PartSpec
+    from xyntetik_runner_amd.engine.model import Model
+    import dataclasses
+    arch, cfg = config_from_dict(TINY_A)
+    spec = arch.build_spec(cfg)
+    layer = spec.layers[0]
+    assert set(layer.norms) == {"mixer_norm", "feed_forward_norm"}
+    third = dict(layer.norms, extra_norm=PartSpec("rmsnorm", {"size": 64, "eps": 1e-5}, prefix="x."))
+    for bad in (dataclasses.replace(layer, norms=third),
+                dataclasses.replace(layer, norms={"mixer_norm": layer.norms["mixer_norm"]}),
+                dataclasses.replace(layer, feed_forward=None)):
+        with pytest.raises(ValueError):
+            Model(dataclasses.replace(spec, layers=[bad] + list(spec.layers[1:])))
+    names = Model(spec).expected()
+    assert "model.layers.0.input_layernorm.weight" in names and "model.layers.1.post_attention_layernorm.weight" in names
