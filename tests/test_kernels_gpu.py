@@ -553,13 +553,18 @@ def test_projection_with_rotation_and_cache_write(ops, dt, H, Hk, D, rot, inter,
     want_v = proj[:, Q + K:].cpu().reshape(T, Hk, D)
     tol = 1e-5 if dt == "float32" else 6e-3
     results = []
-    for fuse in (True, False):
+    asked = []
+    def step_table():                  # the step's cosines and sines, made once for all layers
+        asked.append(1)
+        return ops.rope_table(ctx.positions, inv, 1.0)
+    for fuse in (True, False, "with the step's table"):
         kc = torch.full((n_pages, Hk, ps, D), float("nan"), device=DEV, dtype=DT[dt])
         vc = torch.full((n_pages, Hk, D, ps), float("nan"), device=DEV, dtype=DT[dt])
-        ops.fuse_rope = fuse
+        ops.fuse_rope = bool(fuse)
         try:
             q = ops.project_rope_kv_write(h, ops.pack_weight(wp), bp, kc, vc, ctx.positions, ctx.req_of_token,
-                                          ctx.block_table(0), inv, H, Hk, D, rot, inter, 1.0, ps, paired=paired)
+                                          ctx.block_table(0), inv, H, Hk, D, rot, inter, 1.0, ps, paired=paired,
+                                          cs_table=step_table if fuse not in (True, False) and rot else None)
         finally:
             ops.fuse_rope = True
         assert q.dtype == DT[dt] and rel(q.cpu().reshape(T, H, D), want_q) < tol
@@ -576,8 +581,11 @@ def test_projection_with_rotation_and_cache_write(ops, dt, H, Hk, D, rot, inter,
         assert torch.isnan(vc.float().cpu().permute(0, 3, 1, 2)[~written]).all()
         results.append((q.float().cpu(), torch.nan_to_num(kc.float().cpu()), torch.nan_to_num(vc.float().cpu())))
     if dt == "bfloat16":
-        for one, two in zip(*results):          # the same sums and formulas: at most a rounding apart
+        for one, two, three in zip(*results):   # the same sums and formulas: at most a rounding apart
             assert rel(one, two) < 4e-3
+            assert torch.equal(one, three)      # a table made beforehand holds what the product would make itself
+        # the table is asked for only where the tile kernel rotates (from 512 rows)
+        assert len(asked) == (1 if rot and T >= 512 and (inter or paired) and D % 16 == 0 else 0)
 
 
 def ref_attention(q, k_seq, v_seq, starts, q_lens, scale, window):

@@ -102,6 +102,7 @@ struct XrGemmRope {
     void* q_out;
     void* k_cache;
     void* v_cache;
+    const void* cs_table;   // [M][rot/2] (cosine, sine) pairs made by xr_rope_table for these rows, or null: the product makes its own
 };
 
 // what a caller passes to fold a norm into a product of at most 16 rows (see GemmArgs)
@@ -1054,6 +1055,19 @@ extern "C" int xr_pack_weight(void* dst, const void* src, int N, int K, hipStrea
     return XR_OK;
 }
 
+// The table of a step's rotation angles, [M][half] (cosine, sine) times mscale, that a product of
+// many rows takes in XrGemmRope.cs_table: the same for every layer that rotates by the same
+// frequencies, so a step makes it once.
+extern "C" int xr_rope_table(void* cs, const int* positions, const float* inv_freq, int M, int half, float mscale,
+                             hipStream_t stream) {
+    XR_REQUIRE(cs && positions && inv_freq && M >= 0 && half > 0, "rope_table: bad operands (M=%d, half=%d)", M, half);
+    XR_REQUIRE(((uintptr_t)cs % 8) == 0, "rope_table: the table must be 8-byte aligned");
+    if (M == 0) return XR_OK;
+    k_rope_table<<<(unsigned)(((size_t)M * half + 255) / 256), 256, 0, stream>>>((float2*)cs, positions, inv_freq, M, half, mscale);
+    XR_CHECK_LAUNCH("rope_table");
+    return XR_OK;
+}
+
 // epi: 0 store, 1 add into float out, 2 gated (w has 2N rows: gate rows then up rows; act: XR_ACT_*).
 // variant: 0 = choose by shape; 1 = skinny; 10..20 = tile shapes; 30, 31 = few rows with K split;
 //          +1000 = row tiles of one weight tile follow each other.
@@ -1112,7 +1126,7 @@ extern "C" int xr_gemm_bf16(void* out, const void* a, const void* w, const float
         XR_REQUIRE(variant == 0 && epi == EPI_STORE && !(norm && norm->xg),
                    "gemm: rotation and cache write are folded only into a plain product whose kernel the library chooses");
         if (rope_direct) {
-            XR_REQUIRE(workspace && (size_t)M * (rope->rot / 2 + 1) * sizeof(float2) <= workspace_bytes,
+            XR_REQUIRE(rope->cs_table || (workspace && (size_t)M * (rope->rot / 2 + 1) * sizeof(float2) <= workspace_bytes),
                        "gemm: rotation after a product of %d rows needs a workspace for its table", M);
             XR_REQUIRE(((uintptr_t)rope->q_out % 8) == 0 && ((uintptr_t)rope->k_cache % 8) == 0 && ((uintptr_t)rope->v_cache % 16) == 0,
                        "gemm: queries and caches must be 16-byte aligned");
@@ -1136,7 +1150,9 @@ extern "C" int xr_gemm_bf16(void* out, const void* a, const void* w, const float
         g.rope.mscale = rope->mscale; g.rope.page_shift = shift < 0 ? 0 : shift; g.rope.page_mask = rope->page_size - 1;
         g.rope.page_size = rope->page_size;
         g.rope.q_out = (bf16_t*)rope->q_out; g.rope.k_cache = (bf16_t*)rope->k_cache; g.rope.v_cache = (bf16_t*)rope->v_cache;
-        if (rope_direct) {
+        if (rope_direct && rope->cs_table) {
+            g.rope.cs = (const float2*)rope->cs_table;      // made once for the step, for every layer with this rotation
+        } else if (rope_direct) {
             g.rope.cs = (const float2*)workspace;
             const int half = rope->rot / 2;
             if (half > 0) {

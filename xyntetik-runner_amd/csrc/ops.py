@@ -54,6 +54,7 @@ _PROTOS = {
     "xr_gemm_ref": [_p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _p],
     "xr_gemm_bf16": [_p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _p, _sz, _p, _p, _p],
     "xr_pack_weight": [_p, _p, _i, _i, _p],
+    "xr_rope_table": [_p, _p, _p, _i, _i, _f, _p],
     "xr_attention_ref": [_p, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _f, _i, _i, _p],
     "xr_sample": [_p, _p, _i, _i, _i, _p, _p, _p, _p, _p, _p, _p, _p, _i, _p, _i, _p, _p],
 }
@@ -125,7 +126,7 @@ class _GemmRope(C.Structure):
     """XrGemmRope of the library."""
     _fields_ = [("positions", _p), ("req_of_token", _p), ("block_table", _p), ("table_stride", _i),
                 ("inv_freq", _p), ("H", _i), ("Hk", _i), ("D", _i), ("rot", _i), ("interleaved", _i),
-                ("mscale", _f), ("page_size", _i), ("q_out", _p), ("k_cache", _p), ("v_cache", _p)]
+                ("mscale", _f), ("page_size", _i), ("q_out", _p), ("k_cache", _p), ("v_cache", _p), ("cs_table", _p)]
 
 
 def paired_order(D: int, rot: int) -> list:
@@ -458,9 +459,20 @@ class Ops:
             1 if interleaved else 0, float(mscale), page_size, dtype_code(store.dtype), 1 if paired else 0,
             _stream()))
 
+    def rope_table(self, positions: torch.Tensor, inv_freq: torch.Tensor, mscale: float = 1.0) -> torch.Tensor:
+        """``[T, rot/2, 2]`` float32: cosine and sine (times ``mscale``) of every row's angles, as
+        ``project_rope_kv_write`` takes them for a product of many rows (``cs_table``); the same for
+        every layer that rotates by ``inv_freq``, so a step needs it once."""
+        self._dev(positions, inv_freq)
+        T, half = positions.numel(), inv_freq.numel()
+        out = torch.empty((T, half, 2), dtype=torch.float32, device=positions.device)
+        self.lib.check(self.lib.xr_rope_table(out.data_ptr(), positions.data_ptr(), inv_freq.data_ptr(), T, half,
+                                              float(mscale), _stream()))
+        return out
+
     def project_rope_kv_write(self, h, w, bias, k_cache, v_cache, positions, req_of_token, block_table,
                               inv_freq, H: int, Hk: int, D: int, rot: int, interleaved: bool, mscale: float,
-                              page_size: int, paired: bool = False) -> torch.Tensor:
+                              page_size: int, paired: bool = False, cs_table=None) -> torch.Tensor:
         """``[q | k | v] = h @ w^T (+ bias)``, queries and keys rotated, keys and values written
         to their pages; returns the rotated queries ``[T, H*D]`` in the compute dtype.
 
@@ -470,7 +482,8 @@ class Ops:
         stores its own result, up to 64 the kernel that adds the product's K ranges up does, from
         512 the tile kernel (with the rows' cosines and sines from a table made first), which
         saves a kernel and the 32-bit copy of the projections; otherwise the product and
-        ``rope_kv_write`` run one after the other."""
+        ``rope_kv_write`` run one after the other.  ``cs_table``: a callable that returns the
+        step's ``rope_table`` (asked for only where the tile kernel rotates)."""
         rows = h.data if isinstance(h, UnscaledRows) else h
         wt = w.data if isinstance(w, PackedWeight) else w
         T, Q, KV = rows.shape[0], H * D, Hk * D
@@ -494,6 +507,8 @@ class Ops:
             rp.inv_freq, rp.H, rp.Hk, rp.D, rp.rot = _ptr(inv_freq), H, Hk, D, rot
             rp.interleaved, rp.mscale, rp.page_size = 1 if interleaved else 0, float(mscale), page_size
             rp.q_out, rp.k_cache, rp.v_cache = q.data_ptr(), _ptr(k_cache) if Hk else None, _ptr(v_cache) if Hk else None
+            table = cs_table() if (cs_table is not None and T >= self.ROPE_TILE_ROWS and rot > 0) else None
+            rp.cs_table = _ptr(table)
             self.lib.check(self.lib.xr_gemm_bf16(None, rows.data_ptr(), wt.data_ptr(), _ptr(bias), T, w.shape[0],
                                                  rows.shape[1], rows.stride(0), w.shape[0], XR_F32, 0, 0, 0,
                                                  1 if isinstance(w, PackedWeight) else 0,

@@ -227,6 +227,7 @@ class StepContext:
         self.fresh_slots_host = [rc.slot for rc in request_caches if rc.fresh]
         self.slots_host = [rc.slot for rc in request_caches]
         self._plans = {}
+        self.shared = {}        # what parts make once a step and share between layers (a rotation's table)
 
     def attention_plan(self, group: int, group_size: int, window: Optional[int], n_kv_heads: int,
                        page_size: int = 64) -> AttentionPlan:

@@ -122,7 +122,7 @@ class PagedAttention(Mixer):
                 h, self.w_in, self.b_in, cache.k if writes else None, cache.v if writes else None, ctx.positions,
                 ctx.req_of_token, table, rot.inv_freq if rot else None, H, Hk if writes else 0, D,
                 rot.rotary_dim if rot else 0, rot.interleaved if rot else False, rot.mscale if rot else 1.0,
-                cache.page_size, paired=self.paired)
+                cache.page_size, paired=self.paired, cs_table=(lambda: self._step_table(ctx, rot)) if rot else None)
         else:
             # a position encoding of its own works on the 32-bit queries and keys before they are
             # cached; or the keys and values this layer computes are another layer's to store
@@ -140,6 +140,18 @@ class PagedAttention(Mixer):
                               rot.mscale if rot else 1.0, cache.page_size, paired=self.paired)
         return ops.attention(q, cache.k, cache.v, ctx, cache.group, H, Hk, D, cache.page_size, self.scale,
                              self.window)
+
+    def _step_table(self, ctx, rot):
+        """The step's cosines and sines for this rotation, made once and shared by every layer
+        that rotates by the same table (a step context keeps what its parts leave in ``shared``)."""
+        shared = getattr(ctx, "shared", None)
+        if shared is None:
+            return self.rt.ops.rope_table(ctx.positions, rot.inv_freq, rot.mscale)
+        key = ("rope_table", rot.table_key if rot.table_key is not None else rot.inv_freq.data_ptr(), rot.mscale)
+        table = shared.get(key)
+        if table is None:
+            table = shared[key] = self.rt.ops.rope_table(ctx.positions, rot.inv_freq, rot.mscale)
+        return table
 
     def forward(self, ctx, cache, h):
         return self.rt.ops.linear(self._attend(ctx, cache, h), self.w_out, bias=self.b_out)

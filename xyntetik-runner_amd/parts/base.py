@@ -113,6 +113,7 @@ class RotaryParams:
     rotary_dim: int
     interleaved: bool           # False: pairs (j, j + rotary_dim/2); True: pairs (2j, 2j+1)
     mscale: float = 1.0
+    table_key: Any = None       # equal keys promise equal tables (layers then share a step's cosines and sines)
 
 
 class PositionEncoding(Part):

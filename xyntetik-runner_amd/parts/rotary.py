@@ -66,7 +66,8 @@ class Rotary(PositionEncoding):
     def bind(self, tensors, rt) -> None:
         self.rt = rt
         table = rotary_inv_freq(self.rotary_dim, self.theta, self.scaling).to(torch.float32).to(rt.device)
-        self._params = RotaryParams(table, self.rotary_dim, self.interleaved, self.mscale)
+        key = ("rotary", self.rotary_dim, self.theta, repr(sorted(self.scaling.items())) if self.scaling else None)
+        self._params = RotaryParams(table, self.rotary_dim, self.interleaved, self.mscale, table_key=key)
 
     def rotary(self) -> Optional[RotaryParams]:
         return self._params
