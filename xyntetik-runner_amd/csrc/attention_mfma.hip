@@ -74,18 +74,28 @@ __device__ inline uint4 keep_if(bool ok, uint4 v) {     // zero unless ok, word 
 __device__ inline uint32_t pack2(float lo, float hi) { return pack_bf16x2(lo, hi); }
 
 // One tile's softmax step for the lane's row: p[] from s[], the running reference m and sum l,
-// and the rescaling of the output accumulators when the reference moved.  The reference is a
+// and the rescaling of the output accumulators when the reference moved.  A row's scores lie in two
+// lanes (32 apart); the maximum is exchanged every tile, the sum l is kept per lane (both lanes
+// rescale by the same factor) and the two halves are added once, when the row is finished.  The reference is a
 // maximum seen so far, and follows the true maximum only when that has risen by more than
 // MAX_SLACK (in units of log2): any reference gives the same quotient sum(p v) / sum(p), terms up
 // to 2^8 are no strain on 32-bit sums or on bfloat16 P, and the 64 multiplications a lane owes
 // its output when any row of the wave moves its reference become rare (before, nearly every tile
 // of a few thousand keys paid them).
+// the largest of three in one instruction (fmaxf's promise about signalling NaNs costs a second
+// instruction per maximum; a NaN score makes the row's output NaN either way)
+__device__ inline float max3(float a, float b, float c) {
+    float r;
+    asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+    return r;
+}
 #define MAX_SLACK 8.0f
 #define ATTN_SOFTMAX_STEP(KT, KEND)                                                                  \
         if ((KT) + 32 <= (KEND) && (KT) + 31 <= pos_min && (KT) >= lo_max) {                             \
-            float mt = fmaxf(fmaxf(s[0], s[1]), fmaxf(s[2], s[3]));                                      \
+            float mt = max3(s[0], s[1], s[2]);                                                           \
 _Pragma("unroll")                                                                                        \
-            for (int e = 4; e < 16; e += 4) mt = fmaxf(mt, fmaxf(fmaxf(s[e], s[e + 1]), fmaxf(s[e + 2], s[e + 3]))); \
+            for (int e = 3; e < 15; e += 2) mt = max3(mt, s[e], s[e + 1]);                               \
+            mt = fmaxf(mt, s[15]);                                                                       \
             mt = fmaxf(mt, __shfl_xor(mt, 32, 64));                                                      \
             const float mn = mt * c2 > m + MAX_SLACK ? mt * c2 : m;                                      \
             corr = __builtin_amdgcn_exp2f(m - mn);                                                       \
@@ -95,7 +105,6 @@ _Pragma("unroll")                                                               
                 p[e] = __builtin_amdgcn_exp2f(fmaf(s[e], c2, -mn));                                      \
                 rs += p[e];                                                                              \
             }                                                                                            \
-            rs += __shfl_xor(rs, 32, 64);                                                                \
             l = fmaf(l, corr, rs);                                                                       \
             m = mn;                                                                                      \
         } else {                                                                                         \
@@ -117,7 +126,6 @@ _Pragma("unroll")                                                               
                 p[e] = __builtin_amdgcn_exp2f(p[e] - mu);                                                \
                 rs += p[e];                                                                              \
             }                                                                                            \
-            rs += __shfl_xor(rs, 32, 64);                                                                \
             l = fmaf(l, corr, rs);                                                                       \
             m = mn;                                                                                      \
         }                                                                                                \
@@ -167,8 +175,10 @@ _Pragma("unroll")                                                               
 // Long prompt portions: a workgroup of 4 waves takes 128 consecutive rows of one request and
 // key/value head (wave w the rows row0 + 32 w ..) and a range of keys.  The K tile
 // [32 keys][HD] and the V^T tile [HD][32 keys] are copied once into LDS for all four waves,
-// by asynchronous copies that run CTA_STAGES - 1 tiles ahead (measured at head size 128: 4 tiles
-// in LDS give 10% over 3, 5 nothing more), instead of once per wave from
+// by asynchronous copies, two tiles at a time into the places of the two tiles before the ones
+// being worked on (4 tiles in LDS; measured at head size 128, a prompt of 2,048 tokens: a barrier
+// and a round of address arithmetic every tile with three tiles ahead 73 us, every second tile
+// 71 us), instead of once per wave from
 // the caches; each wave then works as above with its fragments read from LDS.  A wave skips
 // the tiles that none of its rows can see, but takes part in every copy and barrier.
 //
@@ -184,8 +194,8 @@ constexpr int NVC = DB * 32 * 4;                            // chunks of a V^T t
 constexpr int CTA_ROWS = 128;
 constexpr int CTA_LOADS = (NKC + NVC + 255) / 256;          // copies per lane and tile
 constexpr int STAGE_CHUNKS = CTA_LOADS * 256;
-constexpr int CTA_STAGES = STAGE_CHUNKS * 16 * 4 <= 64 * 1024 ? 4 : 3;   // tiles in LDS: two workgroups a compute unit, or one
-static_assert(CTA_LOADS * (CTA_STAGES - 2) < 64, "too many copies in flight for the counter");
+constexpr int CTA_STAGES = 4;                               // tiles in LDS (copied two at a time)
+static_assert(CTA_STAGES * STAGE_CHUNKS * 16 <= 160 * 1024, "the tiles do not fit into LDS");
 
 __global__ __launch_bounds__(256, 2) void k_attn_cta(AttnArgs a) {
     extern __shared__ uint4 lds[];                          // [CTA_STAGES][STAGE_CHUNKS]
@@ -314,13 +324,20 @@ __global__ __launch_bounds__(256, 2) void k_attn_cta(AttnArgs a) {
         lo_min = min(lo_min, __shfl_xor(lo_min, o_, 64));
     }
 
+    // The tiles are copied and waited for two at a time: the workgroup meets at a barrier, and the
+    // copies' addresses are worked out, every second tile (two tiles take a wave over 2 us, more
+    // than a copy from L2 needs to land).
+    static_assert(CTA_STAGES % 2 == 0 && CTA_LOADS * 2 < 64, "the tiles in LDS come in pairs");
 #pragma unroll
-    for (int st = 0; st < CTA_STAGES - 1; ++st) CTA_ISSUE(st)
+    for (int st = 0; st < CTA_STAGES - 2; ++st) CTA_ISSUE(st)
     for (int ti = 0; ti < nt; ++ti) {
-        // tile ti has landed when at most the CTA_STAGES-2 younger tiles are still on their way
-        wait_vmcnt<CTA_LOADS * (CTA_STAGES - 2)>();
-        __builtin_amdgcn_s_barrier();                    // for every wave; and tile ti-1 is no longer read
-        CTA_ISSUE(ti + CTA_STAGES - 1)                   // into the place of tile ti-1 (zeros past the end)
+        if ((ti & 1) == 0) {
+            // tiles ti and ti+1 have landed when at most the CTA_STAGES-4 younger ones are on their way
+            wait_vmcnt<CTA_LOADS * (CTA_STAGES - 4)>();
+            __builtin_amdgcn_s_barrier();                // for every wave; and tiles ti-2, ti-1 are no longer read
+            CTA_ISSUE(ti + CTA_STAGES - 2)               // into their places (zeros past the end)
+            CTA_ISSUE(ti + CTA_STAGES - 1)
+        }
         const int kt = kbeg + ti * 32;
         if (kt > pos_max || kt + 32 <= lo_min) continue; // nothing here for this wave's rows
         const uint4* Ks = lds + (ti % CTA_STAGES) * STAGE_CHUNKS;
@@ -370,6 +387,7 @@ __global__ __launch_bounds__(256, 2) void k_attn_cta(AttnArgs a) {
     }
 #undef CTA_ISSUE
     wait_vmcnt<0>();                                     // the trailing copies of zeros
+    l += __shfl_xor(l, 32, 64);                          // the row's sum from its two lanes
 
     ATTN_WRITE_OUT(slot)
 }
@@ -568,6 +586,7 @@ __global__ __launch_bounds__(64 * STREAM_WAVES) void k_attn_stream(AttnArgs a) {
     }
 #undef STREAM_ISSUE
     wait_vmcnt<0>();                                     // the trailing copies of zeros
+    l += __shfl_xor(l, 32, 64);                          // the row's sum from its two lanes
     __syncthreads();                                     // the rings are free
 
     // ---- combine the waves: sum_w 2^(m_w - max) O_w over sum_w 2^(m_w - max) l_w
