@@ -195,23 +195,43 @@ constexpr int CTA_ROWS = 128;
 constexpr int CTA_LOADS = (NKC + NVC + 255) / 256;          // copies per lane and tile
 constexpr int STAGE_CHUNKS = CTA_LOADS * 256;
 constexpr int CTA_STAGES = 4;                               // tiles in LDS (copied two at a time)
-static_assert(CTA_STAGES * STAGE_CHUNKS * 16 <= 160 * 1024, "the tiles do not fit into LDS");
+// Two sets of four waves share an item where LDS has room for two rings: the first set takes the
+// first half of the item's tiles, the second set the rest, and their results are combined through
+// LDS at the end.  A compute unit then has two waves a SIMD from ONE item, and the items, which
+// start longest first, follow one another on it: a causal prompt's blocks see 1 to n keys, and with
+// one set an item (two items to a unit, a long one beside a short one) the long one ran on alone,
+// one wave a SIMD, for most of its time (2,048 tokens, 8 key/value heads: 70 us, now 5x).
+constexpr int CTA_SETS = 2 * CTA_STAGES * STAGE_CHUNKS * 16 <= 144 * 1024 ? 2 : 1;
+constexpr int CTA_THREADS = 256 * CTA_SETS;
+constexpr int CTA_RING_BYTES = CTA_SETS * CTA_STAGES * STAGE_CHUNKS * 16;
+constexpr int CTA_COMBINE_BYTES = CTA_SETS == 2 ? 4 * ROWS * (HD + 4 + 2) * 4 : 0;
+constexpr int CTA_LDS_BYTES = CTA_RING_BYTES > CTA_COMBINE_BYTES ? CTA_RING_BYTES : CTA_COMBINE_BYTES;
+static_assert(CTA_LDS_BYTES <= 160 * 1024, "the tiles do not fit into LDS");
 
-__global__ __launch_bounds__(256, 2) void k_attn_cta(AttnArgs a) {
-    extern __shared__ uint4 lds[];                          // [CTA_STAGES][STAGE_CHUNKS]
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int kvh = blockIdx.y;
-    // Items come longest first.  Workgroups are handed to the compute units in the order of
-    // their numbers, two to a unit at this kernel's size, the second 256 numbers later.  When
-    // all of them run at once (at most 512), the upper half of the key/value heads takes the
-    // items in reverse, so that a unit's two workgroups are a long one and a short one (a
-    // causal prompt's blocks see 1 to n keys); with more, the longest must simply start first.
-    const bool pair_up = gridDim.x * gridDim.y <= 512 && blockIdx.y * 2 >= gridDim.y;
-    const int item_no = pair_up ? a.n_cta_items - 1 - (int)blockIdx.x : (int)blockIdx.x;
+__global__ __launch_bounds__(CTA_THREADS, CTA_SETS == 2 ? 1 : 2) void k_attn_cta(AttnArgs a) {
+    extern __shared__ uint4 lds_all[];                      // [CTA_SETS][CTA_STAGES][STAGE_CHUNKS]
+    const int tid = threadIdx.x & 255, lane = tid & 63, wave = tid >> 6;       // within the set
+    const int set = __builtin_amdgcn_readfirstlane((int)threadIdx.x >> 8);
+    uint4* lds = lds_all + set * CTA_STAGES * STAGE_CHUNKS;
+    // Items come longest first, and workgroups start in the order of their numbers: an item's
+    // key/value heads are numbered side by side, so that the longest items of every head start
+    // first.  (With 8 key/value heads a head's items then also run on one of the 8 dies and share
+    // its L2.)
+    // (One set, two workgroups to a unit, the second 256 numbers later: when all run at once, the
+    // second half of the numbers is taken in reverse, so that a unit gets a long and a short item.)
+    unsigned wg = blockIdx.x;
+    if (CTA_SETS == 1 && gridDim.x <= 512 && wg >= (gridDim.x + 1) / 2) wg = gridDim.x - 1 - (wg - (gridDim.x + 1) / 2);
+    const int item_no = (int)(wg / (unsigned)a.Hk);
+    const int kvh = (int)wg - item_no * a.Hk;
     const int* it = a.cta_items + (size_t)item_no * ITEM_INTS;
-    const int req = it[0], row0 = it[1] + wave * ROWS, kbeg = it[2], kend = it[3];
+    const int req = it[0], row0 = it[1] + wave * ROWS;
     const int slot = it[4] < 0 ? -1 : it[4] + wave;
     const int q0 = it[5], q_len = it[6], start = it[7];
+    // the set's share of the item's keys; both sets go through the loop as often as the first
+    const int nt_item = (it[3] - it[2] + 31) >> 5;
+    const int nt_first = CTA_SETS == 2 ? (nt_item + 1) >> 1 : nt_item;
+    const int kbeg = it[2] + set * nt_first * 32;
+    const int kend = (set == 0 && CTA_SETS == 2 && it[2] + nt_first * 32 < it[3]) ? it[2] + nt_first * 32 : it[3];
     const int G = a.H / a.Hk;
     const int lr = lane & 31, lg = lane >> 5;
     const int seq_len = start + q_len;
@@ -273,7 +293,7 @@ __global__ __launch_bounds__(256, 2) void k_attn_cta(AttnArgs a) {
         my_page = bt[in ? pi : 0];
         my_page = in ? my_page : -1;
     }
-    const int nt = (kend - kbeg + 31) >> 5;
+    const int nt = kend > kbeg ? (kend - kbeg + 31) >> 5 : 0;
     // a tile lies within one page (pages hold at least 32 positions, tiles begin at multiples of 32)
 #define CTA_ISSUE(TI)                                                                                    \
     {                                                                                                    \
@@ -330,7 +350,7 @@ __global__ __launch_bounds__(256, 2) void k_attn_cta(AttnArgs a) {
     static_assert(CTA_STAGES % 2 == 0 && CTA_LOADS * 2 < 64, "the tiles in LDS come in pairs");
 #pragma unroll
     for (int st = 0; st < CTA_STAGES - 2; ++st) CTA_ISSUE(st)
-    for (int ti = 0; ti < nt; ++ti) {
+    for (int ti = 0; ti < nt_first; ++ti) {
         if ((ti & 1) == 0) {
             // tiles ti and ti+1 have landed when at most the CTA_STAGES-4 younger ones are on their way
             wait_vmcnt<CTA_LOADS * (CTA_STAGES - 4)>();
@@ -339,7 +359,7 @@ __global__ __launch_bounds__(256, 2) void k_attn_cta(AttnArgs a) {
             CTA_ISSUE(ti + CTA_STAGES - 1)
         }
         const int kt = kbeg + ti * 32;
-        if (kt > pos_max || kt + 32 <= lo_min) continue; // nothing here for this wave's rows
+        if (ti >= nt || kt > pos_max || kt + 32 <= lo_min) continue; // nothing here for this wave's rows
         const uint4* Ks = lds + (ti % CTA_STAGES) * STAGE_CHUNKS;
         const uint4* Vs = Ks + NKC;
         uint4 kf[KD], vf[2][DB];
@@ -389,6 +409,50 @@ __global__ __launch_bounds__(256, 2) void k_attn_cta(AttnArgs a) {
     wait_vmcnt<0>();                                     // the trailing copies of zeros
     l += __shfl_xor(l, 32, 64);                          // the row's sum from its two lanes
 
+    if (CTA_SETS == 2) {
+        // the second set hands its rows' maxima, sums and unnormalised outputs to the first
+        __syncthreads();                                 // the rings are free
+        float* xo = reinterpret_cast<float*>(lds_all);   // [4 waves][ROWS][HD + 4]
+        float* xml = xo + 4 * ROWS * (HD + 4);           // [4 waves][ROWS][2]
+        float* mine = xo + (wave * ROWS + lr) * (HD + 4);
+        if (set == 1) {
+#pragma unroll
+            for (int d = 0; d < DB; ++d)
+#pragma unroll
+                for (int e4 = 0; e4 < 4; ++e4) {
+                    const int dd = d * 32 + e4 * 8 + lg * 4;
+                    if (dd < HD)
+                        *reinterpret_cast<float4*>(mine + dd) = make_float4(o[d][e4 * 4 + 0], o[d][e4 * 4 + 1],
+                                                                            o[d][e4 * 4 + 2], o[d][e4 * 4 + 3]);
+                }
+            if (lg == 0) {
+                xml[(wave * ROWS + lr) * 2] = m;
+                xml[(wave * ROWS + lr) * 2 + 1] = l;
+            }
+        }
+        __syncthreads();
+        if (set == 1) return;
+        const float m1 = xml[(wave * ROWS + lr) * 2], l1 = xml[(wave * ROWS + lr) * 2 + 1];
+        const float mn = fmaxf(m, m1);
+        const float f0 = m == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(m - mn);
+        const float f1 = m1 == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(m1 - mn);
+        l = l * f0 + l1 * f1;
+        m = mn;
+#pragma unroll
+        for (int d = 0; d < DB; ++d)
+#pragma unroll
+            for (int e4 = 0; e4 < 4; ++e4) {
+                const int dd = d * 32 + e4 * 8 + lg * 4;
+                if (dd < HD) {
+                    const float4 x = *reinterpret_cast<const float4*>(mine + dd);
+                    o[d][e4 * 4 + 0] = o[d][e4 * 4 + 0] * f0 + x.x * f1;
+                    o[d][e4 * 4 + 1] = o[d][e4 * 4 + 1] * f0 + x.y * f1;
+                    o[d][e4 * 4 + 2] = o[d][e4 * 4 + 2] * f0 + x.z * f1;
+                    o[d][e4 * 4 + 3] = o[d][e4 * 4 + 3] * f0 + x.w * f1;
+                }
+            }
+    }
+
     ATTN_WRITE_OUT(slot)
 }
 
@@ -416,8 +480,14 @@ static_assert(STREAM_LDS_BYTES <= 160 * 1024, "the rings do not fit into LDS");
 __global__ __launch_bounds__(64 * STREAM_WAVES) void k_attn_stream(AttnArgs a) {
     extern __shared__ uint4 lds[];
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int kvh = blockIdx.y;
-    const int* it = a.items + (size_t)blockIdx.x * ITEM_INTS;
+    // Workgroups start in the order of their numbers and the items come longest first: an item's
+    // key/value heads are numbered side by side, so that the longest items of every head start
+    // first and the shortest fill the end (numbered head by head, the last head's longest item
+    // started among the last and ran on alone: 32 requests of 192 to 2,176 keys with 32 key/value
+    // heads took 143 us, now 127).
+    const int item_no = (int)(blockIdx.x / (unsigned)a.Hk);
+    const int kvh = (int)blockIdx.x - item_no * a.Hk;
+    const int* it = a.items + (size_t)item_no * ITEM_INTS;
     const int req = it[0], row0 = it[1], kbeg = it[2], kend = it[3], slot = it[4];
     const int q0 = it[5], q_len = it[6], start = it[7];
     const int G = a.H / a.Hk;
@@ -720,6 +790,7 @@ extern "C" int xr_attention_mfma(void* out, const void* q, const void* k_cache, 
     XR_REQUIRE(shift >= 4, "attention: the MFMA kernel needs a page size that is a power of two of at least 16, got %d", page_size);
     XR_REQUIRE(window >= 0, "attention: window %d is negative", window);
     XR_REQUIRE(n_items >= 0 && n_jobs >= 0 && n_cta_items >= 0, "attention: negative work counts");
+    XR_REQUIRE((long long)n_cta_items * Hk < (1LL << 31) && (long long)n_items * Hk < (1LL << 31), "attention: %d items of %d key/value heads are more workgroups than a launch takes", n_items + n_cta_items, Hk);
     XR_REQUIRE(n_cta_items == 0 || page_size >= 32, "attention: 128-row items need pages of at least 32 positions, got %d", page_size);
     XR_REQUIRE(n_jobs == 0 || (part_o && part_ml && jobs), "attention: split work without partial buffers");
     if (n_items + n_cta_items == 0) return XR_OK;
@@ -730,7 +801,7 @@ extern "C" int xr_attention_mfma(void* out, const void* q, const void* k_cache, 
     a.part_o = part_o; a.part_ml = part_ml; a.n_items = n_items; a.H = H; a.Hk = Hk;
     a.page_shift = shift; a.page_mask = page_size - 1; a.page_size = page_size; a.scale = scale; a.window = window;
     if (n_cta_items > 0) {
-        constexpr int smem = CTA_STAGES * STAGE_CHUNKS * 16;
+        constexpr int smem = CTA_LDS_BYTES;
         static bool attr_set = false;
         if (!attr_set) {
             hipError_t e = hipFuncSetAttribute((const void*)k_attn_cta, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
@@ -738,7 +809,7 @@ extern "C" int xr_attention_mfma(void* out, const void* q, const void* k_cache, 
             XR_REQUIRE(e == hipSuccess, "attention: %d bytes of LDS refused: %s", smem, hipGetErrorString(e));
             attr_set = true;
         }
-        k_attn_cta<<<dim3(n_cta_items, Hk), 256, smem, stream>>>(a);
+        k_attn_cta<<<dim3((unsigned)n_cta_items * (unsigned)Hk), CTA_THREADS, smem, stream>>>(a);
         XR_CHECK_LAUNCH("attention_cta");
     }
     if (n_items > 0) {
@@ -750,7 +821,7 @@ extern "C" int xr_attention_mfma(void* out, const void* q, const void* k_cache, 
             XR_REQUIRE(e == hipSuccess, "attention: %d bytes of LDS refused: %s", STREAM_LDS_BYTES, hipGetErrorString(e));
             attr_set = true;
         }
-        k_attn_stream<<<dim3(n_items, Hk), 64 * STREAM_WAVES, STREAM_LDS_BYTES, stream>>>(a);
+        k_attn_stream<<<dim3((unsigned)n_items * (unsigned)Hk), 64 * STREAM_WAVES, STREAM_LDS_BYTES, stream>>>(a);
         XR_CHECK_LAUNCH("attention_stream");
     }
     if (n_jobs > 0) {
