@@ -89,6 +89,15 @@ __device__ inline float max3(float a, float b, float c) {
     asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
     return r;
 }
+// the larger of a lane's value and that of the lane 32 places away, in both lanes: one swap of
+// register halves between lanes (gfx950) and one maximum, where an exchange through the LDS
+// crossbar made every tile's softmax wait for its round trip
+__device__ inline float max_across_halves(float x) {
+    const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    float o;
+    asm("v_max_f32 %0, %1, %2" : "=v"(o) : "v"(__uint_as_float(r[0])), "v"(__uint_as_float(r[1])));
+    return o;
+}
 #define MAX_SLACK 8.0f
 #define ATTN_SOFTMAX_STEP(KT, KEND)                                                                  \
         if ((KT) + 32 <= (KEND) && (KT) + 31 <= pos_min && (KT) >= lo_max) {                             \
@@ -96,7 +105,7 @@ __device__ inline float max3(float a, float b, float c) {
 _Pragma("unroll")                                                                                        \
             for (int e = 3; e < 15; e += 2) mt = max3(mt, s[e], s[e + 1]);                               \
             mt = fmaxf(mt, s[15]);                                                                       \
-            mt = fmaxf(mt, __shfl_xor(mt, 32, 64));                                                      \
+            mt = max_across_halves(mt);                                                                  \
             const float mn = mt * c2 > m + MAX_SLACK ? mt * c2 : m;                                      \
             corr = __builtin_amdgcn_exp2f(m - mn);                                                       \
             float rs = 0.f;                                                                              \
@@ -116,7 +125,7 @@ _Pragma("unroll")                                                               
                 p[e] = ok ? s[e] * c2 : -INFINITY;                                                       \
                 mt = fmaxf(mt, p[e]);                                                                    \
             }                                                                                            \
-            mt = fmaxf(mt, __shfl_xor(mt, 32, 64));                                                      \
+            mt = max_across_halves(mt);                                                                  \
             const float mn = mt > m + MAX_SLACK ? mt : m;                                                \
             const float mu = mn == -INFINITY ? 0.f : mn;                                                 \
             corr = __builtin_amdgcn_exp2f(m - mu);                                                       \
