@@ -308,10 +308,13 @@ def main():
         points[f"prefill_{ctx_max}_in_2048_portions"] = round(ctx_max / long_s, 1)
         log(f"prefill of {ctx_max} tokens in portions of 2048: {long_s * 1e3:.1f} ms, {ctx_max / long_s:.0f} tok/s")
     if args.mixed:
-        n_prompt, n_dec, secs, n_steps = measure_mixed(runner, cfg, args.mixed, 128, seed=9)
-        log(f"mixed: {args.mixed} requests, {n_prompt} prompt + {n_dec} decoded tokens in {secs:.2f} s "
-            f"({n_steps} steps): {(n_prompt + n_dec) / secs:.0f} tok/s in all, {n_dec / secs:.0f} decoded tok/s")
-        points["mixed_total_tok_s"] = round((n_prompt + n_dec) / secs, 1)
+        # the workload twice: the first pass also records the decode graphs of its batch sizes (as the
+        # warm-up steps do for the decode figures), the second is the figure; both are reported
+        for name in ("mixed_first_pass_tok_s", "mixed_total_tok_s"):
+            n_prompt, n_dec, secs, n_steps = measure_mixed(runner, cfg, args.mixed, 128, seed=9)
+            log(f"mixed ({name}): {args.mixed} requests, {n_prompt} prompt + {n_dec} decoded tokens in {secs:.3f} s "
+                f"({n_steps} steps): {(n_prompt + n_dec) / secs:.0f} tok/s in all, {n_dec / secs:.0f} decoded tok/s")
+            points[name] = round((n_prompt + n_dec) / secs, 1)
     line = {
         "metric": f"decode tokens/s, {shape_name}, batch {B}, {P}-token prompts (random weights)",
         "value": round(tps, 1), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,

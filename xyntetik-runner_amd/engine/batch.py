@@ -47,7 +47,7 @@ ATTN_CTA_ROWS = 128     # rows of an item that a whole workgroup takes
 ATTN_CTA_MIN_ROWS = 64  # a request brings at least this many rows to be served by workgroups
 ATTN_STREAM_SLOTS = 256 # workgroups of the streaming kernel that run at a time (one a compute unit)
 ATTN_MIN_RANGE = 4      # tiles: the shortest key range worth a workgroup
-ATTN_CTA_FILL = 256     # 128-row items (times key/value heads) that give every compute unit one
+ATTN_CTA_FILL = 256     # 128-row items (times key/value heads) that give every compute unit one workgroup
 
 
 def key_ranges(tiles: int, share: float) -> int:
@@ -102,15 +102,17 @@ def plan_attention(starts, q_lens, group_size: int, window: Optional[int], n_kv_
     if cta_blocks:
         chunk = cta_tiles
         if chunk is None:
-            # Whole blocks when there is one for every compute unit: the merge of split blocks
-            # costs more than the idle end of a step whose last rows see the most keys
-            # (2048 tokens, 8 key/value heads: 102 us whole, 96 us + 19 us of merging split).
-            # Fewer blocks are cut into about as many parts as fill the chip once.
-            if len(cta_blocks) * n_kv_heads >= ATTN_CTA_FILL:
+            # A workgroup (two sets of four waves) fills a compute unit.  Whole blocks when they give
+            # at least half the units one each: the merge of split blocks costs more than the units
+            # left idle (512 tokens after 4,096, 8 key/value heads: 86 us whole, 86 us in ranges of
+            # 32 tiles, 101 us in ranges of 16; 512 tokens from 0: 17 us whole, 26 us split).
+            # Fewer blocks are cut into about as many ranges as there are units (128 tokens after
+            # 8,000: 145 us whole, 44 us in ranges of 32 tiles, 58 us in ranges of 16).
+            if len(cta_blocks) * n_kv_heads >= ATTN_CTA_FILL // 2:
                 chunk = 1 << 30
             else:
                 work = sum(blk[4] for blk in cta_blocks)
-                chunk = max(8, -(-work * n_kv_heads // (2 * ATTN_CTA_FILL)))
+                chunk = max(8, -(-work * n_kv_heads // ATTN_CTA_FILL))
         for b, row0, lo, hi, tiles in cta_blocks:
             parts = -(-tiles // chunk)
             if parts <= 1:
