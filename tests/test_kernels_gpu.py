@@ -751,6 +751,35 @@ def test_attention_finds_one_far_key(ops, dt, far):
     assert rel(got.cpu().reshape(H, D), want) < (1e-5 if dt == "float32" else 1e-2)
 
 
+@pytest.mark.parametrize("start,far", [(0, 3), (32, 5), (32, 40), (64, 10), (64, 50), (64, 70), (224, 100), (224, 140),
+                                        (230, 127), (230, 128), (2000, 1023), (2000, 1024), (2000, 1999)])
+def test_attention_two_wave_sets_share_an_item(ops, start, far):
+    """A 128-row item's tiles go half to one set of waves and half to another, whose results are
+    combined at the end.  One key is made to stand out, in the first half, in the second, at the
+    edge between them, with one to 64 tiles an item (the second set has nothing to do with one
+    tile) and a last tile that is not full: every row that may see the key must return its value."""
+    H, Hk, D, ps, n_new = 4, 1, 128, 64, 38          # 152 rows: one item of 128 rows and one of 24
+    n = start + n_new
+    torch.manual_seed(start * 7 + far)
+    tables, n_pages = scatter_pages([n], ps, far)
+    k = torch.randn(n, Hk, D) * 0.1
+    v = torch.randn(n, Hk, D)
+    q = torch.randn(n_new, H, D) * 0.1 + 4.0
+    k[far] += 4.0
+    kc, vc = fill_cache([k], [v], tables, n_pages, ps, torch.bfloat16)
+    ctx = FakeCtx([start], [n_new], tables, ps, cta_tiles=1000)
+    plan = ctx.attention_plan(0, H // Hk, None, Hk, ps)
+    assert plan.n_cta_items == 2 and plan.n_jobs == 0
+    got = ops.attention(q.bfloat16().to(DEV).reshape(n_new, H * D), kc, vc, ctx, 0, H, Hk, D, ps, 1 / math.sqrt(D))
+    got = got.cpu().reshape(n_new, H, D).float()
+    assert torch.isfinite(got).all()
+    want = ref_attention(q.bfloat16().float(), [k.bfloat16().float()], [v.bfloat16().float()], [start], [n_new], 1 / math.sqrt(D), None)
+    err = (got.double() - want).abs().amax(dim=(1, 2)) / want.abs().amax()
+    assert err.max() < 1.2e-2, f"token {int(err.argmax())}: {float(err.max())}"
+    sees = [t for t in range(n_new) if start + t >= far]
+    assert sees and rel(got[sees], v.bfloat16().float()[far].expand(len(sees), H, D)) < 1e-2
+
+
 @pytest.mark.parametrize("dt", ["float32", "bfloat16"])
 def test_attention_window_edge(ops, dt):
     """The key just outside the window is made huge: it must not be seen; the one just inside must."""
