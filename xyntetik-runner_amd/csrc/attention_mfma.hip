@@ -181,8 +181,9 @@ _Pragma("unroll")                                                               
     }
 
 // ------------------------------------------------------------------------------ workgroup kernel
-// Long prompt portions: a workgroup of 4 waves takes 128 consecutive rows of one request and
-// key/value head (wave w the rows row0 + 32 w ..) and a range of keys.  The K tile
+// Long prompt portions: a set of 4 waves takes 128 consecutive rows of one request and
+// key/value head (wave w the rows row0 + 32 w ..) and a range of keys (a workgroup is one such
+// set, or two that halve the range between them: CTA_SETS below).  The K tile
 // [32 keys][HD] and the V^T tile [HD][32 keys] are copied once into LDS for all four waves,
 // by asynchronous copies, two tiles at a time into the places of the two tiles before the ones
 // being worked on (4 tiles in LDS; measured at head size 128, a prompt of 2,048 tokens: a barrier
