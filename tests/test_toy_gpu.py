@@ -288,16 +288,16 @@ def test_windowed_decoding_through_captured_steps(tmp_path, dtype):
     try:
         d = write_random_model(TOYW_CONFIG, str(tmp_path / "toyw"), seed=6, std=0.08, norm_jitter=0.1)
         cfg, w = P.load_folder(d)
-        runner = ModelRunner.from_folder(d, dtype=dtype, max_tokens=512, page_size=16, max_requests=2)
+        runner = ModelRunner.from_folder(d, dtype=dtype, max_tokens=640, page_size=16, max_requests=2)
         assert runner.graphs.usable and [g.spec.window for g in runner.manager.groups] == [40, None]
         for lc in runner.storage.layers:
             lc.k.fill_(float("nan")); lc.v.fill_(float("nan"))
-        reqs = {"a": prompt_ids(200, cfg["vocab_size"], 41), "b": prompt_ids(170, cfg["vocab_size"], 42)}
+        reqs = {"a": prompt_ids(300, cfg["vocab_size"], 41), "b": prompt_ids(170, cfg["vocab_size"], 42)}
         want = {k: plain_toy_window(cfg, w, v) for k, v in reqs.items()}
-        n0 = {"a": 30, "b": 7}
+        n0 = {"a": 130, "b": 7}
         got = {k: [] for k in reqs}
         out = runner.step([StepEntry(k, reqs[k][:n0[k]], list(range(n0[k]))) for k in reqs]).cpu().numpy()
-        got["a"].append(out[:30]); got["b"].append(out[30:])
+        got["a"].append(out[:130]); got["b"].append(out[130:])
         fewest = 99
         for i in range(160):
             entries = [StepEntry(k, [reqs[k][n0[k] + i]], [0]) for k in reqs]
@@ -309,6 +309,10 @@ def test_windowed_decoding_through_captured_steps(tmp_path, dtype):
             fewest = min(fewest, sum(p >= 0 for p in tabs[0]))
             assert sum(p >= 0 for p in tabs[0]) <= 40 // 16 + 2 and all(p >= 0 for p in tabs[1])
         assert runner.graphs.replays >= 150 and fewest <= 4
+        if dtype == "bfloat16":
+            # the windowed layer's work list has fewer key ranges a request than the other layer's
+            per_plan = [{key[1]: n for key, n in ctx._plan_splits.items()} for ctx, _, _ in runner.graphs.graphs.values()]
+            assert any(sp[40] < sp[None] for sp in per_plan), per_plan
         assert -1 in runner.manager.get("a").tables[0]           # pages were given back while it decoded
         tol = (2e-5, 2e-6) if dtype == "float32" else (2e-2, 3e-3)
         for k in reqs:

@@ -49,8 +49,14 @@ class StaticDecodeContext:
     """A ``StepContext`` for one token per request whose device arrays never move."""
 
     def __init__(self, ops, device, batch_cap: int, n_splits: int, table_widths: List[int],
-                 windowed: Optional[List[bool]] = None):
+                 windowed: Optional[List[bool]] = None, max_tiles: Optional[int] = None):
+        """``n_splits``: the most key ranges a request is cut into; ``max_tiles``: the longest request's
+        tiles when the context is made.  Every attention plan (group size, window, key/value heads)
+        gets a number of key ranges of its own from these: a windowed layer, or one with more
+        key/value heads, needs fewer ranges to fill the chip than the bucket's longest request
+        with the fewest heads."""
         self.ops, self.device = ops, device
+        self.max_tiles = max_tiles
         # groups whose requests give pages back while they live (their table rows are rewritten every step)
         self.windowed = list(windowed) if windowed is not None else [True] * len(table_widths)
         self.B = self.T = batch_cap
@@ -66,13 +72,14 @@ class StaticDecodeContext:
         self._plan_keys: List[Tuple[int, Optional[int], int]] = []
         self._plans: Dict[Tuple[int, Optional[int], int], AttentionPlan] = {}
         self._plan_off: Dict[Tuple[int, Optional[int], int], int] = {}
+        self._plan_splits: Dict[Tuple[int, Optional[int], int], int] = {}
         self._alloc()
         self.fresh_slots_host: List[int] = []
         self._copied = None
 
     def _alloc(self) -> None:
-        B, S = self.B, self.S
-        n_plan = len(self._plan_keys) * (B * S * 8 + B * 7)
+        B = self.B
+        n_plan = sum(B * self._plan_splits[k] * 8 + B * 7 for k in self._plan_keys)
         offs = np.concatenate([[0], np.cumsum(self._sizes)]).astype(np.int64)
         total = int(offs[-1]) + n_plan
         self._offs = offs
@@ -91,6 +98,7 @@ class StaticDecodeContext:
         self._tables = [d[o[9 + g]:o[10 + g]].view(B, w) for g, w in enumerate(self.table_width)]
         base = int(offs[-1])
         for k in self._plan_keys:
+            S = self._plan_splits[k]
             self._plan_off[k] = base
             items = d[base:base + B * S * 8]
             jobs = d[base + B * S * 8:base + B * S * 8 + B * 7]
@@ -107,6 +115,10 @@ class StaticDecodeContext:
         if key not in self._plans:
             if torch.cuda.is_current_stream_capturing():
                 raise RuntimeError("an attention plan was first asked for during graph capture")
+            tiles = self.max_tiles
+            if tiles is not None and window:
+                tiles = min(tiles, -(-window // ATTN_TILE) + 1)
+            self._plan_splits[key] = self.S if tiles is None else min(self.S, splits_for(self.B, tiles, n_kv_heads))
             self._plan_keys.append(key)
             self._alloc()
             self.fill(*self._last)
@@ -172,7 +184,7 @@ class StaticDecodeContext:
 
     def _fill_plan(self, h, base: int, key, starts) -> None:
         group_size, window, _ = key
-        B, S = self.B, self.S
+        B, S = self.B, self._plan_splits[key]
         items = h[base:base + B * S * 8].reshape(B, S, 8)
         jobs = h[base + B * S * 8:base + B * S * 8 + B * 7].reshape(B, 7)
         hi = starts.astype(np.int64) + 1                          # keys [lo, hi)
@@ -215,7 +227,9 @@ class DecodeGraphs:
         kv, st, _ = runner.model.cache_needs()
         # state slots are served eagerly, and so are parts that look at their data on the host
         self.usable = not any(s is not None for s in st) and runner.model.capturable()
-        self.kv_heads = max((k.num_kv_heads for k in kv if k is not None), default=1)
+        # the bucket's number of key ranges is that of the group with the fewest key/value heads
+        # (the one that needs most ranges to fill the chip); every plan then takes what it needs
+        self.kv_heads = min((k.num_kv_heads for k in kv if k is not None), default=1)
         self.replays = 0
         self.captures = 0
 
@@ -244,7 +258,8 @@ class DecodeGraphs:
             return logits[:n]
         # first time: run the step eagerly on the static context, then record it for later
         ctx = StaticDecodeContext(r.ops, r.device, cap, S, width,
-                                  windowed=[g.spec.window is not None for g in r.manager.groups])
+                                  windowed=[g.spec.window is not None for g in r.manager.groups],
+                                  max_tiles=-(-max_len // ATTN_TILE))
         ctx.fill(entries, rcs, token_source)
         x = r.model.forward(ctx, r.storage.layers)
         out = r.model.logits(ctx, x, ctx.want_rows)
