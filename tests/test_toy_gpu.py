@@ -45,13 +45,15 @@ def register_toy():
 
         def forward(self, ctx, cache, h):
             u = ctx.ops.linear(h, self.w_in, out_dtype=torch.float32)            # the framework's kernels
-            ys, r = [], 0
-            for slot, n in zip(ctx.slots_host, ctx.q_lens):                       # the scan itself: plain torch
-                s = cache.state[slot]
+            slots = ctx.slots.long()            # on the device: nothing here looks at data on the host,
+            ys, r = [], 0                       # so decode steps of this mixer can be recorded as graphs
+            for b, n in enumerate(ctx.q_lens):                                    # the scan itself: plain torch
+                row = slots[b:b + 1]
+                s = cache.state.index_select(0, row)[0]
                 for i in range(n):
                     s = self.decay * s + (1 - self.decay) * u[r + i]
                     ys.append(s)
-                cache.state[slot] = s
+                cache.state.index_copy_(0, row, s[None])
                 r += n
             y = torch.stack(ys).to(h.dtype)
             return ctx.ops.linear(y, self.w_out)
@@ -166,11 +168,11 @@ def test_toy_steps_like_its_plain_counterpart(toy, dtype):
     from xyntetik_runner_amd.engine import ModelRunner, StepEntry
     d, cfg, w = toy
     runner = ModelRunner.from_folder(d, dtype=dtype, max_tokens=192, page_size=4, max_requests=3)
-    assert runner.graphs is not None and not runner.graphs.usable               # state: decode steps run eagerly
+    assert runner.graphs is not None and runner.graphs.usable
     assert len(runner.manager.groups) == 1 and runner.manager.groups[0].spec.window == 6
     assert runner.storage.layers[3].k is runner.storage.layers[0].k and not runner.storage.layers[3].owns
     assert runner.storage.layers[2].k is not runner.storage.layers[0].k
-    assert runner.storage.layers[1].state.shape == (3, 20) and runner.storage.layers[1].k is None
+    assert runner.storage.layers[1].state.shape == (3 + 1, 20) and runner.storage.layers[1].k is None   # the last row is nobody's
     reqs = {f"r{i}": prompt_ids(n, 101, 30 + i) for i, n in enumerate([37, 9, 22, 50])}
     want = {k: plain_toy(cfg, w, v) for k, v in reqs.items()}
     got = {k: [] for k in reqs}
@@ -208,6 +210,47 @@ def test_toy_steps_like_its_plain_counterpart(toy, dtype):
     for rid in reqs:
         mx, mean = logit_error(np.concatenate(got[rid]), want[rid])
         assert mx <= tol[0] and mean <= tol[1], (rid, mx, mean)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_toy_state_through_recorded_decode_steps(toy, dtype):
+    """Three requests decode one token a step: the steps are recorded as graphs (a bucket of four
+    rows, so one row pads the batch and writes the state row that is nobody's), the mixer's state
+    rows are found by the slots on the device, and a request that begins in such a step (its
+    prompt is one token) starts from zeroed state although every row held NaN before."""
+    from xyntetik_runner_amd.engine import ModelRunner, StepEntry
+    d, cfg, w = toy
+    runner = ModelRunner.from_folder(d, dtype=dtype, max_tokens=256, page_size=4, max_requests=3)
+    for lc in runner.storage.layers:
+        if lc.state is not None:
+            lc.state.fill_(float("nan"))
+        if lc.k is not None and lc.owns:
+            lc.k.fill_(float("nan")); lc.v.fill_(float("nan"))
+    reqs = {f"r{i}": prompt_ids(n, 101, 60 + i) for i, n in enumerate([45, 38, 41])}
+    want = {k: plain_toy(cfg, w, v) for k, v in reqs.items()}
+    n0 = {"r0": 5, "r1": 1, "r2": 3}                       # r1 begins inside a recorded step
+    got = {k: [] for k in reqs}
+    first = [k for k in reqs if n0[k] > 1]
+    out = runner.step([StepEntry(k, reqs[k][:n0[k]], list(range(n0[k]))) for k in first]).cpu().numpy()
+    r = 0
+    for k in first:
+        got[k].append(out[r:r + n0[k]]); r += n0[k]
+    prog = {k: (n0[k] if k in first else 0) for k in reqs}
+    for step in range(36):
+        entries = [StepEntry(k, [reqs[k][prog[k]]], [0]) for k in reqs]
+        out = runner.step(entries).cpu().numpy()
+        for i, k in enumerate(reqs):
+            got[k].append(out[i:i + 1]); prog[k] += 1
+        runner.manager.check()
+    assert runner.graphs.replays >= 30
+    null_row = runner.storage.layers[1].state[runner.storage.null_slot]
+    assert not torch.isnan(runner.storage.layers[1].state[:3]).any() and null_row.shape == (20,)
+    tol = (2e-5, 2e-6) if dtype == "float32" else (2e-2, 3e-3)
+    for k in reqs:
+        rows = np.concatenate(got[k])
+        assert np.isfinite(rows).all()
+        mx, mean = logit_error(rows, want[k][:len(rows)])
+        assert mx <= tol[0] and mean <= tol[1], (k, mx, mean)
 
 
 def test_unknown_part_kind_is_a_clear_error():

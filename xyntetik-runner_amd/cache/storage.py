@@ -3,7 +3,8 @@
 For every entry of the run order that owns a cache: keys ``[pages, Hk, page_size, D]``
 and values ``[pages, Hk, D, page_size]`` (values transposed inside a page so that
 attention reads several positions of one channel with one load), in the engine's
-dtype.  For every entry whose mixer has state of fixed size: ``[slots, *shape]``.
+dtype.  For every entry whose mixer has state of fixed size: ``[slots + 1, *shape]``; row
+``null_slot`` (the last) belongs to no request.
 Page 0 is the null page.  Nothing is zeroed when a page changes hands: reads are
 bounded by a request's length, so a page's old contents are never seen.
 """
@@ -25,7 +26,7 @@ class LayerCache:
     owns: bool                 # this entry writes keys and values (False: it reads another entry's)
     k: Optional[torch.Tensor]
     v: Optional[torch.Tensor]
-    state: Optional[torch.Tensor] = None    # [slots, *shape]
+    state: Optional[torch.Tensor] = None    # [slots + 1, *shape]; the last row is nobody's
 
 
 class CacheStorage:
@@ -34,6 +35,7 @@ class CacheStorage:
                  dtype: torch.dtype, device: torch.device):
         """``kv_specs[i]``/``state_specs[i]``/``cache_of[i]`` describe entry ``i`` of the run order."""
         self.page_size, self.n_pages, self.n_slots = page_size, pages_per_group + 1, n_slots
+        self.null_slot = n_slots
         self.group_specs: List[KVSpec] = []
         self.layers: List[LayerCache] = []
         for i, (kv, st) in enumerate(zip(kv_specs, state_specs)):
@@ -61,7 +63,8 @@ class CacheStorage:
                 v = torch.zeros((self.n_pages, kv.num_kv_heads, kv.head_dim, page_size), dtype=dtype, device=device)
             state = None
             if st is not None:
-                state = torch.zeros((n_slots,) + tuple(st.shape), dtype=st.dtype, device=device)
+                # one row more than requests: the last is nobody's (rows that pad a recorded step use it)
+                state = torch.zeros((n_slots + 1,) + tuple(st.shape), dtype=st.dtype, device=device)
             self.layers.append(LayerCache(group, page_size, True, k, v, state))
 
     def bytes_per_token(self) -> int:

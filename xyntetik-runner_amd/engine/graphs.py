@@ -49,7 +49,7 @@ class StaticDecodeContext:
     """A ``StepContext`` for one token per request whose device arrays never move."""
 
     def __init__(self, ops, device, batch_cap: int, n_splits: int, table_widths: List[int],
-                 windowed: Optional[List[bool]] = None, max_tiles: Optional[int] = None):
+                 windowed: Optional[List[bool]] = None, max_tiles: Optional[int] = None, null_slot: int = 0):
         """``n_splits``: the most key ranges a request is cut into; ``max_tiles``: the longest request's
         tiles when the context is made.  Every attention plan (group size, window, key/value heads)
         gets a number of key ranges of its own from these: a windowed layer, or one with more
@@ -57,6 +57,7 @@ class StaticDecodeContext:
         with the fewest heads."""
         self.ops, self.device = ops, device
         self.max_tiles = max_tiles
+        self.null_slot = null_slot          # the state row of the rows that pad the batch
         # groups whose requests give pages back while they live (their table rows are rewritten every step)
         self.windowed = list(windowed) if windowed is not None else [True] * len(table_widths)
         self.B = self.T = batch_cap
@@ -109,6 +110,11 @@ class StaticDecodeContext:
     def block_table(self, group: int) -> torch.Tensor:
         return self._tables[group]
 
+    @property
+    def slots_host(self):
+        raise RuntimeError("this step is recorded as a graph: a part with state reads its rows' slots from "
+                           "ctx.slots (on the device), or sets capturable = False to be run eagerly")
+
     def attention_plan(self, group: int, group_size: int, window: Optional[int], n_kv_heads: int,
                        page_size: int = 64) -> AttentionPlan:
         key = (group_size, window, n_kv_heads)
@@ -143,7 +149,7 @@ class StaticDecodeContext:
         h[o[2]:o[3]] = np.arange(B, dtype=np.int32)
         h[o[3]:o[4]] = np.arange(B + 1, dtype=np.int32)
         h[o[4]:o[5]] = starts + 1
-        slots = np.zeros(B, dtype=np.int32)
+        slots = np.full(B, self.null_slot, dtype=np.int32)
         slots[:n] = [rc.slot for rc in rcs]
         h[o[5]:o[6]] = slots
         h[o[6]:o[7]] = 0
@@ -225,8 +231,8 @@ class DecodeGraphs:
         self.graphs: Dict[Tuple[int, int, int], Tuple[StaticDecodeContext, torch.cuda.CUDAGraph, torch.Tensor]] = {}
         self.pool = None
         kv, st, _ = runner.model.cache_needs()
-        # state slots are served eagerly, and so are parts that look at their data on the host
-        self.usable = not any(s is not None for s in st) and runner.model.capturable()
+        # parts that look at their data on the host are served eagerly (`capturable` False)
+        self.usable = runner.model.capturable()
         # the bucket's number of key ranges is that of the group with the fewest key/value heads
         # (the one that needs most ranges to fill the chip); every plan then takes what it needs
         self.kv_heads = min((k.num_kv_heads for k in kv if k is not None), default=1)
@@ -259,7 +265,7 @@ class DecodeGraphs:
         # first time: run the step eagerly on the static context, then record it for later
         ctx = StaticDecodeContext(r.ops, r.device, cap, S, width,
                                   windowed=[g.spec.window is not None for g in r.manager.groups],
-                                  max_tiles=-(-max_len // ATTN_TILE))
+                                  max_tiles=-(-max_len // ATTN_TILE), null_slot=r.storage.null_slot)
         ctx.fill(entries, rcs, token_source)
         x = r.model.forward(ctx, r.storage.layers)
         out = r.model.logits(ctx, x, ctx.want_rows)

@@ -162,6 +162,7 @@ class ModelRunner:
         for e in entries:
             if any(w != 0 for w in e.want):
                 raise ValueError(f"request {e.req_id!r}: wanted place outside its one token")
+        self._zero_state_rows([rc.slot for rc in rcs if rc.fresh])
         logits = self.graphs.run(entries, rcs, token_source)
         rows = [i for i, e in enumerate(entries) for _ in e.want]
         if not rows:
@@ -171,12 +172,16 @@ class ModelRunner:
         return logits[torch.tensor(rows, dtype=torch.long, device=self.device)]
 
     def _zero_fresh_state(self, ctx: StepContext) -> None:
-        if not ctx.fresh_slots_host:
+        self._zero_state_rows(ctx.fresh_slots_host)
+
+    def _zero_state_rows(self, slots: List[int]) -> None:
+        """The state rows of requests that use their slot for the first time begin at zero."""
+        if not slots:
             return
         rows = None
         for lc in self.storage.layers:
             if lc.state is None:
                 continue
             if rows is None:
-                rows = torch.tensor(ctx.fresh_slots_host, dtype=torch.int32, device=self.device)
-            self.ops.fill_rows_(lc.state, rows, len(ctx.fresh_slots_host), 0)
+                rows = torch.tensor(slots, dtype=torch.int32, device=self.device)
+            self.ops.fill_rows_(lc.state, rows, len(slots), 0)

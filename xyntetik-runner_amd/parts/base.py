@@ -130,6 +130,11 @@ class Mixer(Part):
         return None
 
     def state_spec(self) -> Optional[StateSpec]:
+        """Fixed-size state per request: ``cache.state [slots + 1, *shape]``, request ``b`` of a step
+        owning row ``ctx.slots[b]`` (on the device; zero when the request first uses it).  A mixer
+        that finds its rows through ``ctx.slots`` can be recorded into a HIP graph, where the rows
+        that pad a batch use the last state row, which is nobody's; one that reads the slots on
+        the host (``ctx.slots_host``, absent in a recorded step) sets ``capturable = False``."""
         return None
 
     def forward(self, ctx, cache, h: torch.Tensor) -> torch.Tensor:
