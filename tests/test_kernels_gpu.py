@@ -397,6 +397,31 @@ def test_linear_plain_kernel(ops, M, N, K, dt):
     assert rel(out, base.double() + a.double() @ w.double().T) < 2e-6
 
 
+@pytest.mark.parametrize("M,N,K", [(1, 7, 8), (3, 50, 260), (8, 1000, 4096), (16, 33, 14336), (13, 65, 1028), (2, 128256 // 16, 64)])
+def test_linear_32bit_few_rows(ops, M, N, K):
+    """Up to 16 rows of 32-bit operands take the kernel that streams the weights (a wave 8 weight rows):
+    against the float64 product, with bias, accumulation, a bfloat16 result and rows that are a view
+    of a wider matrix; and a row's result is bit for bit the same whatever rows are beside it."""
+    torch.manual_seed(M * 1000 + N)
+    wide = torch.randn(M, K + 8, device=DEV)
+    a = wide[:, :K]                                   # row stride K + 8
+    w = torch.randn(N, K, device=DEV)
+    b = torch.randn(N, device=DEV)
+    want = a.double() @ w.double().T + b.double()
+    got = ops.linear(a, w, bias=b, out_dtype=torch.float32)
+    assert rel(got, want) < 2e-6
+    base = torch.randn(M, N, device=DEV)
+    out = base.clone()
+    ops.linear(a, w, out=out, accumulate=True)
+    assert rel(out, base.double() + a.double() @ w.double().T) < 2e-6
+    assert rel(ops.linear(a, w, bias=b, out_dtype=torch.bfloat16).float(), want) < 6e-3
+    alone = ops.linear(a[:1].contiguous(), w, bias=b, out_dtype=torch.float32)
+    assert torch.equal(alone[0], got[0])
+    if M < 16:                                        # and whatever kernel instance (1, 4, 8 or 16 rows) serves it
+        more = torch.cat([a, torch.randn(16 - M, K, device=DEV)]).contiguous()
+        assert torch.equal(ops.linear(more, w, bias=b, out_dtype=torch.float32)[:M], got)
+
+
 def test_linear_one_hot_rows_pick_weight_rows(ops):
     """A one-hot input returns the matching weight column: a transposed or mis-strided operand fails."""
     N, K = 96, 64

@@ -83,6 +83,71 @@ __global__ __launch_bounds__(256) void k_gemm_ref(TO* __restrict__ out, const TI
     }
 }
 
+// Up to 16 rows of 32-bit operands (decoded tokens): the product is bound by how fast the weights
+// arrive, and the tile kernel above, 64 weight rows a workgroup, leaves most of the chip idle then
+// (a decode step of the Llama-3.1-8B shape took 136 ms).  Here a wave takes 8 weight rows: a lane
+// sums, for every row of `a` and each of them, the columns 4 l .. 4 l + 3 (mod 256) in ascending
+// order by FMA, and the lanes' sums are added in a fixed tree.  A row's result does not depend
+// on the rows beside it; it differs from the tile kernel's by the order of the sum only.
+template <int MT, typename TO, bool ACC>
+__global__ __launch_bounds__(256) void k_gemv_ref(TO* __restrict__ out, const float* __restrict__ a,
+                                                   const float* __restrict__ w, const float* __restrict__ bias,
+                                                   int M, int N, int K, int lda, int ldo) {
+    constexpr int COLS = 8;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int n0 = (blockIdx.x * 4 + wave) * COLS;
+    if (n0 >= N) return;
+    float acc[COLS][MT];
+#pragma unroll
+    for (int c = 0; c < COLS; ++c)
+#pragma unroll
+        for (int m = 0; m < MT; ++m) acc[c][m] = 0.f;
+    for (int k = lane * 4; k < K; k += 256) {
+        float4 av[MT];
+#pragma unroll
+        for (int m = 0; m < MT; ++m)
+            av[m] = m < M ? *reinterpret_cast<const float4*>(a + (size_t)m * lda + k) : make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+        for (int c = 0; c < COLS; ++c) {
+            const int n = n0 + c;
+            const float4 wv = n < N ? *reinterpret_cast<const float4*>(w + (size_t)n * K + k) : make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+            for (int m = 0; m < MT; ++m) {
+                float t = acc[c][m];
+                t = fmaf(av[m].x, wv.x, t);
+                t = fmaf(av[m].y, wv.y, t);
+                t = fmaf(av[m].z, wv.z, t);
+                t = fmaf(av[m].w, wv.w, t);
+                acc[c][m] = t;
+            }
+        }
+    }
+#pragma unroll
+    for (int c = 0; c < COLS; ++c)
+#pragma unroll
+        for (int m = 0; m < MT; ++m) {
+            float v = acc[c][m];
+#pragma unroll
+            for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+            const int n = n0 + c;
+            if (lane == 0 && m < M && n < N) {
+                if (bias) v += bias[n];
+                const size_t at = (size_t)m * ldo + n;
+                if (ACC) v += ld<TO>(out, at);
+                st<TO>(out, at, v);
+            }
+        }
+}
+
+template <int MT>
+static void launch_gemv_ref(void* out, const float* a, const float* w, const float* bias, int M, int N, int K,
+                            int lda, int ldo, int out_dtype, int accumulate, hipStream_t stream) {
+    const unsigned blocks = (unsigned)((N + 31) / 32);
+    if (out_dtype == XR_BF16) k_gemv_ref<MT, bf16_t, false><<<blocks, 256, 0, stream>>>((bf16_t*)out, a, w, bias, M, N, K, lda, ldo);
+    else if (accumulate) k_gemv_ref<MT, float, true><<<blocks, 256, 0, stream>>>((float*)out, a, w, bias, M, N, K, lda, ldo);
+    else k_gemv_ref<MT, float, false><<<blocks, 256, 0, stream>>>((float*)out, a, w, bias, M, N, K, lda, ldo);
+}
+
 // accumulate != 0: out (float) += product.
 extern "C" int xr_gemm_ref(void* out, const void* a, const void* w, const float* bias, int M, int N, int K,
                            int lda, int ldo, int in_dtype, int out_dtype, int accumulate, hipStream_t stream) {
@@ -90,6 +155,17 @@ extern "C" int xr_gemm_ref(void* out, const void* a, const void* w, const float*
     XR_REQUIRE(lda >= K && ldo >= N, "gemm: row strides lda=%d ldo=%d are shorter than K=%d N=%d", lda, ldo, K, N);
     XR_REQUIRE(!accumulate || out_dtype == XR_F32, "gemm: accumulation needs a 32-bit output");
     if (M == 0) return XR_OK;
+    if (M <= 16 && in_dtype == XR_F32 && (out_dtype == XR_F32 || out_dtype == XR_BF16) && K % 4 == 0 && lda % 4 == 0 &&
+        ((uintptr_t)a % 16) == 0 && ((uintptr_t)w % 16) == 0) {
+        const float* af = (const float*)a;
+        const float* wf = (const float*)w;
+        if (M == 1) launch_gemv_ref<1>(out, af, wf, bias, M, N, K, lda, ldo, out_dtype, accumulate, stream);
+        else if (M <= 4) launch_gemv_ref<4>(out, af, wf, bias, M, N, K, lda, ldo, out_dtype, accumulate, stream);
+        else if (M <= 8) launch_gemv_ref<8>(out, af, wf, bias, M, N, K, lda, ldo, out_dtype, accumulate, stream);
+        else launch_gemv_ref<16>(out, af, wf, bias, M, N, K, lda, ldo, out_dtype, accumulate, stream);
+        XR_CHECK_LAUNCH("gemv_ref");
+        return XR_OK;
+    }
     dim3 grid((N + RBN - 1) / RBN, (M + RBM - 1) / RBM);
 #define G(TI, TO, ACC) k_gemm_ref<TI, TO, ACC><<<grid, 256, 0, stream>>>((TO*)out, (const TI*)a, (const TI*)w, bias, M, N, K, lda, ldo)
     if (in_dtype == XR_F32 && out_dtype == XR_F32) { if (accumulate) G(float, float, true); else G(float, float, false); }
