@@ -2,7 +2,7 @@
 // portions and decoded tokens in one launch.  Compiled once per head size (XR_HEAD_DIM,
 // a multiple of 16 up to 256).
 //
-// The formulas are the reference's (/root/reference/src/model.c:3548-3589: scores (q.k)*scale
+// The formulas are the reference's (src/model.c:3548-3589: scores (q.k)*scale
 // over the keys a position may see, softmax with the maximum taken out, weighted values;
 // window bound :6326); the arrangement is not.  The query rows that share one key/value
 // head -- (token, head-in-group) pairs of one request -- are packed 32 to a block, so the
@@ -21,7 +21,7 @@
 // wants from it: P^T goes from accumulator to operand without leaving the lane.
 // Scores, maxima, sums and the output accumulate in 32-bit; P is rounded to bfloat16
 // for the second product.  Items that cover part of a row block's keys write partial
-// results that k_attn_merge combines (/root/reference/src/kernels.cu:2171-2270 does this
+// results that k_attn_merge combines (src/kernels.cu:2171-2270 does this
 // with 8 fixed slices for decoding).  Page sizes are powers of two from 16; a key that does
 // not exist (past the request's end, or in a page the window has given back) is copied from
 // a block of zeros, and the words of V^T past the end in the last tile are masked on use.
@@ -83,7 +83,13 @@ __device__ inline uint32_t pack2(float lo, float hi) { return pack_bf16x2(lo, hi
 // its output when any row of the wave moves its reference become rare (before, nearly every tile
 // of a few thousand keys paid them).
 // the largest of three in one instruction (fmaxf's promise about signalling NaNs costs a second
-// instruction per maximum; a NaN score makes the row's output NaN either way)
+// instruction per maximum; a NaN score makes the row's output NaN either way).
+// The compiler does not count the wait states an instruction written as assembly owes the matrix
+// unit: the first reader of a product's result must be an instruction of the compiler's own (it
+// then waits until the whole result is written), and `a` must come from such an instruction.  A
+// chain that began with max3 on the accumulator itself read registers the product had not written
+// yet: the reference of the running softmax was then some older maximum, which gives the same
+// quotient, but a rounding that changed from run to run with the timing of the waves.
 __device__ inline float max3(float a, float b, float c) {
     float r;
     asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
@@ -101,10 +107,10 @@ __device__ inline float max_across_halves(float x) {
 #define MAX_SLACK 8.0f
 #define ATTN_SOFTMAX_STEP(KT, KEND)                                                                  \
         if ((KT) + 32 <= (KEND) && (KT) + 31 <= pos_min && (KT) >= lo_max) {                             \
-            float mt = max3(s[0], s[1], s[2]);                                                           \
+            float mt = fmaxf(s[0], s[15]);      /* the compiler's own instruction reads s first */       \
+            mt = max3(mt, s[1], s[2]);                                                                   \
 _Pragma("unroll")                                                                                        \
             for (int e = 3; e < 15; e += 2) mt = max3(mt, s[e], s[e + 1]);                               \
-            mt = fmaxf(mt, s[15]);                                                                       \
             mt = max_across_halves(mt);                                                                  \
             const float mn = mt * c2 > m + MAX_SLACK ? mt * c2 : m;                                      \
             corr = __builtin_amdgcn_exp2f(m - mn);                                                       \
