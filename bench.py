@@ -7,7 +7,7 @@ fraction of the HBM roofline.
 A "step" is one decode step of the engine (schedule, model step, sampling) for a batch of
 8 requests, each with a 2,048-token prompt already in the cache.  One JSON line goes to
 stdout.  The reference's own bench times a 512-token prompt and 128 greedy tokens of one
-sequence and ignores end-of-text while it does (/root/reference/src/main.c:1435-1515).
+sequence and ignores end-of-text while it does (src/main.c:1435-1515).
 """
 import argparse
 import json
@@ -116,8 +116,9 @@ def measure_achievable(runner):
     return n_bytes / (read_ms * 1e-3) / 1e9, 2.0 * M * N * K / (mm_ms * 1e-3)
 
 
-def measure_decode(runner, cfg, batch, prompt_len, steps, warmup, seed):
-    """tokens/s of `steps` decode steps with `batch` requests whose prompts are already cached."""
+def measure_decode(runner, cfg, batch, prompt_len, steps, warmup, seed, alone=False):
+    """tokens/s of `steps` decode steps with `batch` requests whose prompts are already cached;
+    afterwards one more step's logits are checked (`check_decode_logits`)."""
     import numpy as np
     import torch
     from xyntetik_runner_amd.engine import Engine
@@ -145,11 +146,55 @@ def measure_decode(runner, cfg, batch, prompt_len, steps, warmup, seed):
     ctx1 = sum(eng.requests[i].n_tokens for i in ids)
     if ctx1 - ctx0 != batch * steps:
         raise RuntimeError(f"decode batch {batch}: {ctx1 - ctx0} tokens decoded in {steps} steps")
-    for i in ids:
-        eng.scheduler.abort(eng.requests.pop(i))
+    replays = runner.graphs.replays if runner.graphs is not None else 0
+    check = check_decode_logits(runner, eng, ids, batch, alone)
     if runner.graphs is not None:
+        if runner.graphs.replays <= replays:
+            raise RuntimeError(f"decode batch {batch}: the checked step did not go through a recorded graph")
         log(f"  graphs: {runner.graphs.captures} captured, {runner.graphs.replays} replays so far")
-    return batch * steps / dt, dt / steps, (ctx0 + ctx1) / 2
+    return batch * steps / dt, dt / steps, (ctx0 + ctx1) / 2, check
+
+
+def sane_logits(rows, what):
+    """The reference's rule for a run that computed nothing: all-zero logits fail
+    (tests/test_gpu_identity.c:190-201); so do logits that are not finite, and rows that are constant."""
+    import torch
+    if not bool(torch.isfinite(rows).all()):
+        raise RuntimeError(f"{what}: logits are not finite")
+    if bool((rows.abs().amax(dim=-1) == 0).any()) or bool((rows.std(dim=-1) == 0).any()):
+        raise RuntimeError(f"{what}: a row of logits is all zero or all equal")
+
+
+def check_decode_logits(runner, eng, ids, batch, alone):
+    """One more decode step of the timed batch, through the same recorded graph, with its logits
+    looked at: every row finite, not zero, not constant.  With ``alone``, the first request's row is
+    also compared with the same tokens run as a request of its own (its prompt in portions of 2,048,
+    the last token as a decode step of one): (max, mean) difference as fractions of the mean logit
+    range.  Ends the requests."""
+    import torch
+    from xyntetik_runner_amd.engine.batch import StepEntry
+    eng.run_ahead = False
+    eng.step()                       # the step that was queued ahead, if any: now the host knows every token
+    reqs = [eng.requests[i] for i in ids]
+    if any(r.remaining != 1 for r in reqs):
+        raise RuntimeError(f"decode batch {batch}: a request is not decoding")
+    logits = runner.step([StepEntry(r.id, [r.output[-1]], [0]) for r in reqs])
+    sane_logits(logits, f"decode batch {batch}")
+    row = logits[0].clone()
+    tokens = list(reqs[0].prompt) + list(reqs[0].output)
+    for i in ids:
+        eng.abort(i)
+    if not alone:
+        return None
+    for a in range(0, len(tokens) - 1, 2048):
+        runner.step([StepEntry("alone", tokens[a:min(a + 2048, len(tokens) - 1)], [])])
+    single = runner.step([StepEntry("alone", tokens[-1:], [0])])[0]
+    runner.finish("alone")
+    sane_logits(single[None], f"decode batch {batch}, the first request alone")
+    span = float((single.max() - single.min()))
+    d = (row - single).abs()
+    return {"max": round(float(d.max()) / span, 5), "mean": round(float(d.mean()) / span, 6),
+            "same_top": bool(int(row.argmax()) == int(single.argmax()))}
 
 
 def measure_mixed(runner, cfg, n_requests, steps_each, seed):
@@ -170,13 +215,13 @@ def measure_mixed(runner, cfg, n_requests, steps_each, seed):
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     n_steps = 0
+    done = []
     while eng.has_work():
-        eng.step()
+        done += [o.request for o in eng.step() if o.finished]
         n_steps += 1
     torch.cuda.synchronize()
     secs = time.perf_counter() - t0
-    done = [eng.requests.pop(rid) for rid in list(eng.requests)]
-    if any(len(r.output) != steps_each for r in done):
+    if len(done) != n_requests or any(len(r.output) != steps_each for r in done):
         raise RuntimeError("mixed workload: a request ended early")
     return sum(lens), n_requests * steps_each, secs, n_steps
 
@@ -185,8 +230,11 @@ def measure_prefill(runner, cfg, T, repeats, seed):
     import numpy as np
     import torch
     from xyntetik_runner_amd.engine.batch import StepEntry
+    """Seconds for a prompt of T tokens in one step, up to the logits of its last position on the
+    host: the median of ``repeats`` runs after one that is not counted (the reference reports
+    medians, docs/benchmarks.md:16)."""
     rng = np.random.default_rng(seed)
-    best = None
+    times = []
     for r in range(repeats + 1):
         toks = [int(t) for t in rng.integers(0, cfg["vocab_size"], size=T)]
         torch.cuda.synchronize()
@@ -194,14 +242,12 @@ def measure_prefill(runner, cfg, T, repeats, seed):
         out = runner.step([StepEntry(("prefill", r), toks, [T - 1])])
         last = out.cpu()
         dt = time.perf_counter() - t0
-        # the reference's rule for a run that computed nothing: all-zero logits fail
-        # (/root/reference/tests/test_gpu_identity.c:190-201); so do logits that are not finite
-        if not bool(torch.isfinite(last).all()) or float(last.abs().max()) == 0.0 or float(last.std()) == 0.0:
-            raise RuntimeError("prefill: the logits of the prompt's last position are not finite, all zero or all equal")
+        sane_logits(last, "prefill")
         runner.finish(("prefill", r))
         if r > 0:
-            best = dt if best is None else min(best, dt)
-    return best
+            times.append(dt)
+    times.sort()
+    return times[len(times) // 2]
 
 
 def measure_prefill_in_portions(runner, cfg, T, portion, seed):
@@ -237,6 +283,8 @@ def main():
     ap.add_argument("--no-points", action="store_true", help="skip decode at batch 1 and 64")
     ap.add_argument("--dtype", default="bfloat16")
     ap.add_argument("--shape", default="llama-3.1-8b", choices=sorted(SHAPES), help="sizes of the model (same architecture)")
+    ap.add_argument("--record", default="", metavar="FILE",
+                    help="also write the command and the JSON line into FILE (markdown)")
     ap.add_argument("--mixed", type=int, default=0, metavar="N",
                     help="also run N requests with prompts of 128..2048 tokens and 128 decoded tokens each through the scheduler")
     args = ap.parse_args()
@@ -274,30 +322,38 @@ def main():
         log(f"achievable on this GPU: {read_gbs:.0f} GB/s to a kernel that only reads, "
             f"{mm_flops / 1e12:.0f} TFLOP/s bfloat16 on a 8192 x 28672 x 4096 product")
     peak_flops = PEAK["bf16_flops" if args.dtype == "bfloat16" else "fp32_flops"]
-    pre_s = measure_prefill(runner, cfg, 2048, repeats=3, seed=1)
+    pre_s = measure_prefill(runner, cfg, 2048, repeats=5, seed=1)
     pre_rate = prefill_flops(cfg, layers, 2048) / pre_s
-    log(f"prefill 2048 tokens: {pre_s * 1e3:.1f} ms")
+    log(f"prefill 2048 tokens: {pre_s * 1e3:.1f} ms (the median of 5)")
 
     # the decode figure: the median of three repetitions of the whole workload (fresh requests,
     # prompts computed again), as the reference reports a median of its runs
-    # (/root/reference/docs/benchmarks.md:16)
+    # (docs/benchmarks.md:16)
     runs = []
     for rep in range(3):
-        tps, step_s, ctx = measure_decode(runner, cfg, B, P, args.steps, args.warmup, seed=2 + 100 * rep)
+        tps, step_s, ctx, _ = measure_decode(runner, cfg, B, P, args.steps, args.warmup, seed=2 + 100 * rep)
         runs.append((step_s, tps, ctx))
         log(f"decode batch {B}, repetition {rep + 1}: {tps:.1f} tok/s, {step_s * 1e3:.3f} ms/step, "
             f"{decode_bytes(cfg, layers, B, ctx, elt) / step_s / 1e9:.0f} GB/s")
     runs.sort()
     step_s, tps, ctx = runs[1]
     achieved = decode_bytes(cfg, layers, B, ctx, elt) / step_s / 1e9
-    points = {}
+    points, checks = {}, {}
     if not args.no_points:
-        def point(name, b, prompt_len, n, warm, seed):
-            t, sec, c = measure_decode(runner, cfg, b, prompt_len, n, warm, seed=seed)
+        def point(name, b, prompt_len, n, warm, seed, alone=False):
+            t, sec, c, chk = measure_decode(runner, cfg, b, prompt_len, n, warm, seed=seed, alone=alone)
             points[name] = round(t, 1)
             log(f"{name}: {t:.1f} tok/s, {sec * 1e3:.3f} ms/step, {decode_bytes(cfg, layers, b, c, elt) / sec / 1e9:.0f} GB/s")
+            if chk is not None:
+                # one request's logits must not depend on the 63 beside it, beyond the rounding of
+                # bfloat16 operands summed in another order (the reference's bound for two back
+                # ends of one model is a mean of 2e-3 of the logit range, tests/test_gpu_identity.c:50-60)
+                checks[f"{name}_row0_vs_alone"] = chk
+                log(f"{name}: the first request's logits against the same request alone: {chk}")
+                if args.dtype == "bfloat16" and not (chk["mean"] <= 2e-3 and chk["max"] <= 2e-2):
+                    raise RuntimeError(f"{name}: a request's logits in the batch differ from the same request alone: {chk}")
         for b in (1, 64):
-            point(f"decode_b{b}", b, P, max(8, min(args.steps, 64)), min(args.warmup, 8), 3 + b)
+            point(f"decode_b{b}", b, P, max(8, min(args.steps, 64)), min(args.warmup, 8), 3 + b, alone=b == 64)
         # away from the tuned point: contexts at the model's limit, and a prompt of that length in portions
         point(f"decode_b8_ctx{ctx_max}", 8, long_P, long_steps, long_warmup, 21)
         if long_b64:
@@ -330,7 +386,7 @@ def main():
                     "frac": round(pre_rate / peak_flops, 4)},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK["hbm_gbs"], "unit": "GB/s",
                      "frac": round(achieved / PEAK["hbm_gbs"], 4)},
-        "points": points,
+        "points": points, "checks": checks,
         "repetitions_ms_per_step": [round(r[0] * 1e3, 4) for r in runs],
     }
     if read_gbs:
@@ -338,9 +394,16 @@ def main():
         # kernel on one large product, in this very run
         line["roofline"]["measured_peak"] = round(read_gbs, 1)
         line["roofline"]["frac_of_measured"] = round(achieved / read_gbs, 4)
-        line["prefill"]["measured_peak_tflops"] = round(mm_flops / 1e12, 1)
-        line["prefill"]["frac_of_measured"] = round(pre_rate / mm_flops, 4)
-    print(json.dumps(line), flush=True)
+        # no roofline, and it can exceed 1: the step's rate over that of this engine's own matrix
+        # kernel on one large product
+        line["prefill"]["own_gemm_tflops"] = round(mm_flops / 1e12, 1)
+        line["prefill"]["frac_of_own_gemm"] = round(pre_rate / mm_flops, 4)
+    text = json.dumps(line)
+    print(text, flush=True)
+    if args.record:
+        with open(args.record, "w") as f:
+            f.write(f"# bench.py, {shape_name}\n\nCommand:\n\n    python {' '.join(['bench.py'] + sys.argv[1:])}\n\n"
+                    f"Result (one MI355X, random weights, synthetic tokens):\n\n```json\n{json.dumps(line, indent=1)}\n```\n")
     return 0
 
 

@@ -1,7 +1,7 @@
 """A plain, slow Llama dense decoder in numpy float64: whole sequences, no cache.
 
-One function per part, written from the reference's formulas (each cites the file
-and lines under /root/reference/ it follows).  It shares no code with the engine:
+One function per part, written from the reference's formulas (each cites the file and
+lines of the reference it follows, relative to its root).  It shares no code with the engine:
 it reads config.json and model.safetensors with its own few lines and knows nothing
 of pages, batches or kernels.  The tests compare everything the engine does with it.
 """
@@ -97,14 +97,14 @@ def open_folder(model_dir):
 # ----------------------------------------------------------------------------- parts
 def rmsnorm(x, w, eps):
     """y = x * (1/sqrt(mean(x^2) + eps)) * w: eps inside the root, added to the mean.
-    /root/reference/src/model.c:3386-3392"""
+    src/model.c:3386-3392"""
     ss = np.sum(x * x, axis=-1, keepdims=True)
     r = 1.0 / np.sqrt(ss / x.shape[-1] + eps)
     return x * r * w
 
 
 def rope_inv_freq(rot_dim, theta, scaling=None):
-    """inv_freq[j] = theta^(-2j/rot_dim) (/root/reference/src/model.c:285-289), then divided
+    """inv_freq[j] = theta^(-2j/rot_dim) (src/model.c:285-289), then divided
     by per-dimension factors (:291-297).  The reference takes the factors from the file;
     for rope_type "llama3" they follow from config.json: wavelength below orig/high is
     kept, above orig/low divided by factor, between them interpolated in orig/wavelength."""
@@ -116,7 +116,7 @@ def rope_inv_freq(rot_dim, theta, scaling=None):
     if kind in (None, "default"):
         return inv
     factor = scaling["factor"]
-    if kind == "linear":       # /root/reference/src/model.c:317-321
+    if kind == "linear":       # src/model.c:317-321
         return inv / factor
     assert kind == "llama3", kind
     low, high = scaling["low_freq_factor"], scaling["high_freq_factor"]
@@ -136,7 +136,7 @@ def rope_inv_freq(rot_dim, theta, scaling=None):
 
 def rope_angle(position, inv_freq_j):
     """a = pos * inv_freq[j] the way the reference forms it: the table holds floats
-    (/root/reference/src/model.c:286-289) and ``float a = pos * fr[j]`` is a float product (:3520).
+    (src/model.c:286-289) and ``float a = pos * fr[j]`` is a float product (:3520).
     At position 2,048 that product differs from the exact one by up to 1.2e-4 rad for the fastest
     pair, which belongs to the model as it is defined; cosine and sine are then taken exactly."""
     return float(np.float32(position) * np.float32(inv_freq_j))
@@ -146,7 +146,7 @@ def rope(x, positions, inv_freq, interleaved=False):
     """Rotate pair j of every head by a = pos * inv_freq[j]:
     (x0, x1) -> (x0 cos a - x1 sin a, x0 sin a + x1 cos a).  Un-permuted checkpoints pair
     element j with j + rot/2; the other layout pairs 2j with 2j+1.
-    x: [T, heads, D].  /root/reference/src/model.c:3514-3532"""
+    x: [T, heads, D].  src/model.c:3514-3532"""
     T, H, D = x.shape
     half = len(inv_freq)
     y = x.copy()
@@ -174,7 +174,7 @@ def rope_all_at_once(x, positions, inv_freq):
 
 
 def softmax(s):
-    """Maximum out, exponentials, divide by their sum.  /root/reference/src/model.c:3409-3415"""
+    """Maximum out, exponentials, divide by their sum.  src/model.c:3409-3415"""
     e = np.exp(s - np.max(s))
     return e / np.sum(e)
 
@@ -183,7 +183,7 @@ def attention(q, k, v, scale, window=None):
     """q [T, H, D], k/v [T, Hk, D], all of one sequence from position 0.  Head h reads
     key/value head h // (H/Hk); s_t = (q . k_t) * scale for t in [t0, p], t0 = p - window + 1
     when windowed; softmax; o = sum_t p_t v_t.
-    /root/reference/src/model.c:3548-3589 (heads, scores, weighted values), :6326 (t0)"""
+    src/model.c:3548-3589 (heads, scores, weighted values), :6326 (t0)"""
     T, H, D = q.shape
     Hk = k.shape[1]
     mul = H // Hk
@@ -220,12 +220,12 @@ def attention_all_at_once(q, k, v, scale, window=None):
 
 
 def silu(g):
-    """g / (1 + exp(-g)).  /root/reference/src/model.c:4451-4452"""
+    """g / (1 + exp(-g)).  src/model.c:4451-4452"""
     return g / (1.0 + np.exp(-g))
 
 
 def mlp(h, wg, wu, wd, bg=None, bu=None, bd=None):
-    """down(silu(gate h) * (up h)).  /root/reference/src/model.c:6399-6407"""
+    """down(silu(gate h) * (up h)).  src/model.c:6399-6407"""
     g = h @ wg.T + (0 if bg is None else bg)
     u = h @ wu.T + (0 if bu is None else bu)
     return (silu(g) * u) @ wd.T + (0 if bd is None else bd)
@@ -236,7 +236,7 @@ def forward(cfg, w, tokens, return_hidden=False, rows=None, all_at_once=False):
     """Logits [T, V] of one whole sequence (of the positions ``rows`` only, if given).  Order
     per layer: norm, q/k/v, rotation of q and k, attention over positions <= own, output
     projection, add, norm, feed-forward, add; then final norm and head.
-    /root/reference/src/model.c:6148-6483.  ``all_at_once``: rotation and attention by their
+    src/model.c:6148-6483.  ``all_at_once``: rotation and attention by their
     whole-array forms (a long sequence would take the loops minutes)."""
     rope_fn = rope_all_at_once if all_at_once else rope
     attention_fn = attention_all_at_once if all_at_once else attention
@@ -250,10 +250,10 @@ def forward(cfg, w, tokens, return_hidden=False, rows=None, all_at_once=False):
     V = cfg["vocab_size"]
     T = len(tokens)
     pos = np.arange(T)
-    # embedding: row copy, id outside the vocabulary reads row 0 (/root/reference/src/model.c:6148-6162)
+    # embedding: row copy, id outside the vocabulary reads row 0 (src/model.c:6148-6162)
     ids = [t if 0 <= t < V else 0 for t in tokens]
     x = w["model.embed_tokens.weight"][ids].copy()
-    scale = 1.0 / math.sqrt(D)                      # /root/reference/src/model.h:464-467
+    scale = 1.0 / math.sqrt(D)                      # src/model.h:464-467
     for l in range(cfg["num_hidden_layers"]):
         p = f"model.layers.{l}."
         h = rmsnorm(x, w[p + "input_layernorm.weight"], eps)
@@ -270,23 +270,23 @@ def forward(cfg, w, tokens, return_hidden=False, rows=None, all_at_once=False):
         a = o @ w[p + "self_attn.o_proj.weight"].T
         if cfg.get("attention_bias"):
             a = a + w[p + "self_attn.o_proj.bias"]
-        x = x + a                                    # /root/reference/src/model.c:6350-6352
+        x = x + a                                    # src/model.c:6350-6352
         h = rmsnorm(x, w[p + "post_attention_layernorm.weight"], eps)
         mb = cfg.get("mlp_bias")
         x = x + mlp(h, w[p + "mlp.gate_proj.weight"], w[p + "mlp.up_proj.weight"], w[p + "mlp.down_proj.weight"],
                     w.get(p + "mlp.gate_proj.bias") if mb else None, w.get(p + "mlp.up_proj.bias") if mb else None,
-                    w.get(p + "mlp.down_proj.bias") if mb else None)   # /root/reference/src/model.c:6421-6423
+                    w.get(p + "mlp.down_proj.bias") if mb else None)   # src/model.c:6421-6423
     if return_hidden:
         return x
     if rows is not None:
         x = x[list(rows)]
-    h = rmsnorm(x, w["model.norm.weight"], eps)      # /root/reference/src/model.c:6479
+    h = rmsnorm(x, w["model.norm.weight"], eps)      # src/model.c:6479
     head = w["model.embed_tokens.weight"] if cfg.get("tie_word_embeddings") else w["lm_head.weight"]
-    return h @ head.T                                # /root/reference/src/model.c:6481, tied :2353-2366
+    return h @ head.T                                # src/model.c:6481, tied :2353-2366
 
 
 def greedy(cfg, w, prompt, n_new):
-    """Greedy continuation: first index of the maximum (/root/reference/src/sample.c:169-172)."""
+    """Greedy continuation: first index of the maximum (src/sample.c:169-172)."""
     toks = list(prompt)
     out = []
     for _ in range(n_new):
@@ -298,7 +298,7 @@ def greedy(cfg, w, prompt, n_new):
 
 # ----------------------------------------------------------------------------- sampling
 def xorshift64(state):
-    """x ^= x<<13; x ^= x>>7; x ^= x<<17 on 64 bits.  /root/reference/src/sample.c:13-17"""
+    """x ^= x<<13; x ^= x>>7; x ^= x<<17 on 64 bits.  src/sample.c:13-17"""
     x = state & 0xFFFFFFFFFFFFFFFF
     x ^= (x << 13) & 0xFFFFFFFFFFFFFFFF
     x ^= x >> 7
@@ -307,14 +307,14 @@ def xorshift64(state):
 
 
 def rng_f32(state):
-    """(new state, draw in [0,1) from the top 24 bits).  /root/reference/src/sample.c:18-20"""
+    """(new state, draw in [0,1) from the top 24 bits).  src/sample.c:18-20"""
     s = xorshift64(state)
     return s, (s >> 40) / 16777216.0
 
 
 def sample_pick(logits, temp, draw, top_k=0, top_p=1.0, min_p=0.0, repeat_penalty=1.0, recent=(), exempt=()):
     """The reference's pick on a copy of ``logits`` with a given draw.
-    /root/reference/src/sample.c:141-329 (penalty :148-166, greedy :169-172, candidates sorted by
+    src/sample.c:141-329 (penalty :148-166, greedy :169-172, candidates sorted by
     z descending then id ascending :32-38, softmax / top-p / min-p / roulette walk :86-127)."""
     logits = np.array(logits, dtype=np.float32)
     V = len(logits)

@@ -164,3 +164,64 @@ def test_a_reader_may_not_look_further_back_than_the_cache_it_reads_keeps():
             CacheStorage([own, reader], [None] * 2, [None, 0], 4, 3, 2, torch.float32, dev)
     # an owner that keeps every key serves any reader
     CacheStorage([full, narrow, full], [None] * 3, [None, 0, 0], 4, 3, 2, torch.float32, dev)
+
+
+# ----------------------------------------------------------------------------- pools of different sizes
+def test_groups_have_pools_of_their_own_size():
+    from xyntetik_runner_amd.cache import pages_for_spec
+    # 2 requests, steps of at most 8 tokens, pages of 4: a window of 10 touches 3 pages, plus the one
+    # being filled and the one not yet given back, plus the step's own 2
+    assert pages_for_spec(WIN, 4, max_tokens=4000, max_requests=2, max_step_tokens=8) == 2 * (3 + 2) + 2
+    assert pages_for_spec(FULL, 4, max_tokens=4000, max_requests=2, max_step_tokens=8) == 1000
+    assert pages_for_spec(WIN, 4, max_tokens=4000, max_requests=2) == 1000         # steps of any size
+    assert pages_for_spec(WIN, 4, max_tokens=20, max_requests=2, max_step_tokens=8) == 5      # never more than the tokens' pages
+    m = CacheManager([FULL, WIN], page_size=4, pages_per_group=[40, 10], n_slots=2)
+    assert [g.pool.size for g in m.groups] == [40, 10]
+    assert m.capacity_tokens() == 160                       # the group that keeps every key sets the limit
+    assert m.max_portion() == (10 - 4) * 4                  # the windowed one what a step can bring
+    with pytest.raises(ValueError):
+        CacheManager([FULL, WIN], page_size=4, pages_per_group=[40], n_slots=2)
+    with pytest.raises(ValueError):
+        CacheManager([FULL, WIN], page_size=4, pages_per_group=[40, 0], n_slots=2)
+
+
+def test_a_windowed_pool_carries_a_request_longer_than_itself():
+    """Only windowed groups: a request grows to many times the pool's positions in portions no larger
+    than ``max_portion``, and never holds more pages than its window and its portion touch."""
+    m = CacheManager([WIN], page_size=4, pages_per_group=8, n_slots=1)
+    assert m.capacity_tokens() >= 1 << 60
+    step = m.max_portion()
+    assert step == (8 - 4) * 4
+    m.admit("a")
+    n = 0
+    while n < 600:
+        k = min(step, 600 - n)
+        m.reserve("a", n + k)
+        assert m.groups[0].pool.n_out <= 8
+        n += k
+        m.advance("a", n)
+        m.check()
+        assert m.groups[0].pool.n_out <= 4
+    # one token more than max_portion does not fit at this point
+    with pytest.raises(OutOfPages):
+        m.reserve("a", n + step + 5)
+    m.release("a")
+    assert m.all_free()
+
+
+def test_trim_is_counted():
+    """Who keeps a copy of a block table (a recorded step does) sees from ``version`` that pages
+    went back from its end, even when its length is later the same again."""
+    m = CacheManager([FULL], page_size=4, pages_per_group=8, n_slots=2)
+    m.admit("a"); m.admit("b")
+    m.reserve("a", 4); m.advance("a", 4)
+    m.reserve("b", 4); m.advance("b", 4)
+    m.reserve("a", 5); m.reserve("b", 5)
+    before = [list(m.get(r).tables[0]) for r in "ab"]
+    va = m.get("a").version
+    m.trim("a"); m.trim("b")
+    assert m.get("a").version > va
+    m.reserve("a", 5); m.reserve("b", 5)
+    after = [list(m.get(r).tables[0]) for r in "ab"]
+    assert [len(t) for t in after] == [len(t) for t in before] and after != before      # same lengths, other pages
+    m.check()

@@ -139,7 +139,7 @@ def test_no_size_stands_in_code():
 def test_sizes_the_kernels_do_not_take_are_refused_when_the_model_is_built():
     """A head size beyond what the attention and rotation kernels take is an error at load,
     not at the first step (the reference refuses bad geometry at load too,
-    /root/reference/src/model.c:2295-2329)."""
+    src/model.c:2295-2329)."""
     from xyntetik_runner_amd.engine.model import Model
     raw = dict(TINY_A, head_dim=272, num_attention_heads=2, num_key_value_heads=1)
     arch, cfg = config_from_dict(raw)

@@ -47,6 +47,41 @@ def test_greedy_through_the_entry_point(folders, which, lens, n_new):
         near_argmax(cfg, w, p, o, 0.02)
 
 
+def test_the_cache_is_sized_from_the_card_by_default(folders, tmp_path):
+    """A model whose config names a context of 131,072 (as the real Llama-3.1 files do) loads through
+    the entry point with nothing said about the cache: the pool takes what 64 requests of that length
+    need or what 90% of the card leaves, whichever is less, one request of the whole context fits, and
+    generation works.  With almost no memory allowed the error says what is missing
+    (src/model.h:516-592: the reference caps the context it allocates)."""
+    import json
+    import shutil
+    import torch
+    from xyntetik_runner_amd import LLM, SamplingParams
+    from xyntetik_runner_amd.cache import CacheTooSmall
+    d = str(tmp_path / "long_context")
+    shutil.copytree(folders["A"], d)
+    with open(os.path.join(d, "config.json")) as f:
+        cfg = json.load(f)
+    cfg["max_position_embeddings"] = 131072
+    with open(os.path.join(d, "config.json"), "w") as f:
+        json.dump(cfg, f)
+    llm = LLM(d, dtype="bfloat16")
+    m = llm.runner.manager
+    free, total = torch.cuda.mem_get_info()
+    assert 131072 <= m.capacity_tokens() <= 64 * 131072
+    assert llm.runner.storage.bytes_per_token() * m.capacity_tokens() <= 0.9 * total
+    _, w = P.load_folder(folders["A"])
+    prompt = prompt_ids(19, 256, 4)
+    out = llm.generate([prompt], SamplingParams(max_new_tokens=6))[0]
+    near_argmax(cfg, w, prompt, out, 0.02)
+    del llm
+    with pytest.raises(CacheTooSmall, match="does not hold one request of 131072 tokens"):
+        LLM(d, dtype="bfloat16", gpu_memory_fraction=1e-6)
+    # an explicit number of tokens is taken as it is
+    llm = LLM(d, dtype="bfloat16", max_tokens=512)
+    assert llm.runner.manager.capacity_tokens() == 512
+
+
 def test_sampled_tokens_depend_on_the_request_alone(folders):
     from xyntetik_runner_amd import LLM, SamplingParams
     cfg, w = P.load_folder(folders["B"])
@@ -89,7 +124,7 @@ def test_sampling_kernel_matches_plain_sampler():
     cases.append((64, all_equal, dict(temp=1.0, draw=0.5, top_k=0, top_p=1.0, min_p=0.0, repeat_penalty=1.0, recent=[])))
     cases.append((64, all_equal, dict(temp=1.0, draw=0.99, top_k=10, top_p=1.0, min_p=0.0, repeat_penalty=1.0, recent=[])))
     cases.append((64, all_equal, dict(temp=0.0, draw=0.99, top_k=0, top_p=1.0, min_p=0.0, repeat_penalty=1.0, recent=[])))
-    # the reference's own penalty vector (/root/reference/tests/test_sampler.c:200-206): token 1
+    # the reference's own penalty vector (tests/test_sampler.c:200-206): token 1
     cases.append((4, np.array([10.0, 9.0, 1.0, 0.5], dtype=np.float32),
                   dict(temp=0.01, draw=0.7, top_k=0, top_p=1.0, min_p=0.0, repeat_penalty=2.0, recent=[0])))
     exempt = [3]
@@ -132,7 +167,7 @@ def test_sampling_kernel_distribution_and_many_rows():
     mixed_t = torch.tensor([0.0, 1.0] * (n // 2), device=dev)
     got2 = ops.sample(rows, mixed_t, torch.tensor(draws, dtype=torch.float32, device=dev)).cpu().numpy()
     assert np.all(got2[0::2] == 5) and np.array_equal(got2[1::2], got[1::2])
-    # a temperature near zero picks like greedy whatever is drawn (/root/reference/tests/test_sampler.c:200-206)
+    # a temperature near zero picks like greedy whatever is drawn (tests/test_sampler.c:200-206)
     cold = ops.sample(rows, torch.full((n,), 0.01, device=dev), torch.tensor(draws, dtype=torch.float32, device=dev))
     assert np.all(cold.cpu().numpy() == 5)
 
@@ -206,14 +241,17 @@ def test_decode_steps_queued_ahead_change_nothing(folders, dtype):
         runner = ModelRunner.from_folder(folders["A"], dtype=dtype, max_tokens=1024, page_size=16, max_requests=8)
         eng = Engine(runner, stop_ids=[stop], run_ahead=ahead)
         ids = [eng.add_request(p, sp) for p, sp in zip(prompts[:4], params[:4])]
-        done, steps = {}, 0
+        done, ended, steps = {}, {}, 0
         while eng.has_work():
             for o in eng.step():
                 done.setdefault(o.req_id, []).append(o.token)
+                if o.finished:
+                    ended[o.req_id] = o.request
             steps += 1
             if steps == 6:                          # decoding is under way: a fifth request joins
                 ids.append(eng.add_request(prompts[4], params[4]))
-        results[ahead] = [list(eng.requests[i].output) for i in ids]
+        assert not eng.requests                     # a request that has ended is the caller's, not the engine's
+        results[ahead] = [list(ended[i].output) for i in ids]
         ahead_steps[ahead] = eng.stats.steps_ahead
         for i, rid in enumerate(ids):
             assert [t for t in done[rid] if t is not None] == results[ahead][i]
@@ -254,11 +292,11 @@ def test_an_engine_is_used_again_and_a_request_is_aborted_while_a_step_is_queued
     for _ in range(5):
         eng.step()
     assert eng._ahead is not None                                     # a step with all three rows is on its way
-    eng.scheduler.abort(eng.requests[ids[1]])
+    ended = {ids[1]: eng.abort(ids[1])}
     while eng.has_work():
-        eng.step()
-    assert [eng.requests[i].output for i in (ids[0], ids[2])] == [refs[0], refs[2]]
-    assert len(eng.requests[ids[1]].output) < 12
+        ended.update((o.req_id, o.request) for o in eng.step() if o.finished)
+    assert [ended[i].output for i in (ids[0], ids[2])] == [refs[0], refs[2]]
+    assert len(ended[ids[1]].output) < 12 and ended[ids[1]].finish_reason == "aborted" and not eng.requests
     runner.manager.check()
     assert not runner.manager.requests and runner.manager.free_pages() == runner.manager.pages_per_group
 

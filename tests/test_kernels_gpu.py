@@ -121,7 +121,7 @@ def test_gated_product_with_gates_far_from_zero(ops, M):
     """Gate values of -200 and +200 through the fused epilogues: the weight-streaming kernel's
     (8 rows), the kernel's that adds up K ranges (40 rows) and the tile kernel's, which uses the
     hardware's 2^x and reciprocal (300 rows).  act(-200) * up is 0 and no NaN
-    (/root/reference/src/model.c:4442-4452), act(200) is 200."""
+    (src/model.c:4442-4452), act(200) is 200."""
     from xyntetik_runner_amd.csrc.ops import PackedWeight
     K, F = 64, 96
     a = torch.ones(M, K, device=DEV).bfloat16()
@@ -420,6 +420,22 @@ def test_linear_32bit_few_rows(ops, M, N, K):
     if M < 16:                                        # and whatever kernel instance (1, 4, 8 or 16 rows) serves it
         more = torch.cat([a, torch.randn(16 - M, K, device=DEV)]).contiguous()
         assert torch.equal(ops.linear(more, w, bias=b, out_dtype=torch.float32)[:M], got)
+
+
+def test_linear_32bit_sum_order_changes_at_17_rows_and_both_are_close(ops):
+    """Up to 16 rows are summed by the streaming kernel, 17 and more by the tile kernel, in another
+    order: over the 14,336 columns of the widest product both stay within 1e-6 of the float64
+    product, and so does their difference for the same row."""
+    torch.manual_seed(5)
+    K, N = 14336, 96
+    a = torch.randn(17, K, device=DEV)
+    w = torch.randn(N, K, device=DEV) * 0.02
+    want = a.double() @ w.double().T
+    few = ops.linear(a[:16].contiguous(), w, out_dtype=torch.float32)
+    many = ops.linear(a, w, out_dtype=torch.float32)
+    assert rel(few, want[:16]) < 1e-6 and rel(many, want) < 1e-6
+    assert rel(few, many[:16]) < 1e-6
+    assert not torch.equal(few, many[:16])          # (if this ever holds, the header's caveat can go)
 
 
 def test_linear_one_hot_rows_pick_weight_rows(ops):

@@ -57,7 +57,7 @@ def test_rope_rotation_direction_and_pairing():
     x = np.array([[[1.0, 0.0]]])
     assert np.allclose(P.rope(x, [1], inv)[0, 0], [0.0, 1.0], atol=1e-7)         # (the angle is a float: pi/2 to 24 bits)
     # half-split on un-permuted rows == adjacent pairs on rows permuted as [0, D/2, 1, D/2+1, ...]
-    # (the converter's relation, /root/reference/src/model.c:1464-1466)
+    # (the converter's relation, src/model.c:1464-1466)
     D = 8
     inv = P.rope_inv_freq(D, 10000.0)
     v = rng.normal(size=(1, 1, D))
@@ -98,7 +98,7 @@ def _engine_table(rot, theta, scaling=None):
 @pytest.mark.parametrize("table", [_plain_table, _engine_table], ids=["plain", "engine"])
 def test_llama3_scaling_is_continuous_monotone_and_linear_in_frequency(table):
     """What fixes the interpolation between the two bands beside its text
-    (hook: /root/reference/src/model.c:291-297, where the reference divides by the factors a file
+    (hook: src/model.c:291-297, where the reference divides by the factors a file
     brings): the scaled/unscaled ratio is 1 below wavelength orig/high and 1/factor above
     orig/low, so a rule that joins them must meet both values at the band's edges, fall
     monotonically between them, and, being linear in orig/wavelength, give the mean of the two

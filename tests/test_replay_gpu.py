@@ -110,20 +110,31 @@ def test_long_portions_of_several_requests_in_one_step(models, tmp_path, dtype):
     check(traces.collect(steps, out, cfg["vocab_size"]), want, dtype, "D/long portions")
 
 
+def poison(runner):
+    """Every page of every layer holds NaN: a read beyond a request's length, or of a page it does
+    not own, shows in the logits."""
+    for lc in runner.storage.layers:
+        if lc.owns and lc.k is not None:
+            lc.k.fill_(float("nan"))
+            lc.v.fill_(float("nan"))
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-def test_pages_are_used_again_and_old_contents_never_show(models, tmp_path, dtype):
-    """The pool holds barely more than the live requests; every page is poisoned with NaN before
-    the replay, so a read beyond a request's length, or of a page it does not own, shows."""
-    import torch
+@pytest.mark.parametrize("which,page_size", [("B", 8), ("B", 16), ("B", 64), ("D", 16), ("D", 64)])
+def test_pages_are_used_again_and_old_contents_never_show(models, tmp_path, dtype, which, page_size):
+    """The pool holds barely more than the live requests and every page is poisoned with NaN before
+    the replay.  With pages of 8 positions bfloat16 attention is the 32-bit-arithmetic kernel; with 16
+    and 64 it is the matrix-core kernels (decoded tokens and short portions, and for the longer
+    requests of model D the 128-row blocks) and the products that rotate and cache their own result
+    (src/engine.c:218-221: a cached row is a function of its request's own tokens only)."""
     from xyntetik_runner_amd.engine.runner import ModelRunner
     from xyntetik_runner_amd.trace import replay
     import io
-    d, cfg, reqs, plens, want = models["B"]
+    d, cfg, reqs, plens, want = models[which]
     steps = traces.mixed(reqs, plens, max_live=2, seed=5)
-    mt = traces.max_live_tokens(steps, 64)
-    runner = ModelRunner.from_folder(d, dtype=dtype, max_tokens=mt, page_size=8, max_requests=2)
-    for lc in runner.storage.layers:
-        lc.k.fill_(float("nan")); lc.v.fill_(float("nan"))
+    mt = traces.max_live_tokens(steps, max(64, page_size))
+    runner = ModelRunner.from_folder(d, dtype=dtype, max_tokens=mt, page_size=page_size, max_requests=2)
+    poison(runner)
     seen = set()
     orig_step = runner.step
 
@@ -139,7 +150,158 @@ def test_pages_are_used_again_and_old_contents_never_show(models, tmp_path, dtyp
     for rid, p in seen:
         pages_by_req.setdefault(p, set()).add(rid)
     assert any(len(v) > 1 for v in pages_by_req.values()), "no page was used by two requests"
-    check(traces.collect(steps, out, cfg["vocab_size"]), want, dtype, "B/reuse")
+    check(traces.collect(steps, out, cfg["vocab_size"]), want, dtype, f"{which}/reuse, pages of {page_size}")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("which,page_size", [("A", 16), ("B", 64), ("D", 64)])
+def test_which_pages_a_request_gets_does_not_matter(models, tmp_path, dtype, which, page_size):
+    """The same mixed trace twice, in a pool three times the size it needs: once with the free list
+    as it is made (lowest page first), once shuffled, so that every request's pages lie scattered
+    and in another order.  A page number is an address and nothing else (tests/test_prefix.c:17-20:
+    rows land where the table says and read back the same), so the logits are the same to the bit."""
+    import random
+    from xyntetik_runner_amd.engine.runner import ModelRunner
+    from xyntetik_runner_amd.trace import replay
+    import io
+    d, cfg, reqs, plens, want = models[which]
+    steps = traces.mixed(reqs, plens, max_live=3, seed=11)
+    mt = 3 * traces.max_live_tokens(steps, max(64, page_size))
+    got, tables = {}, {}
+    for shuffled in (False, True):
+        runner = ModelRunner.from_folder(d, dtype=dtype, max_tokens=mt, page_size=page_size, max_requests=3)
+        poison(runner)
+        if shuffled:
+            for g in runner.manager.groups:
+                random.Random(17).shuffle(g.pool._free)
+        used = []
+        orig_step = runner.step
+
+        def spying_step(entries, _orig=orig_step, _runner=runner, _used=used):
+            r = _orig(entries)
+            _used.append(sorted((str(rc.req_id), tuple(rc.tables[0])) for rc in _runner.manager.requests.values()))
+            return r
+        runner.step = spying_step
+        out = str(tmp_path / f"o{int(shuffled)}")
+        replay(runner, traces.to_lines(steps), out, report=io.StringIO())
+        runner.manager.check()
+        got[shuffled], tables[shuffled] = traces.collect(steps, out, cfg["vocab_size"]), used
+    assert tables[True] != tables[False], "the shuffled free list gave the same pages"
+    check(got[False], want, dtype, f"{which}/pages in order")
+    for rid in want:
+        assert np.array_equal(got[True][rid], got[False][rid]), f"request {rid}: logits depend on the page numbers"
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_step_that_fails_leaves_the_recorded_steps_tables_right(models, dtype):
+    """Two requests decode through a recorded step and both take a new page in the same step; that
+    step fails after its block tables have gone to the device.  The pages it reserved go back, and the
+    next step hands them out the other way round (the page given back last is taken first): the
+    recorded step's copy of the tables must follow, or each request reads the other's page."""
+    from xyntetik_runner_amd.engine.batch import StepEntry
+    from xyntetik_runner_amd.engine.runner import ModelRunner
+    d, cfg, reqs, plens, want = models["A"]
+    a, b = reqs["r3"], reqs["r4"]                     # 80 and 166 tokens
+    runner = ModelRunner.from_folder(d, dtype=dtype, max_tokens=512, page_size=16, max_requests=2)
+    runner.step([StepEntry("a", a[:14], []), StepEntry("b", b[:30], [])])
+    got = {"a": [], "b": []}
+
+    def decode(i):
+        out = runner.step([StepEntry("a", [a[14 + i]], [0]), StepEntry("b", [b[30 + i]], [0])]).cpu().numpy()
+        got["a"].append(out[0]); got["b"].append(out[1])
+    decode(0); decode(1)                              # lengths 16 and 32: the next token of each opens a page
+    assert runner.graphs.captures >= 1
+    before = {r: list(runner.manager.get(r).tables[0]) for r in "ab"}
+    run = runner.graphs.run
+
+    def fails_after_the_tables_are_copied(*args, **kw):
+        run(*args, **kw)
+        raise RuntimeError("injected")
+    runner.graphs.run = fails_after_the_tables_are_copied
+    with pytest.raises(RuntimeError, match="injected"):
+        decode(2)
+    runner.graphs.run = run
+    assert {r: list(runner.manager.get(r).tables[0]) for r in "ab"} == before and runner.length("a") == 16
+    runner.manager.check()
+    for i in range(2, 20):
+        decode(i)
+    runner.manager.check()
+    for rid, toks, n0 in (("a", a, 14), ("b", b, 30)):
+        mx, mean = logit_error(np.stack(got[rid]), want["r3" if rid == "a" else "r4"][n0:n0 + 20])
+        assert mx <= TOL[dtype][0] and mean <= TOL[dtype][1], (rid, mx, mean)
+
+
+WIDE = {"A": 16, "B": 64, "D": 64}       # page sizes
+
+
+@pytest.fixture(scope="module")
+def wide(models):
+    """64 requests for each of three models: prompts of 1 to 150 tokens and 8 to 32 given decoded
+    tokens, with the plain logits of every place."""
+    out = {}
+    for which in WIDE:
+        d, cfg, _, _, _ = models[which]
+        _, w = P.load_folder(d)
+        rng = np.random.default_rng(40 + len(out))
+        plen = [int(n) for n in rng.integers(1, 151, size=64)]
+        plen[0], plen[1], plen[2] = 1, 150, 64
+        ndec = [8 + int(n) for n in rng.integers(0, 25, size=64)]
+        ndec[0], ndec[5] = 32, 8
+        toks = [prompt_ids(plen[i] + ndec[i], cfg["vocab_size"], 900 + i) for i in range(64)]
+        want = [P.forward(cfg, w, t, all_at_once=True) for t in toks]
+        out[which] = (d, cfg, plen, ndec, toks, want)
+    return out
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("n_live", [20, 40, 64])
+@pytest.mark.parametrize("which", list(WIDE))
+def test_many_requests_decode_through_recorded_steps(wide, which, n_live, dtype):
+    """20, 40 and 64 requests decode side by side (tests/test_batch.c:49-60, :203-215, past its 8):
+    the recorded steps for 32 and 64 rows, whose products take the kernels for 17 to 64 rows, with
+    rows that pad the batch (12 and 24 from the first step on, more as requests end at different
+    times), requests of 1 to 150 prompt tokens at different positions in every step, and every row
+    of every step against the plain implementation."""
+    from xyntetik_runner_amd.engine.batch import StepEntry
+    from xyntetik_runner_amd.engine.runner import ModelRunner
+    d, cfg, plen, ndec, toks, want = wide[which]
+    ps = WIDE[which]
+    ids = list(range(n_live))
+    mt = sum(-(-(plen[i] + ndec[i]) // max(64, ps)) * max(64, ps) for i in ids)
+    runner = ModelRunner.from_folder(d, dtype=dtype, max_tokens=mt, page_size=ps, max_requests=n_live)
+    poison(runner)
+    got = {i: [] for i in ids}
+    for g0 in range(0, n_live, 7):                    # the prompts, 7 requests a step
+        group = ids[g0:g0 + 7]
+        out = runner.step([StepEntry(i, toks[i][:plen[i]], list(range(plen[i]))) for i in group]).cpu().numpy()
+        r = 0
+        for i in group:
+            got[i].append(out[r:r + plen[i]])
+            r += plen[i]
+    assert runner.graphs.replays == 0 and runner.graphs.captures == 0
+    n_steps, widths = 0, set()
+    for k in range(max(ndec[i] for i in ids)):
+        live = [i for i in ids if k < ndec[i]]
+        out = runner.step([StepEntry(i, [toks[i][plen[i] + k]], [0]) for i in live]).cpu().numpy()
+        widths.add(len(live))
+        n_steps += 1
+        for r, i in enumerate(live):
+            got[i].append(out[r:r + 1])
+            if k == ndec[i] - 1:
+                runner.finish(i)
+    assert n_steps >= 24 and len(widths) > 3, "the batch never shrank"
+    # every decode step went through a recorded step (its first run records it)
+    assert runner.graphs.replays + runner.graphs.captures == n_steps and runner.graphs.replays > n_steps // 2
+    runner.manager.check()
+    assert runner.manager.all_free()
+    for i in ids:
+        rows = np.concatenate(got[i])
+        assert rows.shape == want[i].shape and np.isfinite(rows).all() and np.abs(rows).max() > 0
+        mx, mean = logit_error(rows, want[i])
+        if not (mx <= TOL[dtype][0] and mean <= TOL[dtype][1]):
+            dd = np.abs(rows - want[i]).max(axis=1)
+            raise AssertionError(f"{which} {dtype} {n_live} live, request {i} (prompt {plen[i]}): max {mx:.3e} mean "
+                                 f"{mean:.3e}; worst place {int(dd.argmax())}")
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
@@ -293,7 +455,7 @@ def test_decoding_with_norms_folded_into_the_products(models, which):
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_the_references_batch_workload(models, dtype):
-    """The workload of the reference's own batching test (/root/reference/tests/test_batch.c:49-60,
+    """The workload of the reference's own batching test (tests/test_batch.c:49-60,
     :203-215): 8 sequences with prompts of 5, 11, 8, 17, 6, 14, 9 and 20 tokens, ids
     ((seq+1)*7919 + i*104729) mod V, 24 greedy steps, decoded 1, 2, 4 and 8 at a time, so that
     every sequence of a batch sits at another position in every step.  Whole logits rows are

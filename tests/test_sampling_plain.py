@@ -1,5 +1,5 @@
 """The plain sampler against the vectors the reference's tests hold
-(/root/reference/tests/test_sampler.c:184-324) and against the host-side generator."""
+(tests/test_sampler.c:184-324) and against the host-side generator."""
 import numpy as np
 import pytest
 
@@ -37,7 +37,7 @@ def test_greedy_vectors():
     assert P.sample_pick(lg, 1.0, 0.0, repeat_penalty=10.0, recent=[1], exempt=[1]) == 1
     assert P.sample_pick(lg, 1.0, 0.0, repeat_penalty=10.0, recent=[7, -1, 1000]) == 1   # ids outside are ignored
     # the reference's own vector: token 0 was seen, a penalty of 2 halves its 10 to 5, below token 1's 9,
-    # and a temperature of 0.01 leaves no choice (/root/reference/tests/test_sampler.c:200-206)
+    # and a temperature of 0.01 leaves no choice (tests/test_sampler.c:200-206)
     for draw in (0.0, 0.3, 0.999):
         assert P.sample_pick([10.0, 9.0, 1.0, 0.5], 0.01, draw, repeat_penalty=2.0, recent=[0]) == 1
 

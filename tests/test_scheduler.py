@@ -164,3 +164,46 @@ def test_a_slice_of_a_requests_tokens():
             assert req.token_slice(a, b) == whole[a:b], (a, b)
     req.n_computed = 5
     assert req.remaining == 2
+
+
+def run_step_as_the_runner_does(s, token=7):
+    """``run_step``, and the cache manager is told what is cached now, as the step function tells
+    it (pages that a window has passed go back then)."""
+    plan = s.schedule()
+    for r, n in plan.entries:
+        s.manager.advance(r.id, r.n_computed + n)
+    for r in s.ran(plan):
+        s.accept(r, token)
+    s.manager.check()
+    return plan
+
+
+def test_portions_are_cut_to_what_the_windowed_pools_can_hold():
+    """Every layer keeps a window of 10 keys, the pool has 8 pages of 4: a prompt of 200 tokens is no
+    longer than the cache holds (windowed layers set no limit), runs in portions of at most
+    (8 - 4) x 4 = 16 tokens although the budget is 64, nobody is preempted and nothing fails."""
+    m = CacheManager([KVSpec(1, 32, 10)], page_size=4, pages_per_group=8, n_slots=2)
+    s = Scheduler(m, max_batched_tokens=64, max_running=2, max_model_len=1024)
+    assert s.capacity_tokens() > 1 << 60
+    s.add(req("a", 200, new=4))
+    sizes = []
+    while s.running or s.waiting:
+        plan = run_step_as_the_runner_does(s)
+        assert not plan.preempted and not plan.failed
+        sizes.append(plan.n_tokens)
+        assert len(sizes) < 60
+    assert sizes[:13] == [16] * 12 + [8] and sizes[13:] == [1] * 3
+    assert m.all_free()
+
+
+def test_a_full_attention_group_still_limits_the_length():
+    m = CacheManager([SPEC, KVSpec(1, 32, 10)], page_size=4, pages_per_group=[10, 8], n_slots=2)
+    s = Scheduler(m, max_batched_tokens=64, max_running=2, max_model_len=1024)
+    assert s.capacity_tokens() == 40
+    with pytest.raises(ValueError, match="does not fit the cache"):
+        s.add(req("a", 40))
+    s.add(req("b", 39, new=1))
+    while s.running or s.waiting:
+        plan = run_step_as_the_runner_does(s)
+        assert not plan.failed
+    assert m.all_free()

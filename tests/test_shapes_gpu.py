@@ -6,7 +6,7 @@ random weights: the matrix kernels are chosen by size, and several of their bran
 at these sizes only (few rows against a matrix 14336 wide, the head's 128256 columns, the tile
 shapes and the split launches of a 2,048-row product, the q/k/v tile that rotates and caches 32
 heads).  The reference holds its GPU path to its CPU path on the model it benchmarks
-(/root/reference/tests/test_gpu_identity.c:50-60, :91-105) and fails on all-zero logits
+(tests/test_gpu_identity.c:50-60, :91-105) and fails on all-zero logits
 (:190-201); so does this.
 """
 import numpy as np
@@ -29,7 +29,7 @@ SHAPE_8B_2_OF_32_LAYERS = {
 # Of the mean logit range: (max, mean).  float32 as for the small models (measured here: 1.4e-6 and
 # 1.9e-7).  bfloat16: the maximum as for the small models; the mean is the reference's own bound for
 # two back ends of one model, mean |d| <= 2e-3 of the mean logit range
-# (/root/reference/tests/test_gpu_identity.c:50-60).  The small models' 1e-3 is what this model's
+# (tests/test_gpu_identity.c:50-60).  The small models' 1e-3 is what this model's
 # honest rounding comes to: rows at position 0, which no attention error reaches, differ by 4.6e-4;
 # rows behind 2,000 keys by 1.0e-3 whichever kernels run (norms folded or not, rotation fused or
 # not), because queries and cached keys carry 8 bits (1.1e-3 rms each), which moves a score of
@@ -133,6 +133,58 @@ def test_8b_widths_2_of_32_layers_mixed(shape_8b, dtype):
     assert [sum(len(t) for _, t, _ in st) for st in steps[:5]] == [49, 1026, 602, 386, 42]
     got, runner = run_steps(d, dtype, steps)
     compare(got, want, dtype, "mixed")
+
+
+class Kept:
+    """Tensors on demand, each widened once and kept (about 12 GB for two layers of these widths)."""
+
+    def __init__(self, w):
+        self.w, self.kept = w, {}
+
+    def __contains__(self, name):
+        return name in self.w
+
+    def __getitem__(self, name):
+        if name not in self.kept:
+            self.kept[name] = self.w[name]
+        return self.kept[name]
+
+    def get(self, name, default=None):
+        return self[name] if name in self.w else default
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_8b_widths_2_of_32_layers_40_requests_decode_side_by_side(shape_8b, dtype):
+    """The benchmark's wide decode steps at the benchmark's widths: 40 requests with prompts of 3 to
+    60 tokens decode 6 tokens each through the recorded step for 64 rows (24 rows pad it), whose
+    products are the kernels for 17 to 64 rows with K split among workgroups and the kernels that add
+    the parts up (with the norm, or rotating and caching); then 20 of them go on alone (the step for
+    32 rows).  Every decoded row against the plain implementation."""
+    from xyntetik_runner_amd.engine import ModelRunner, StepEntry
+    d, cfg, _, _, _ = shape_8b
+    _, w = P.open_folder(d)
+    w = Kept(w)
+    V = cfg["vocab_size"]
+    n_req, n_dec = 40, 6
+    rng = np.random.default_rng(3)
+    plen = [int(n) for n in rng.integers(3, 61, size=n_req)]
+    toks = [prompt_ids(plen[i] + n_dec + 3, V, 700 + i) for i in range(n_req)]
+    runner = ModelRunner.from_folder(d, dtype=dtype, max_tokens=n_req * 128, page_size=64, max_requests=n_req)
+    for g0 in range(0, n_req, 10):
+        runner.step([StepEntry(i, toks[i][:plen[i]], []) for i in range(g0, g0 + 10)])
+    got = {i: [] for i in range(n_req)}
+    for k in range(n_dec + 3):
+        live = list(range(n_req)) if k < n_dec else list(range(0, n_req, 2))
+        out = runner.step([StepEntry(i, [toks[i][plen[i] + k]], [0]) for i in live]).cpu().numpy()
+        for r, i in enumerate(live):
+            got[i].append(out[r])
+    assert runner.graphs.captures == 2 and runner.graphs.replays == n_dec + 3 - 2
+    for i in range(n_req):
+        rows = np.stack(got[i])
+        want = P.forward(cfg, w, toks[i][:plen[i] + len(rows)], rows=list(range(plen[i], plen[i] + len(rows))), all_at_once=True)
+        assert np.isfinite(rows).all() and np.abs(rows).max() > 0
+        mx, mean = logit_error(rows, want)
+        assert mx <= TOL[dtype][0] and mean <= TOL[dtype][1], (dtype, i, plen[i], mx, mean)
 
 
 # ----------------------------------------------------------------------------- the other two shapes

@@ -67,7 +67,7 @@ def prompt_ids(n: int, vocab: int, seed: int):
 
 def logit_error(got, want):
     """(max |d|, mean |d|) as fractions of the mean logit range of ``want``
-    (the reference's measure, /root/reference/tests/test_gpu_identity.c:41-60)."""
+    (the reference's measure, tests/test_gpu_identity.c:41-60)."""
     got = np.asarray(got, dtype=np.float64)
     want = np.asarray(want, dtype=np.float64)
     rng = float(np.mean(want.max(axis=-1) - want.min(axis=-1)))

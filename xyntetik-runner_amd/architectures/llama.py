@@ -2,9 +2,9 @@
 
 Every layer is the same pre-norm block of grouped-query attention with rotary
 position encoding and a SiLU-gated feed-forward
-(/root/reference/src/model.c:6168-6473); the tensors carry the names of un-permuted
+(src/model.c:6168-6473); the tensors carry the names of un-permuted
 checkpoints, so the rotation pairs element j with j + rotary_dim/2
-(/root/reference/src/model.c:1464-1466 explains the other pairing).
+(src/model.c:1464-1466 explains the other pairing).
 """
 from __future__ import annotations
 

@@ -9,10 +9,10 @@ for state of fixed size (zeroed by the step function before its first use), whet
 or not any layer has such state.
 
 The reference keeps one contiguous cache per sequence and never gives rows back
-while the process lives (/root/reference/src/model.c:3089-3101, :3351-3354); what it
+while the process lives (src/model.c:3089-3101, :3351-3354); what it
 does promise is kept here per request: row i of a request is a function of its
-tokens [0, i] only (/root/reference/src/engine.c:218-221) and the tokens recorded for
-a request are exactly those whose rows are cached (/root/reference/src/engine.c:852-861).
+tokens [0, i] only (src/engine.c:218-221) and the tokens recorded for
+a request are exactly those whose rows are cached (src/engine.c:852-861).
 
 Page 0 of every group is never handed out: padded rows of a batch write there.
 This file is pure host logic; ``storage.py`` owns the device tensors.
@@ -20,7 +20,7 @@ This file is pure host logic; ``storage.py`` owns the device tensors.
 from __future__ import annotations
 
 from dataclasses import dataclass, field
-from typing import Dict, Hashable, List, Optional, Sequence
+from typing import Dict, Hashable, List, Optional, Sequence, Union
 
 from ..parts.base import KVSpec
 from .pages import OutOfPages, Pool
@@ -42,6 +42,7 @@ class RequestCache:
     n_tokens: int = 0                      # positions [0, n_tokens) are cached
     tables: List[List[int]] = field(default_factory=list)   # one block table per group
     fresh: bool = True                     # the slot has not been used by this request yet
+    version: int = 0                       # counts the times a table lost pages at its end (`trim`)
 
 
 def first_needed_position(n_tokens: int, window: Optional[int]) -> int:
@@ -51,14 +52,36 @@ def first_needed_position(n_tokens: int, window: Optional[int]) -> int:
     return max(0, n_tokens - window + 1)
 
 
+def pages_for_spec(spec: KVSpec, page_size: int, max_tokens: int, max_requests: int,
+                   max_step_tokens: Optional[int] = None) -> int:
+    """How many pages a group needs so that ``max_requests`` requests holding ``max_tokens`` tokens
+    together can run steps of up to ``max_step_tokens`` tokens (None: of any size).
+
+    A group that keeps every key needs the tokens' pages.  A group that keeps a window needs, for
+    every request, the pages its window touches plus the one being filled and the one not yet
+    given back, and, over all requests of a step, the pages of the step's tokens: a portion's pages
+    are all held until the portion is cached.
+    """
+    full = max(1, -(-int(max_tokens) // page_size))
+    if spec.window is None or max_step_tokens is None:
+        return full
+    per_request = -(-spec.window // page_size) + 2
+    return min(full, max_requests * per_request + -(-int(max_step_tokens) // page_size))
+
+
 class CacheManager:
-    def __init__(self, group_specs: Sequence[KVSpec], page_size: int, pages_per_group: int, n_slots: int):
+    def __init__(self, group_specs: Sequence[KVSpec], page_size: int, pages_per_group: Union[int, Sequence[int]],
+                 n_slots: int):
+        """``pages_per_group``: one number for all groups or one per group (see ``pages_for_spec``)."""
         if page_size < 1 or page_size & (page_size - 1):
             raise ValueError(f"page size {page_size} must be a power of two")
-        if pages_per_group < 1:
+        sizes = [pages_per_group] * len(group_specs) if isinstance(pages_per_group, int) else list(pages_per_group)
+        if len(sizes) != len(group_specs):
+            raise ValueError(f"{len(sizes)} pool sizes for {len(group_specs)} groups")
+        if any(n < 1 for n in sizes) or (isinstance(pages_per_group, int) and pages_per_group < 1):
             raise ValueError("a group needs at least one page")
         self.page_size = page_size
-        self.groups = [GroupInfo(s, page_size, Pool(pages_per_group, first=1, what="page")) for s in group_specs]
+        self.groups = [GroupInfo(s, page_size, Pool(n, first=1, what="page")) for s, n in zip(group_specs, sizes)]
         self.slots = Pool(n_slots, what="state slot")
         self.requests: Dict[Hashable, RequestCache] = {}
         self._no_pages = [0] * len(self.groups)
@@ -67,7 +90,29 @@ class CacheManager:
     # ------------------------------------------------------------------ sizes
     @property
     def pages_per_group(self) -> int:
+        """The pool size of the first group (of every group, when they were given one number)."""
         return self.groups[0].pool.size if self.groups else 0
+
+    def all_free(self) -> bool:
+        """No page of any group and no state slot is out."""
+        return all(g.pool.n_out == 0 for g in self.groups) and self.slots.n_out == 0
+
+    def capacity_tokens(self) -> int:
+        """The most tokens one request can hold: what the smallest pool of a group that keeps every
+        key holds.  A group that keeps a window gives pages back as a request grows and sets no limit."""
+        full = [g.pool.size * self.page_size for g in self.groups if g.spec.window is None]
+        return min(full) if full else 1 << 62
+
+    def max_portion(self) -> int:
+        """The most tokens of one request that a step can run, whatever its length: the pages of a
+        windowed group must hold the window behind the portion's first token and the portion
+        (groups that keep every key limit a request's length, not its portions)."""
+        best = 1 << 62
+        for g in self.groups:
+            if g.spec.window is not None:
+                behind = -(-g.spec.window // self.page_size) + 1
+                best = min(best, max(1, (g.pool.size - behind) * self.page_size))
+        return best
 
     def pages_for(self, n_tokens: int) -> int:
         return -(-n_tokens // self.page_size)
@@ -128,6 +173,7 @@ class CacheManager:
             table = rc.tables[gi]
             while len(table) > keep:
                 page = table.pop()
+                rc.version += 1             # who copied the table must not take its length for its contents
                 if page >= 0:
                     g.pool.give(page)
 

@@ -11,7 +11,7 @@ bounded by a request's length, so a page's old contents are never seen.
 from __future__ import annotations
 
 from dataclasses import dataclass
-from typing import Dict, List, Optional
+from typing import Callable, Dict, List, Optional, Union
 
 import torch
 
@@ -31,12 +31,17 @@ class LayerCache:
 
 class CacheStorage:
     def __init__(self, kv_specs: List[Optional[KVSpec]], state_specs: List[Optional[StateSpec]],
-                 cache_of: List[Optional[int]], page_size: int, pages_per_group: int, n_slots: int,
+                 cache_of: List[Optional[int]], page_size: int,
+                 pages_per_group: Union[int, Callable[[KVSpec], int]], n_slots: int,
                  dtype: torch.dtype, device: torch.device):
-        """``kv_specs[i]``/``state_specs[i]``/``cache_of[i]`` describe entry ``i`` of the run order."""
-        self.page_size, self.n_pages, self.n_slots = page_size, pages_per_group + 1, n_slots
+        """``kv_specs[i]``/``state_specs[i]``/``cache_of[i]`` describe entry ``i`` of the run order.
+        ``pages_per_group``: one number for every group, or a function of a group's ``KVSpec``
+        (a group that keeps a window of keys needs fewer pages than one that keeps them all)."""
+        self.page_size, self.n_slots = page_size, n_slots
+        sized = pages_per_group if callable(pages_per_group) else (lambda spec: pages_per_group)
         self.null_slot = n_slots
         self.group_specs: List[KVSpec] = []
+        self.group_pages: List[int] = []        # usable pages of each group (the null page comes on top)
         self.layers: List[LayerCache] = []
         for i, (kv, st) in enumerate(zip(kv_specs, state_specs)):
             owner = cache_of[i]
@@ -58,9 +63,11 @@ class CacheStorage:
             if kv is not None:
                 if kv not in self.group_specs:
                     self.group_specs.append(kv)
+                    self.group_pages.append(max(1, int(sized(kv))))
                 group = self.group_specs.index(kv)
-                k = torch.zeros((self.n_pages, kv.num_kv_heads, page_size, kv.head_dim), dtype=dtype, device=device)
-                v = torch.zeros((self.n_pages, kv.num_kv_heads, kv.head_dim, page_size), dtype=dtype, device=device)
+                n_pages = self.group_pages[group] + 1
+                k = torch.zeros((n_pages, kv.num_kv_heads, page_size, kv.head_dim), dtype=dtype, device=device)
+                v = torch.zeros((n_pages, kv.num_kv_heads, kv.head_dim, page_size), dtype=dtype, device=device)
             state = None
             if st is not None:
                 # one row more than requests: the last is nobody's (rows that pad a recorded step use it)

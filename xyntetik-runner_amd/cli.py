@@ -1,5 +1,5 @@
 """The command line, with the reference's option names and meanings where it has them
-(/root/reference/src/main.c:188-340 usage, :505-639 parsing):
+(src/main.c:188-340 usage, :505-639 parsing):
 
   -m PATH   model folder (config.json + model.safetensors; the reference takes a GGUF file)
   -p TEXT   prompt; \\n, \\t, \\\\ are unescaped; echoed before the completion (:509, :1519, :1541)
@@ -231,7 +231,7 @@ def main(argv: Optional[List[str]] = None) -> int:
         sys.stdout.write(",".join(map(str, prompt)) if as_ids else text)
         sys.stdout.flush()
     rid = engine.add_request(prompt, params)
-    req = engine.requests[rid]
+    req = engine.requests[rid]          # (the engine drops it when it ends; its last output brings it again)
     t0 = time.perf_counter()
     t_first = None
     n_gen = 0

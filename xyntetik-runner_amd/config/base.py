@@ -3,8 +3,8 @@
 A value of the wrong type, sign or range is an error that names the key; it is
 never passed on as garbage.  The reference reads its hyper-parameters with typed
 getters that fall back to a default on a wrong type, a negative or a NaN
-(/root/reference/src/gguf.c:494-567) and then refuses bad geometry in one place
-(/root/reference/src/model.c:2295-2329); here both steps raise ``ConfigError``.
+(src/gguf.c:494-567) and then refuses bad geometry in one place
+(src/model.c:2295-2329); here both steps raise ``ConfigError``.
 """
 from __future__ import annotations
 
@@ -13,7 +13,7 @@ import math
 import os
 from typing import Any, Mapping, Optional, Sequence
 
-# Upper bound of every axis, as in /root/reference/src/model.c:2295-2329.
+# Upper bound of every axis, as in src/model.c:2295-2329.
 MAX_AXIS = 1 << 20
 _MISSING = object()
 

@@ -1,7 +1,7 @@
 """``LlamaConfig``: the Llama dense decoder's hyper-parameters, typed.
 
 Key by key this is the reference's hyper-parameter block
-(/root/reference/src/model.c:1422-1470) under the names ``config.json`` uses:
+(src/model.c:1422-1470) under the names ``config.json`` uses:
 
 ===============================  ==============================  =========
 reference GGUF key                config.json key                 default
@@ -20,7 +20,7 @@ rows of ``token_embd``            ``vocab_size``                  required (:233
 no ``output.weight``              ``tie_word_embeddings``         false (:2353)
 ===============================  ==============================  =========
 
-The geometry checks are those of /root/reference/src/model.c:2295-2329.
+The geometry checks are those of src/model.c:2295-2329.
 """
 from __future__ import annotations
 
@@ -36,9 +36,9 @@ class RopeScaling:
 
     ``rope_type`` "llama3" rescales each rotary frequency by its wavelength; the
     reference does not compute this itself but divides its table by per-dimension
-    factors that the file brings (/root/reference/src/model.c:291-297), which is
+    factors that the file brings (src/model.c:291-297), which is
     the same thing.  "linear" divides every frequency by ``factor``
-    (/root/reference/src/model.c:317-321).
+    (src/model.c:317-321).
     """
     rope_type: str
     factor: float

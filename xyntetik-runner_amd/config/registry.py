@@ -4,7 +4,7 @@
 configuration class and the builder that turns a configuration into a
 ``ModelSpec``.  An unknown name is an error that lists the known ones, as the
 reference refuses a GGUF architecture that is not on its allowlist
-(/root/reference/src/model.c:751-763, :1395-1418).
+(src/model.c:751-763, :1395-1418).
 """
 from __future__ import annotations
 

@@ -8,7 +8,7 @@ name prefix it is given.
 The reference keeps the same facts as per-layer arrays on its model record:
 which layers are windowed, which layer owns the cache rows a layer reads
 (``model_kv_owner``), per-layer head counts and rotary widths
-(/root/reference/src/model.h:423-510).
+(src/model.h:423-510).
 """
 from __future__ import annotations
 

@@ -5,8 +5,8 @@
 // For the token at position p of its request and query head h (key/value head
 // h / (H/Hk), contiguous groups): s_t = (q . K_t) * scale for t in [lo, p], causal by
 // the loop bound, lo = max(0, p - window + 1) for a windowed layer
-// (/root/reference/src/model.c:3553-3573, :6326); softmax with the maximum taken out
-// (/root/reference/src/model.c:3409-3415); out = sum_t p_t V_t (:3576-3587).  The
+// (src/model.c:3553-3573, :6326); softmax with the maximum taken out
+// (src/model.c:3409-3415); out = sum_t p_t V_t (:3576-3587).  The
 // softmax runs over blocks of 64 keys with a running maximum and sum, which gives the
 // same value up to rounding.
 #include "common.h"

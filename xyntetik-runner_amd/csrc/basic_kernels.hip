@@ -6,7 +6,7 @@
 
 // ---------------------------------------------------------------- embedding
 // x[t] = table[id_t]; an id outside [0, V) reads row 0
-// (/root/reference/src/model.c:6148-6162).
+// (src/model.c:6148-6162).
 template <typename TW>
 __global__ void k_embedding(float* __restrict__ out, const TW* __restrict__ table,
                             const int* __restrict__ ids, int E, int V, float scale) {
@@ -50,7 +50,7 @@ extern "C" int xr_embedding(float* out, const void* table, const int* ids, int T
 
 // ---------------------------------------------------------------- RMSNorm
 // y_i = x_i * r * w_i with r = 1/sqrt(mean(x^2) + eps): eps inside the root, added to
-// the mean; multiply order (x*r)*w (/root/reference/src/model.c:3386-3392).
+// the mean; multiply order (x*r)*w (src/model.c:3386-3392).
 template <typename TO, typename TW>
 __global__ void k_rmsnorm(TO* __restrict__ out, const float* __restrict__ x, const TW* __restrict__ w,
                           const int* __restrict__ rows, int E, int ldx, float eps) {
@@ -152,9 +152,9 @@ extern "C" int xr_rmsnorm(void* out, const float* x, const void* w, const int* r
 // ---------------------------------------------------------------- rotary + cache write
 // Rotation of pair index j of a head by a = pos * inv_freq[j]:
 //   (x0, x1) -> (x0*c - x1*s, x0*s + x1*c), c = cos(a)*mscale, s = sin(a)*mscale
-// (/root/reference/src/model.c:3514-3532).  Half-split pairs (j, j + rot/2) are what
+// (src/model.c:3514-3532).  Half-split pairs (j, j + rot/2) are what
 // un-permuted checkpoints need; interleaved pairs (2j, 2j+1) are the other option.
-// Keys are cached rotated, values as they are (/root/reference/src/model.c:6300-6311).
+// Keys are cached rotated, values as they are (src/model.c:6300-6311).
 // Cache layout per layer: K [page][kv_head][slot][d], V [page][kv_head][d][slot].
 struct RopeArgs {
     const float* q_in;      // [T, in_stride] 32-bit
@@ -322,8 +322,8 @@ extern "C" int xr_rope_kv_write(const float* q_in, const float* k_in, const floa
 }
 
 // ---------------------------------------------------------------- gate
-// h = act(g) * u; act = SiLU: g / (1 + exp(-g)) (/root/reference/src/model.c:4451-4452,
-// /root/reference/src/kernels.cu:2868-2874).  gu row = [gate(F) | up(F)].
+// h = act(g) * u; act = SiLU: g / (1 + exp(-g)) (src/model.c:4451-4452,
+// src/kernels.cu:2868-2874).  gu row = [gate(F) | up(F)].
 template <typename TI, typename TO>
 __global__ void k_gate_mul(TO* __restrict__ out, const TI* __restrict__ gu, int F, int ld_gu, size_t n, int act) {
     size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;

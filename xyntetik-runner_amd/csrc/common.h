@@ -84,7 +84,7 @@ __host__ __device__ inline uint32_t pack_bf16x2(float lo, float hi) {
 // FAST: with the hardware's 2^x and reciprocal (1 ulp each)
 template <bool FAST> __device__ inline float gate_act(int act, float g) {
     switch (act) {
-    default:    // XR_ACT_SILU: g / (1 + exp(-g)) (/root/reference/src/model.c:4451-4452)
+    default:    // XR_ACT_SILU: g / (1 + exp(-g)) (src/model.c:4451-4452)
         return FAST ? g * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(g * -1.44269504f))
                     : g / (1.0f + expf(-g));
     }

@@ -16,13 +16,13 @@
 // at 8 rows: 101 -> 86 us for the four products of a layer of the 8B shape.
 // Epilogues: store (float or bfloat16), add into a float output (the residual stream),
 // and SwiGLU: with w = [gate rows; up rows] the kernel writes silu(gate) * up, so the
-// [M, 2F] intermediate never reaches memory (/root/reference/src/model.c:6399-6404).
+// [M, 2F] intermediate never reaches memory (src/model.c:6399-6404).
 // Up to 64 rows two more things ride on a product, in the skinny kernel's epilogue (up to 16
 // rows) or in the kernel that adds up a split product's K ranges: the RMSNorm that follows a
-// product into the residual stream (/root/reference/src/model.c:3386-3392), and for the
+// product into the residual stream (src/model.c:3386-3392), and for the
 // q/k/v product the rotation of queries and keys and the write of keys and values to their
 // pages (RopeFuse), so that a decode step launches 6 kernels a layer.
-// The reference's float-weight "GEMM" is a multi-column matvec (/root/reference/src/kernels.cu:116-144);
+// The reference's float-weight "GEMM" is a multi-column matvec (src/kernels.cu:116-144);
 // its tensor-core kernels (:856) exist for quantised weights only.
 #include "common.h"
 #include "async_copy.h"
@@ -216,7 +216,7 @@ __device__ inline void write_tiles(float* stage, const f32x16 (&t)[NT], void* ds
 }
 
 // The cosines and sines a product of many rows needs to rotate its own result, once for all
-// its tiles: the same formulas as rope_store (/root/reference/src/model.c:3514-3532).
+// its tiles: the same formulas as rope_store (src/model.c:3514-3532).
 __global__ __launch_bounds__(256) void k_rope_table(float2* cs, const int* positions, const float* inv_freq,
                                                     int M, int half, float mscale) {
     const int q = blockIdx.x * 256 + threadIdx.x;

@@ -1,9 +1,13 @@
 // Plain matrix product out[M,N] = a[M,K] * w[N,K]^T (+ bias) with 32-bit FMA only:
 // the matrix product of the true 32-bit path, and the yardstick of the MFMA kernels.
 // Weights are [n_out][n_in] row-major as the reference keeps them
-// (/root/reference/src/model.c:193-205); each output is a sum over k in ascending
-// order, whatever the batch, so a row's result does not depend on its neighbours.
-// The sum has two levels: runs of RBK * RB_FOLD = 128 columns are summed by FMA, and the runs'
+// (src/model.c:193-205).  A row's result does not depend on the rows beside it, but the order
+// of its sum over k depends on how many rows the product has: with more than 16 rows the tile
+// kernel below sums in ascending order in two levels, with up to 16 the kernel further down
+// (k_gemv_ref) gives every lane every 64th group of four columns and adds the lanes' sums in a
+// tree.  A token's 32-bit result therefore differs in its last bits between a step of 16 rows and
+// one of 17 (both stay within 1e-6 of the exact product at K = 14,336).
+// The tile kernel's two levels: runs of RBK * RB_FOLD = 128 columns are summed by FMA, and the runs'
 // sums are added up with a compensated (Kahan) sum.  One running 32-bit sum over the 14,336
 // columns of a wide feed-forward loses about 1e-5 of the result to rounding, which at such
 // widths is as much as a real fault may be; summed this way a product is about ten times closer

@@ -1,9 +1,7 @@
 // An entry point that allocates nothing.
 //
-// It has no counterpart in the reference, whose sampler runs on the host over logits copied
-// back (/root/reference/src/sample.c:141, /root/reference/src/cuda.c:4423).  It is for callers
-// that cannot allocate device memory: code under HIP graph capture, tight serving loops, and
-// harnesses that forbid hipMalloc.
+// It has no counterpart in the reference.  It is for callers that cannot allocate device
+// memory: code under HIP graph capture, tight serving loops, and harnesses that forbid hipMalloc.
 //
 // xr_sample_static is xr_sample with the work area of the greedy rows' first pass (a row's
 // logits are read by 32 workgroups, each leaving the maximum of its range) in a device array

@@ -1,8 +1,8 @@
 // Sampling on the device: one workgroup per row of logits.
 //
 // temp <= 0: the first index of the maximum, logits untouched
-// (/root/reference/src/sample.c:169-172).  temp > 0, in the reference's order
-// (/root/reference/src/sample.c:148-166, :86-127, :302-328):
+// (src/sample.c:169-172).  temp > 0, in the reference's order
+// (src/sample.c:148-166, :86-127, :302-328):
 //   repeat penalty over the recent window (each occurrence counts; exempt ids skipped;
 //   a positive logit is divided, another multiplied), z = logit / temp, candidates in
 //   the total order "z descending, then id ascending", top-k (softmax over the k kept),

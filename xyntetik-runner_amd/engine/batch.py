@@ -7,9 +7,9 @@ request in this batch; per request and cache group the block table.  One pinned
 host buffer carries all of it to the device in a single copy.
 
 The reference has two narrower primitives, n consecutive tokens of one sequence
-(/root/reference/src/model.h:667-670) and one token each of up to 8 sequences with
-per-column position and cache pointers (/root/reference/src/model.h:796-807,
-/root/reference/src/cuda.c:4213-4236); an entry list covers both and their mixtures.
+(src/model.h:667-670) and one token each of up to 8 sequences with
+per-column position and cache pointers (src/model.h:796-807,
+src/cuda.c:4213-4236); an entry list covers both and their mixtures.
 """
 from __future__ import annotations
 

@@ -6,7 +6,7 @@ has run, and finished requests give back what they hold.  In steady decoding the
 step's kernels are queued before the host reads this step's tokens (``_launch_ahead``), so
 the GPU does not wait for the host's turn.  The first generated token
 is sampled from the logits of the prompt's last position, as in the reference
-(/root/reference/src/engine.c:1939-1956); unlike it, no step is run for a token after
+(src/engine.c:1939-1956); unlike it, no step is run for a token after
 which nothing will be sampled.
 """
 from __future__ import annotations
@@ -32,6 +32,7 @@ class StepOutput:
     token: Optional[int]          # None: the request ended without a new token (stop token, failure)
     finished: bool
     finish_reason: Optional[str] = None
+    request: Optional[Request] = None      # with ``finished``: the request as it ended (the engine keeps it no longer)
 
 
 @dataclass
@@ -108,6 +109,12 @@ class Engine:
     def has_work(self) -> bool:
         return self.scheduler.has_work()
 
+    def abort(self, req_id: Hashable, reason: str = "aborted") -> Request:
+        """Take a request out between two steps; what it holds goes back, and it is returned as it ended."""
+        req = self.requests.pop(req_id)
+        self.scheduler.abort(req, reason)
+        return req
+
     # ------------------------------------------------------------------ one step
     def step(self) -> List[StepOutput]:
         outs: List[StepOutput] = []
@@ -116,7 +123,7 @@ class Engine:
             plan = self.scheduler.schedule()
             self.stats.preemptions += len(plan.preempted)
             for req in plan.failed:
-                outs.append(StepOutput(req.id, None, True, req.finish_reason))
+                outs.append(self._ended(StepOutput(req.id, None, True, req.finish_reason), req))
             if not plan.entries:
                 if not plan.failed and self.scheduler.has_work():
                     raise RuntimeError("the scheduler has work but could plan nothing")
@@ -136,7 +143,8 @@ class Engine:
                 new = req.output[-1] if len(req.output) > before else None
                 if new is not None:
                     self.stats.generated_tokens += 1
-                outs.append(StepOutput(req.id, new, done, req.finish_reason))
+                out = StepOutput(req.id, new, done, req.finish_reason)
+                outs.append(self._ended(out, req) if done else out)
         dt = time.perf_counter() - cur.t0
         if cur.decode:
             self.stats.decode_seconds += dt
@@ -145,9 +153,15 @@ class Engine:
         self.stats.steps += 1
         return outs
 
+    def _ended(self, out: StepOutput, req: Request) -> StepOutput:
+        """A request that is over leaves the engine's table with the output that reports its end."""
+        self.requests.pop(req.id, None)
+        out.request = req
+        return out
+
     def _record(self, plan: StepPlan) -> List[Request]:
         """The plan's tokens are cached: every request's sampler window sees its tokens once, prompt
-        included (/root/reference/src/engine.c:881); returns the requests whose next token is sampled."""
+        included (src/engine.c:881); returns the requests whose next token is sampled."""
         ready = self.scheduler.ran(plan)
         for req, _ in plan.entries:
             for t in req.token_slice(req.n_accepted, req.n_computed):
@@ -227,11 +241,14 @@ class Engine:
             params = [params or SamplingParams()] * len(prompts)
         ids = [self.add_request(p, sp) for p, sp in zip(prompts, params)]
         self.stats.prompt_tokens += sum(len(p) for p in prompts)
+        ended: Dict[Hashable, Request] = {}
         while self.has_work():
-            self.step()
+            for o in self.step():
+                if o.finished:
+                    ended[o.req_id] = o.request
         out = []
         for rid in ids:
-            req = self.requests.pop(rid)
+            req = ended[rid]
             if req.finish_reason == "cache_full":
                 raise RuntimeError(f"request {rid!r} does not fit the cache even alone "
                                    f"({self.scheduler.capacity_tokens()} positions)")

@@ -8,7 +8,7 @@ Everything a step's kernels read that changes from step to step -- token ids, po
 block tables, the attention work list -- lives in one device buffer at fixed addresses
 that is refilled with a single copy before each replay, the way the reference keeps the
 position and the cache pointers of its captured decode step in device memory
-(/root/reference/src/cuda.c:4388-4411, :4242-4264).  Rows that pad a batch up to its
+(src/cuda.c:4388-4411, :4242-4264).  Rows that pad a batch up to its
 bucket read and write the null page and their logits are dropped.
 
 No memset is recorded: the step's kernels write every byte they later read.
@@ -49,7 +49,7 @@ class StaticDecodeContext:
     """A ``StepContext`` for one token per request whose device arrays never move."""
 
     def __init__(self, ops, device, batch_cap: int, n_splits: int, table_widths: List[int],
-                 windowed: Optional[List[bool]] = None, max_tiles: Optional[int] = None, null_slot: int = 0):
+                 windowed: Optional[List[bool]] = None, max_tiles: Optional[int] = None, *, null_slot: int):
         """``n_splits``: the most key ranges a request is cut into; ``max_tiles``: the longest request's
         tiles when the context is made.  Every attention plan (group size, window, key/value heads)
         gets a number of key ranges of its own from these: a windowed layer, or one with more
@@ -77,6 +77,7 @@ class StaticDecodeContext:
         self._alloc()
         self.fresh_slots_host: List[int] = []
         self._copied = None
+        self.shared = {}        # what parts make once a pass over the layers and share (a rotation's table)
 
     def _alloc(self) -> None:
         B = self.B
@@ -137,6 +138,7 @@ class StaticDecodeContext:
         if self._copied is not None:
             self._copied.synchronize()          # the last copy has read the pinned buffer
         self._last = (entries, rcs, token_source)
+        self.shared.clear()
         B, S, o = self.B, self.S, self._offs
         n = len(entries)
         h = self._host.numpy()
@@ -167,15 +169,17 @@ class StaticDecodeContext:
                         held[b] = None
                     continue
                 t = rc.tables[g]
-                # a table only grows at its end while its request lives, unless a window gives pages back
-                if not self.windowed[g] and held[b] is not None and held[b][0] is rc and held[b][1] == len(t):
+                # a table only grows at its end while its request lives, unless a window gives pages
+                # back or a step that failed gave back what it had reserved (which `version` counts)
+                if (not self.windowed[g] and held[b] is not None and held[b][0] is rc
+                        and held[b][1] == len(t) and held[b][2] == rc.version):
                     continue
                 if len(t) > w:
                     raise ValueError("a request outgrew the block table of its graph bucket")
                 tab[b, :] = -1
                 tab[b, 0] = NULL_PAGE
                 tab[b, :len(t)] = t
-                held[b] = (rc, len(t))
+                held[b] = (rc, len(t), rc.version)
         self.starts = [int(s) for s in starts]
         self.seq_lens = [s + 1 for s in self.starts]
         self.max_seq_len = max(self.seq_lens)
@@ -277,6 +281,7 @@ class DecodeGraphs:
         gc.collect()
         gc_was_on = gc.isenabled()
         gc.disable()
+        ctx.shared.clear()          # what the eager pass left is not part of the recording
         try:
             with torch.cuda.graph(graph, pool=self.pool):
                 gx = r.model.forward(ctx, r.storage.layers)
@@ -286,6 +291,7 @@ class DecodeGraphs:
                 gc.enable()
         if self.pool is None:
             self.pool = graph.pool()
+        ctx.shared.clear()          # a table made while recording belongs to the graph's memory
         self.graphs[key] = (ctx, graph, glogits)
         self.captures += 1
         return out[:n]

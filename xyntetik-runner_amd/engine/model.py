@@ -1,7 +1,7 @@
 """A model: the parts of a ``ModelSpec``, built, bound to their tensors, and run.
 
 The forward pass is the reference's, step by step
-(/root/reference/src/model.c:6148-6483): embedding, the layers in their run order,
+(src/model.c:6148-6483): embedding, the layers in their run order,
 then final norm and output head on the rows whose logits are wanted only
 (:6478-6481).
 """

@@ -12,7 +12,7 @@ from typing import Dict, Hashable, List, Optional, Sequence
 
 import torch
 
-from ..cache import CacheManager, CacheStorage, OutOfPages
+from ..cache import CacheManager, CacheStorage, OutOfPages, cache_groups, memory_budget, size_pools
 from ..config import ModelSpec, load_config
 from ..csrc.ops import load_ops
 from ..parts.base import Runtime
@@ -35,8 +35,16 @@ def parse_dtype(name) -> torch.dtype:
 
 
 class ModelRunner:
-    def __init__(self, spec: ModelSpec, tensors_or_store, dtype, max_tokens: int, page_size: int = 64,
-                 max_requests: int = 64, device: str = "cuda:0", use_graphs: bool = True, consume_state: bool = False):
+    def __init__(self, spec: ModelSpec, tensors_or_store, dtype, max_tokens: Optional[int] = None, page_size: int = 64,
+                 max_requests: int = 64, device: str = "cuda:0", use_graphs: bool = True, consume_state: bool = False,
+                 max_step_tokens: Optional[int] = None, gpu_memory_fraction: float = 0.9,
+                 max_model_len: Optional[int] = None):
+        """``max_tokens``: cache positions over all live requests.  None sizes the cache from the
+        card instead: ``gpu_memory_fraction`` of its memory, less what is in use once the weights
+        are bound and what a step's activations take, but no more than ``max_requests`` requests of
+        ``max_model_len`` tokens (default: the model's context) can fill; ``CacheTooSmall`` if not even
+        one such request fits.  ``max_step_tokens``: the most tokens a step will bring (None: any
+        number); layers that keep a window of keys get pools for that instead of for ``max_tokens``."""
         if not torch.cuda.is_available():
             raise RuntimeError("no GPU: this engine runs on an MI355X only and has no CPU path")
         self.device = torch.device(device)
@@ -54,10 +62,24 @@ class ModelRunner:
         self.model.bind(tensors, self.rt)
         del tensors
         kv, st, of = self.model.cache_needs()
-        pages = max(1, -(-int(max_tokens) // page_size))
         self.page_size = page_size
-        self.storage = CacheStorage(kv, st, of, page_size, pages, max_requests, self.dtype, self.device)
-        self.manager = CacheManager(self.storage.group_specs, page_size, pages, max_requests)
+        specs, owners = cache_groups(kv, of)
+        elt = torch.empty((), dtype=self.dtype).element_size()
+        if max_tokens is not None:
+            sizes = size_pools(specs, owners, page_size, elt, max_requests, max_step_tokens, max_tokens=max_tokens)
+        else:
+            torch.cuda.synchronize(self.device)
+            free, total = torch.cuda.mem_get_info(self.device)
+            # what torch holds without having handed it out is as good as free
+            free += torch.cuda.memory_reserved(self.device) - torch.cuda.memory_allocated(self.device)
+            working = max(1 << 30, (max_step_tokens or 2048) << 20)     # a step's activations, generously
+            sizes = size_pools(specs, owners, page_size, elt, max_requests, max_step_tokens,
+                               budget_bytes=memory_budget(total, free, gpu_memory_fraction, working),
+                               max_model_len=max_model_len or spec.max_position)
+        self.storage = CacheStorage(kv, st, of, page_size, lambda s: sizes[specs.index(s)], max_requests,
+                                    self.dtype, self.device)
+        assert self.storage.group_specs == specs
+        self.manager = CacheManager(specs, page_size, self.storage.group_pages, max_requests)
         self.vocab_size = spec.vocab_size
         from .graphs import DecodeGraphs
         self.graphs = DecodeGraphs(self) if use_graphs else None

@@ -20,9 +20,9 @@ Continuous batching with prompts cut into portions under a token budget:
 
 The reference serves prompt chunks and decode steps by turns through a FIFO ticket
 lock and gathers waiting sequences into decode microbatches
-(/root/reference/src/scheduler.c:101-125, :153-220), with a fixed cache per slot so
+(src/scheduler.c:101-125, :153-220), with a fixed cache per slot so
 that running out cannot happen; its finishing rules are kept
-(/root/reference/src/engine.c:1834-1854).  This file is host logic only.
+(src/engine.c:1834-1854).  This file is host logic only.
 """
 from __future__ import annotations
 
@@ -60,7 +60,8 @@ class Scheduler:
 
     # ------------------------------------------------------------------ intake
     def capacity_tokens(self) -> int:
-        return self.manager.pages_per_group * self.manager.page_size if self.manager.groups else 1 << 62
+        """The most tokens a request can hold (layers that keep a window of keys set no limit)."""
+        return self.manager.capacity_tokens()
 
     def add(self, req: Request) -> None:
         if req.n_tokens >= self.max_model_len:
@@ -90,6 +91,7 @@ class Scheduler:
         plan = StepPlan()
         budget = self.max_batched_tokens
         mgr = self.manager
+        portion = mgr.max_portion()         # what the pools of windowed layers let one request run in a step
         # running requests: decoding ones first, then prompts under way
         order, prompts = [], []
         for r in self.running:
@@ -98,7 +100,7 @@ class Scheduler:
         for req in order:
             if budget <= 0 or (plan.preempted and req not in self.running):      # nothing left / preempted meanwhile
                 continue
-            n = min(req.remaining, budget)
+            n = min(req.remaining, budget, portion)
             while True:
                 try:
                     mgr.reserve(req.id, req.n_computed + n)
@@ -132,7 +134,7 @@ class Scheduler:
             req = self.waiting[0]
             if req in plan.preempted:
                 break                  # preempted in this very step: it waits for the next one
-            n = min(req.remaining, budget)
+            n = min(req.remaining, budget, portion)
             mgr.admit(req.id)
             try:
                 mgr.reserve(req.id, n)
@@ -164,7 +166,7 @@ class Scheduler:
 
     def accept(self, req: Request, token: int) -> bool:
         """Take a sampled token; returns True if the request is finished
-        (/root/reference/src/engine.c:1834-1854, :1878)."""
+        (src/engine.c:1834-1854, :1878)."""
         p = req.params
         if token in self.stop_ids and not p.ignore_eos:
             return self._finish(req, "stop")          # the stop token is neither kept nor run

@@ -5,11 +5,11 @@ encoding rotates q and k; k and v go to the cache (k rotated, v as it is); query
 ``h`` reads key/value head ``h // (H / Hk)``; scores are ``(q . k) * scale`` with
 ``scale = 1/sqrt(head_dim)`` unless given, causal by construction, limited to the last
 ``window`` keys if the layer has a window; softmax in 32-bit; ``a = Wo o``
-(/root/reference/src/model.c:6243-6338, ``attn_heads`` :3548-3589, window bound :6326).
+(src/model.c:6243-6338, ``attn_heads`` :3548-3589, window bound :6326).
 
 The three input projections are kept as one ``[Q + 2K, E]`` matrix.  A layer that
 reads another layer's cache (``kv_shared``) has no key or value projection and writes
-nothing (/root/reference/src/model.h:492-494).
+nothing (src/model.h:492-494).
 """
 from __future__ import annotations
 
@@ -28,7 +28,7 @@ class PagedAttention(Mixer):
 
     def __init__(self, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int,
                  position=None, window: Optional[int] = None, scale: Optional[float] = None,
-                 bias: bool = False, out_bias: Optional[bool] = None, kv_shared: bool = False,
+                 bias: bool = False, out_bias: Optional[bool] = None, kv_shared: bool = False, qk_transform=None,
                  q_name: str = "q_proj", k_name: str = "k_proj", v_name: str = "v_proj",
                  o_name: str = "o_proj"):
         if num_heads % num_kv_heads:
@@ -47,6 +47,9 @@ class PagedAttention(Mixer):
         self.kv_shared = bool(kv_shared)
         self.names = (q_name, k_name, v_name, o_name)
         self.position = make_part("position", position) if position is not None else None
+        # applied to the 32-bit projections before the position encoding; with one, the projections
+        # are written out and the kernels that rotate and cache their own result are not used
+        self.qk_transform = make_part("qk_transform", qk_transform) if qk_transform is not None else None
         self.q_size = self.num_heads * self.head_dim
         self.kv_size = self.num_kv_heads * self.head_dim
         self.w_in = self.b_in = self.w_out = self.b_out = None
@@ -69,16 +72,24 @@ class PagedAttention(Mixer):
                 specs[f"{v}.bias"] = ParamSpec((K,), role="vector", init="normal")
         if self.out_bias:
             specs[f"{o}.bias"] = ParamSpec((E,), role="vector", init="normal")
+        if self.qk_transform is not None:
+            for name, ps in self.qk_transform.param_specs().items():
+                if name in specs:
+                    raise ValueError(f"the query/key transform names a tensor {name!r} that the attention has itself")
+                specs[name] = ps
         return specs
 
     @property
     def capturable(self) -> bool:
-        return self.position is None or self.position.capturable
+        return ((self.position is None or self.position.capturable)
+                and (self.qk_transform is None or self.qk_transform.capturable))
 
     def bind(self, tensors, rt) -> None:
         self.rt = rt
         if self.position is not None:
             self.position.bind({}, rt)
+        if self.qk_transform is not None:
+            self.qk_transform.bind({n: tensors[n] for n in self.qk_transform.param_specs()}, rt)
         q, k, v, o = self.names
         H, Hk, D = self.num_heads, self.num_kv_heads, self.head_dim
         mats = [tensors[f"{q}.weight"]]
@@ -95,7 +106,8 @@ class PagedAttention(Mixer):
         # in paired order, so that the product's kernel has both halves of a pair at hand when
         # it rotates its own result (a few decoded tokens); the rotation kernel reads that order too.
         rot = self.position.rotary() if self.position is not None else None
-        self.paired = rot is not None and not rot.interleaved and rot.rotary_dim % 16 == 0 and D % 16 == 0
+        self.paired = (rot is not None and not rot.interleaved and rot.rotary_dim % 16 == 0 and D % 16 == 0
+                       and self.qk_transform is None)      # (a transform sees channels in the checkpoint's order)
         if self.paired:
             from ..csrc.ops import paired_order
             order = paired_order(D, rot.rotary_dim)
@@ -117,19 +129,21 @@ class PagedAttention(Mixer):
         writes = not self.kv_shared and cache.owns
         rot = self.position.rotary() if self.position is not None else None
         table = ctx.block_table(cache.group)
-        if (self.position is None or rot is not None) and writes == (not self.kv_shared):
+        if (self.position is None or rot is not None) and writes == (not self.kv_shared) and self.qk_transform is None:
             q = ops.project_rope_kv_write(
                 h, self.w_in, self.b_in, cache.k if writes else None, cache.v if writes else None, ctx.positions,
                 ctx.req_of_token, table, rot.inv_freq if rot else None, H, Hk if writes else 0, D,
                 rot.rotary_dim if rot else 0, rot.interleaved if rot else False, rot.mscale if rot else 1.0,
                 cache.page_size, paired=self.paired, cs_table=(lambda: self._step_table(ctx, rot)) if rot else None)
         else:
-            # a position encoding of its own works on the 32-bit queries and keys before they are
-            # cached; or the keys and values this layer computes are another layer's to store
+            # a transform or a position encoding of its own works on the 32-bit queries and keys before
+            # they are cached; or the keys and values this layer computes are another layer's to store
             proj = ops.linear(h, self.w_in, bias=self.b_in, out_dtype=torch.float32)
             q_in = proj[:, :Q]
             k_in = proj[:, Q:Q + K] if writes else None
             v_in = proj[:, Q + K:Q + 2 * K] if writes else None
+            if self.qk_transform is not None:
+                self.qk_transform.apply(ctx, q_in.unflatten(1, (H, D)), k_in.unflatten(1, (Hk, D)) if writes else None)
             if self.position is not None and rot is None:
                 self.position.apply(ctx, q_in.unflatten(1, (H, D)), k_in.unflatten(1, (Hk, D)) if writes else None)
             q = torch.empty((T, Q), dtype=rt.dtype, device=h.device)

@@ -14,6 +14,8 @@ Families and what each must offer:
 * ``PositionEncoding``: ``rotary()`` returns the parameters of a rotation that
   the attention kernels apply themselves, or ``None``; then ``apply(ctx, q, k)``
   is called on the 32-bit queries and keys before they are cached.
+* ``QKTransform``: ``apply(ctx, q, k)`` on an attention mixer's 32-bit queries and keys, between
+  their projection and the position encoding, in place.
 * ``Mixer``: ``kv_spec()`` and ``state_spec()`` say what the cache manager must
   keep for it; ``forward(ctx, cache, h) -> y`` returns ``[T, E]`` in the compute
   dtype; ``forward_add(ctx, cache, h, residual)`` adds it into the 32-bit
@@ -125,6 +127,18 @@ class PositionEncoding(Part):
         return None
 
 
+class QKTransform(Part):
+    """Something an attention mixer does to its 32-bit queries and keys between their projection and
+    the position encoding (a norm over every head's channels, say: the reference's optional
+    ``attn_q_norm`` / ``attn_k_norm``, src/model.c:2838-2852, src/model.h:229-235).  Its tensors are named
+    relative to the mixer's prefix."""
+
+    def apply(self, ctx, q: torch.Tensor, k: Optional[torch.Tensor]) -> None:
+        """Transform ``q [T, H, D]`` and ``k [T, Hk, D]`` (None in a layer that computes no keys) in
+        place; channels are in the checkpoint's order."""
+        raise NotImplementedError
+
+
 class Mixer(Part):
     def kv_spec(self) -> Optional[KVSpec]:
         return None
@@ -225,7 +239,8 @@ class Runtime:
 # --------------------------------------------------------------------------- registries
 
 _REGISTRIES: Dict[str, Dict[str, Callable[..., Any]]] = {
-    "norm": {}, "position": {}, "mixer": {}, "feed_forward": {}, "block": {}, "embedding": {}, "head": {},
+    "norm": {}, "position": {}, "qk_transform": {}, "mixer": {}, "feed_forward": {}, "block": {}, "embedding": {},
+    "head": {},
 }
 
 
@@ -242,6 +257,10 @@ def register_norm(kind, factory, replace=False):
 
 def register_position(kind, factory, replace=False):
     _register("position", kind, factory, replace)
+
+
+def register_qk_transform(kind, factory, replace=False):
+    _register("qk_transform", kind, factory, replace)
 
 
 def register_mixer(kind, factory, replace=False):

@@ -2,7 +2,7 @@
 
 "prenorm": ``x += mixer(norm(x)); x += feed_forward(norm(x))`` — norm, projections,
 rotation, cache write, attention, output, add, norm, feed-forward, add, every layer
-alike (/root/reference/src/model.c:6168-6473).
+alike (src/model.c:6168-6473).
 """
 from __future__ import annotations
 

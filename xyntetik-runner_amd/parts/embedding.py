@@ -1,5 +1,5 @@
 """Token embedding: one row of the table per token, as 32-bit rows of the residual
-stream; an id outside the vocabulary reads row 0 (/root/reference/src/model.c:6148-6162).
+stream; an id outside the vocabulary reads row 0 (src/model.c:6148-6162).
 """
 from __future__ import annotations
 

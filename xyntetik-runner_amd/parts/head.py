@@ -1,5 +1,5 @@
 """The output head: ``logits = W h`` in 32-bit, with ``W`` its own tensor or the
-embedding table when the model ties them (/root/reference/src/model.c:2353-2366, :6481).
+embedding table when the model ties them (src/model.c:2353-2366, :6481).
 """
 from __future__ import annotations
 
@@ -28,7 +28,7 @@ class LinearHead(Part):
         if weight is None:
             raise ValueError("a tied head needs the embedding table")
         # In the kernels' own order where they have one.  A tied head shares one buffer with the
-        # embedding (/root/reference/src/model.c:2354 aliases the pointer): where the table is
+        # embedding (src/model.c:2354 aliases the pointer): where the table is
         # packed for the head's product, the embedding gathers its rows from the packed table too.
         self.weight = rt.ops.pack_weight(weight)
         if self.tied and self.weight is not weight and hasattr(tied_to, "share_table"):

@@ -1,9 +1,9 @@
 """Gated feed-forward: ``down(act(gate(h)) * up(h))``; act = SiLU is the one activation built
-(/root/reference/src/model.c:6399-6407, ``gated_act`` :4451-4452).
+(src/model.c:6399-6407, ``gated_act`` :4451-4452).
 
 ``gate`` and ``up`` are kept as one ``[2F, E]`` matrix so that one product makes both;
 the reference does the reverse for a checkpoint that stores them fused
-(``slice_rows``, /root/reference/src/model.c:238-248).
+(``slice_rows``, src/model.c:238-248).
 """
 from __future__ import annotations
 

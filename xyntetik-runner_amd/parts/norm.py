@@ -1,5 +1,5 @@
 """RMSNorm: ``y = x / sqrt(mean(x^2) + eps) * w`` in 32-bit
-(/root/reference/src/model.c:3386-3392; kernel /root/reference/src/kernels.cu:32-48).
+(src/model.c:3386-3392; kernel src/kernels.cu:32-48).
 """
 from __future__ import annotations
 

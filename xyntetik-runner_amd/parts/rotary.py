@@ -1,6 +1,6 @@
 """Rotary position encoding: the frequency table and its scaling rules.
 
-``inv_freq[j] = theta^(-2j / rotary_dim)`` (/root/reference/src/model.c:285-289).
+``inv_freq[j] = theta^(-2j / rotary_dim)`` (src/model.c:285-289).
 The reference then divides by per-dimension factors that the model file brings for
 "llama 3.x long-context models" (:291-297) and does not compute them itself; the
 "llama3" rule below computes the same divisors from ``rope_scaling``:
@@ -11,9 +11,9 @@ The reference then divides by per-dimension factors that the model file brings f
     otherwise, with s = (orig / wavelen - low) / (high - low):
                                          (1 - s) * inv_freq / factor + s * inv_freq
 
-"linear" divides every frequency by ``factor`` (/root/reference/src/model.c:317-321).
+"linear" divides every frequency by ``factor`` (src/model.c:317-321).
 The rotation itself (pairing, angle = position * inv_freq in 32-bit) is applied by
-the kernel that writes keys to the cache (/root/reference/src/model.c:3514-3532).
+the kernel that writes keys to the cache (src/model.c:3514-3532).
 """
 from __future__ import annotations
 
@@ -66,7 +66,9 @@ class Rotary(PositionEncoding):
     def bind(self, tensors, rt) -> None:
         self.rt = rt
         table = rotary_inv_freq(self.rotary_dim, self.theta, self.scaling).to(torch.float32).to(rt.device)
-        key = ("rotary", self.rotary_dim, self.theta, repr(sorted(self.scaling.items())) if self.scaling else None)
+        # the class is part of the key: a subclass that computes another table must not share this one's
+        key = (type(self).__qualname__, self.rotary_dim, self.theta,
+               repr(sorted(self.scaling.items())) if self.scaling else None)
         self._params = RotaryParams(table, self.rotary_dim, self.interleaved, self.mscale, table_key=key)
 
     def rotary(self) -> Optional[RotaryParams]:

@@ -2,11 +2,11 @@
 
 The options are the reference's five knobs with its defaults for an unknown model
 family: temperature, top-k, top-p, min-p and a repeat penalty over the last 256
-tokens (/root/reference/src/sample.h:9-20).  ``temperature <= 0`` asks for the argmax
-and applies no penalty (/root/reference/src/sample.c:141-172).  The random numbers come
+tokens (src/sample.h:9-20).  ``temperature <= 0`` asks for the argmax
+and applies no penalty (src/sample.c:141-172).  The random numbers come
 from xorshift64, one draw for each sampled token; state 0 is a fixed point, so seed 0 is
 refused, and an absent seed is taken from the clock
-(/root/reference/src/sample.c:13-20, /root/reference/src/main.c:833-845).
+(src/sample.c:13-20, src/main.c:833-845).
 """
 from __future__ import annotations
 
@@ -74,7 +74,7 @@ class SamplerState:
 
     def accept(self, token: int) -> None:
         """Record a token (prompt or generated) in the ring of the last 256
-        (/root/reference/src/sample.c:27-31)."""
+        (src/sample.c:27-31)."""
         self.recent[self.head] = int(token)
         self.head = (self.head + 1) % RECENT_WINDOW
         if self.n_recent < RECENT_WINDOW:

@@ -11,10 +11,10 @@ wanted places, in the order of the entries and of ``want``, as little-endian 32-
 floats ``[wanted, vocab]``.  After every step a line ``done <step>`` is printed.
 
 The reference's nearest tools walk a fixed token sequence for scoring
-(/root/reference/src/main.c:1344-1433) and teacher-force tokens in its tests
-(/root/reference/tests/test_gpu_identity.c:91-105); decoded tokens are given, never
+(src/main.c:1344-1433) and teacher-force tokens in its tests
+(tests/test_gpu_identity.c:91-105); decoded tokens are given, never
 sampled, so an early difference cannot change later inputs
-(/root/reference/tests/test_attn_tol.c:136).
+(tests/test_attn_tol.c:136).
 """
 from __future__ import annotations
 

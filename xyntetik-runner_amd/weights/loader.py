@@ -1,9 +1,9 @@
 """Binding a model's tensors by name, with one error that tells everything wrong.
 
 The reference looks every tensor up by name, refuses the load when one is missing
-(``need_tensor``, /root/reference/src/model.c:158-170) and checks each shape
+(``need_tensor``, src/model.c:158-170) and checks each shape
 against the geometry with a message that names tensor, layer, got and expected
-(``check_shape``, /root/reference/src/model.c:193-205).  Here all findings of one
+(``check_shape``, src/model.c:193-205).  Here all findings of one
 load are gathered: missing tensors, tensors the model has no use for, and wrong
 shapes or dtypes come in a single ``WeightError``.
 

@@ -5,7 +5,7 @@ tensor's values do not depend on which other tensors exist or in which order the
 are made.  Matrices are N(0, std) (std 0.02 unless told otherwise) rounded to the
 storage dtype; norm weights are 1, or 1 + N(0, jitter).  The reference's fixture
 generator plays the same role with an LCG and weights uniform in +-0.04, norm
-weights 1.0 (/root/reference/scripts/make-test-model.py:238-252).
+weights 1.0 (scripts/make-test-model.py:238-252).
 """
 from __future__ import annotations
 

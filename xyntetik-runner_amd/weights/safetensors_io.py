@@ -6,7 +6,7 @@ and the tensor bytes, offsets counted from the end of the header.
 
 The checks are those the reference makes on its own container: every tensor's
 byte range lies inside the mapping and is overflow-checked
-(/root/reference/src/gguf.c:229-280), names are unique (:191-215), and a lookup is
+(src/gguf.c:229-280), names are unique (:191-215), and a lookup is
 by exact name (:579-583).  The file is memory-mapped; a tensor's bytes are touched
 only when it is asked for.
 """
