@@ -30,8 +30,13 @@ LLAMA_3_1_8B = {
 LLAMA_2_7B = dict(LLAMA_3_1_8B, num_key_value_heads=32, intermediate_size=11008, vocab_size=32000, rope_theta=10000.0,
                   rope_scaling=None, max_position_embeddings=4096)
 LLAMA_3_1_70B = dict(LLAMA_3_1_8B, num_hidden_layers=80, hidden_size=8192, num_attention_heads=64, intermediate_size=28672)
+# a small shape of the same architecture with heads of 64 and tied embeddings (the sizes of a 1B-class Llama)
+LLAMA_1B = dict(LLAMA_3_1_8B, num_hidden_layers=16, hidden_size=2048, head_dim=64, intermediate_size=8192,
+                tie_word_embeddings=True, max_position_embeddings=131072,
+                rope_scaling={"rope_type": "llama3", "factor": 32.0, "low_freq_factor": 1.0, "high_freq_factor": 4.0,
+                              "original_max_position_embeddings": 8192})
 SHAPES = {"llama-3.1-8b": ("Llama-3.1-8B shape", LLAMA_3_1_8B), "llama-2-7b": ("Llama-2-7B shape", LLAMA_2_7B),
-          "llama-3.1-70b": ("Llama-3.1-70B shape", LLAMA_3_1_70B)}
+          "llama-3.1-70b": ("Llama-3.1-70B shape", LLAMA_3_1_70B), "llama-1b-head64": ("Llama 1B-class shape, heads of 64", LLAMA_1B)}
 PEAK = {"hbm_gbs": 8000.0, "bf16_flops": 2.5e15, "fp32_flops": 157.3e12}
 
 
@@ -123,17 +128,23 @@ def measure_decode(runner, cfg, batch, prompt_len, steps, warmup, seed, alone=Fa
     import torch
     from xyntetik_runner_amd.engine import Engine
     from xyntetik_runner_amd.sampling import SamplingParams
-    eng = Engine(runner, max_batched_tokens=max(2048, prompt_len), max_running=batch,
+    # (prompts up to 8,192 tokens go in one step each, longer ones in portions of 2,048)
+    budget = max(2048, prompt_len) if prompt_len <= 8192 else 2048
+    eng = Engine(runner, max_batched_tokens=budget, max_running=batch,
                  max_model_len=cfg["max_position_embeddings"], stop_ids=[])
     rng = np.random.default_rng(seed)
-    # a request admitted first decodes while the others' prompts are still computed (up to
-    # `batch` steps): nobody may finish before the last timed step
-    sp = SamplingParams(temperature=0.0, max_new_tokens=batch + warmup + steps + 8, ignore_eos=True)
+    # a request admitted first decodes while the others' prompts are still computed (a step for
+    # every portion of every prompt): nobody may finish before the last timed step
+    sp = SamplingParams(temperature=0.0, max_new_tokens=batch * -(-prompt_len // budget) + warmup + steps + 8, ignore_eos=True)
     ids = [eng.add_request([int(t) for t in rng.integers(0, cfg["vocab_size"], size=prompt_len)], sp) for _ in range(batch)]
+    def step():
+        for o in eng.step():
+            if o.finished:
+                raise RuntimeError(f"decode batch {batch}: request {o.req_id!r} ended before the last timed step ({o.finish_reason})")
     while any(eng.requests[i].n_computed < prompt_len for i in ids):
-        eng.step()
+        step()
     for _ in range(warmup):
-        eng.step()
+        step()
     ctx0 = sum(eng.requests[i].n_tokens for i in ids)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
@@ -283,6 +294,13 @@ def main():
     ap.add_argument("--no-points", action="store_true", help="skip decode at batch 1 and 64")
     ap.add_argument("--dtype", default="bfloat16")
     ap.add_argument("--shape", default="llama-3.1-8b", choices=sorted(SHAPES), help="sizes of the model (same architecture)")
+    ap.add_argument("--max-context", type=int, default=0, metavar="N",
+                    help="the model's context length (max_position_embeddings) instead of the shape's own")
+    ap.add_argument("--contexts", default="", metavar="LIST",
+                    help="decode points at these context lengths (comma separated) instead of the points at the model's limit")
+    ap.add_argument("--context-batches", default="1,8", metavar="LIST", help="batch sizes of the --contexts points")
+    ap.add_argument("--long-prefill", type=int, default=0, metavar="T",
+                    help="length of the prompt that is run in portions of 2,048 (default: the model's context)")
     ap.add_argument("--record", default="", metavar="FILE",
                     help="also write the command and the JSON line into FILE (markdown)")
     ap.add_argument("--mixed", type=int, default=0, metavar="N",
@@ -296,25 +314,33 @@ def main():
     layers_full = cfg["num_hidden_layers"]
     layers = args.layers or layers_full
     cfg["num_hidden_layers"] = layers
+    if args.max_context:
+        cfg["max_position_embeddings"] = args.max_context
     P, B = args.prompt_len, args.batch
     elt = 2 if args.dtype == "bfloat16" else 4
     ctx_max = cfg["max_position_embeddings"]
     long_steps, long_warmup = 32, 4
-    long_P = ctx_max - 128                      # a context that ends just under the model's limit
     span = P + args.warmup + args.steps + 80 + max(64, B)
     pool = max(max(64, B) * (-(-span // 64) * 64) + 4096, args.mixed * (2048 + 128 + 64))
-    # the points at the context limit need room for 64 requests of that length, if the card has it
+    # The points away from the tuned one: (context, batch) pairs.  By default the model's limit at
+    # batch 8 and, if the card has room for 64 requests of that length beside the weights, at batch 64.
     import torch
     kv_per_token = 2 * cfg["num_key_value_heads"] * cfg["head_dim"] * layers * elt
     body, head = matmul_params(cfg, layers)
-    weight_bytes = (body + 2 * head) * elt
-    long_pool = 64 * (-(-(long_P + 128) // 64) * 64) + 4096
+    weight_bytes = (body + (1 if cfg.get("tie_word_embeddings") else 2) * head) * elt
     total_mem = torch.cuda.get_device_properties(0).total_memory
-    long_b64 = not args.no_points and weight_bytes + long_pool * kv_per_token < 0.8 * total_mem
-    if long_b64:
-        pool = max(pool, long_pool)
-    elif not args.no_points:
-        pool = max(pool, 8 * (-(-(long_P + 128) // 64) * 64) + 4096)
+
+    def pool_for(ctx, b):
+        return b * (-(-(ctx + 128) // 64) * 64) + 4096
+    if args.contexts:
+        ctx_points = [(int(c), int(b)) for c in args.contexts.split(",") for b in args.context_batches.split(",")]
+    else:
+        ctx_points = [(ctx_max, 8), (ctx_max, 64)]
+    left_out = [cb for cb in ctx_points if weight_bytes + pool_for(*cb) * kv_per_token >= 0.8 * total_mem or cb[0] > ctx_max]
+    ctx_points = [cb for cb in ctx_points if cb not in left_out]
+    long_T = args.long_prefill or min(ctx_max, 32768)
+    if not args.no_points:
+        pool = max([pool, long_T + 4096] + [pool_for(*cb) for cb in ctx_points])
     spec, runner = build_runner(cfg, args.dtype, max_tokens=pool, max_requests=max(64, args.mixed))
 
     read_gbs, mm_flops = measure_achievable(runner) if args.dtype == "bfloat16" else (None, None)
@@ -359,15 +385,16 @@ def main():
                                        f"(allowed: mean {bound:.1e}, max {10 * bound:.1e} of the logit range)")
         for b in (1, 64):
             point(f"decode_b{b}", b, P, max(8, min(args.steps, 64)), min(args.warmup, 8), 3 + b, alone=b == 64)
-        # away from the tuned point: contexts at the model's limit, and a prompt of that length in portions
-        point(f"decode_b8_ctx{ctx_max}", 8, long_P, long_steps, long_warmup, 21)
-        if long_b64:
-            point(f"decode_b64_ctx{ctx_max}", 64, long_P, long_steps, long_warmup, 22)
-        else:
-            log(f"decode_b64_ctx{ctx_max}: left out, the cache of 64 such requests does not fit beside the weights")
-        long_s = measure_prefill_in_portions(runner, cfg, ctx_max, 2048, seed=23)
-        points[f"prefill_{ctx_max}_in_2048_portions"] = round(ctx_max / long_s, 1)
-        log(f"prefill of {ctx_max} tokens in portions of 2048: {long_s * 1e3:.1f} ms, {ctx_max / long_s:.0f} tok/s")
+        # away from the tuned point: long contexts (they end 128 tokens under the named length), and
+        # a long prompt in portions
+        for i, (c, b) in enumerate(ctx_points):
+            point(f"decode_b{b}_ctx{c}", b, c - 128, long_steps if c <= 8192 else 16, long_warmup, 21 + i)
+        for c, b in left_out:
+            log(f"decode_b{b}_ctx{c}: left out, the cache of {b} such requests does not fit beside the weights "
+                f"or the context is beyond the model's {ctx_max}")
+        long_s = measure_prefill_in_portions(runner, cfg, long_T, 2048, seed=23)
+        points[f"prefill_{long_T}_in_2048_portions"] = round(long_T / long_s, 1)
+        log(f"prefill of {long_T} tokens in portions of 2048: {long_s * 1e3:.1f} ms, {long_T / long_s:.0f} tok/s")
     if args.mixed:
         # the workload twice: the first pass also records the decode graphs of its batch sizes (as the
         # warm-up steps do for the decode figures), the second is the figure; both are reported

@@ -55,6 +55,10 @@ def test_sample_static_matches_sample_on_two_calls_in_a_row():
         greedy = [r for r in range(W) if temp_h[r] == 0]
         assert [got[r] for r in greedy] == [int(np.argmax(lg[r])) for r in greedy]
         assert got[0] == 17 and got[W - 1] == 0
+        # the sampled rows against the plain sampler (not only against the sibling entry point)
+        import plain_llama as Plain
+        for r in range(1, W, 4):
+            assert got[r] == Plain.sample_pick(lg[r], 0.7, float(draw[r].item())), r
         assert torch.equal(logits.cpu(), torch.tensor(lg))          # logits untouched
 
 

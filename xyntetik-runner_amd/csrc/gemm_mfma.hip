@@ -1190,6 +1190,8 @@ extern "C" int xr_gemm_bf16(void* out, const void* a, const void* w, const float
             // columns of the full rounds go to that tile and the rest to a second launch with a
             // smaller one (3 rounds + 1 of half-size tiles instead of 4).  If even the smallest
             // tile does not fill the chip, K is split as well.
+            // (The 256 compute units and the tiles' relative rates below are tuning measured on an
+            // MI355X with the 8B shape's products, not limits: elsewhere they cost speed only.)
             struct Cand { int variant, bm, bn; double rate; };
             const Cand cands[4] = {{14, 256, 256, 1.0}, {26, 256, 192, 0.93}, {12, 256, 128, 0.90}, {17, 128, 128, 0.74}};
             auto width = [&](const Cand& c) { return sw ? c.bn / 2 : c.bn; };

@@ -41,6 +41,9 @@ class AttentionPlan:
     n_cta_items: int = 0
 
 
+# The first four are the attention kernels' shapes.  The last three are tuning, not limits: they
+# say how much work gives every one of an MI355X's 256 compute units a workgroup, measured on the
+# 8B shape's attention; on another chip or shape they cost speed, never correctness.
 ATTN_ROWS = 32          # query rows (token x head-in-group) per work item
 ATTN_TILE = 32          # keys per tile; items begin and end on tile edges
 ATTN_CTA_ROWS = 128     # rows of an item that a whole workgroup takes
