@@ -388,7 +388,10 @@ def main():
         # away from the tuned point: long contexts (they end 128 tokens under the named length), and
         # a long prompt in portions
         for i, (c, b) in enumerate(ctx_points):
-            point(f"decode_b{b}_ctx{c}", b, c - 128, long_steps if c <= 8192 else 16, long_warmup, 21 + i)
+            # (the request admitted first decodes a token for every portion of the others' prompts;
+            # it must not reach the model's limit before the last timed step)
+            ahead = (b - 1) * -(-c // 2048) if c > 8192 else 0
+            point(f"decode_b{b}_ctx{c}", b, c - 128 - ahead, long_steps if c <= 8192 else 16, long_warmup, 21 + i)
         for c, b in left_out:
             log(f"decode_b{b}_ctx{c}: left out, the cache of {b} such requests does not fit beside the weights "
                 f"or the context is beyond the model's {ctx_max}")
