@@ -88,6 +88,20 @@ def test_schedules_match_plain(models, tmp_path, which, dtype, schedule):
     check(got, want, dtype, f"{which}/{schedule}")
 
 
+@pytest.mark.parametrize("seed", [1, 2, 3, 4, 5, 6])
+def test_random_schedules_in_32_bit(models, tmp_path, seed):
+    """Mixed schedules drawn at random (portion sizes, how many requests are live, which are left out of
+    a step, the page size), in 32-bit where any fault of the cache or the batch shows above rounding."""
+    rng = np.random.default_rng(seed)
+    which = ["A", "B", "C"][seed % 3]
+    d, cfg, reqs, plens, want = models[which]
+    chunk = tuple(int(n) for n in rng.integers(2, 40, size=5))
+    page_size = int(rng.choice([2, 4, 8, 16, 32, 64]))
+    steps = traces.mixed(reqs, plens, max_live=int(rng.integers(2, 5)), chunk=chunk, seed=seed)
+    out, runner = run_replay(d, "float32", steps, tmp_path, page_size)
+    check(traces.collect(steps, out, cfg["vocab_size"]), want, "float32", f"{which}/random {seed}, pages of {page_size}, portions {chunk}")
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_long_portions_of_several_requests_in_one_step(models, tmp_path, dtype):
     """A step of more than 512 rows made of three requests: one that goes on at a position that
