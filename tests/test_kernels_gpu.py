@@ -286,12 +286,13 @@ def test_linear_whose_tiles_do_not_fill_the_last_round(ops):
     assert rel(got, r[:, :F] / (1 + torch.exp(-r[:, :F])) * r[:, F:]) < 6e-3
 
 
-@pytest.mark.parametrize("M", [17, 33, 64])
+@pytest.mark.parametrize("M", [17, 33, 64, 100, 300])
 @pytest.mark.parametrize("E,K", [(64, 48), (200, 520), (4096, 1024), (5120, 264)])
 @pytest.mark.parametrize("wdtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("bias", [False, True])
 def test_rmsnorm_by_the_kernel_that_adds_up_a_split_product(ops, M, E, K, wdtype, bias):
-    """17 to 64 rows: residual += a @ w^T (+ bias) and the norm of the result from the product and
+    """17 to 64 rows, and more where the product's tiles are few enough for K to be split:
+    residual += a @ w^T (+ bias) and the norm of the result from the product and
     one more kernel; against the product and the norm's own kernel (the residual to the bit when
     the K ranges are the same, else to rounding) and against float64."""
     torch.manual_seed(M + E)
@@ -562,21 +563,36 @@ def test_rope_kv_write(ops, dt, H, Hk, D, rot, inter, ps, starts, q_lens):
                                                (8, 8, 128, 64, True), (5, 1, 128, 128, False), (2, 2, 32, 0, False)])
 @pytest.mark.parametrize("ps,starts,q_lens", [(16, [0, 13, 40], [9, 3, 1]), (64, [70], [1]), (8, [2, 9, 100, 7], [5, 6, 1, 4]),
                                               (16, [3, 0], [30, 8]), (16, [5, 0, 77], [60, 20, 3]),
-                                              (16, [3, 0, 8, 21], [290, 200, 70, 1]), (64, [64], [520])])
+                                              (16, [3, 0, 8, 21], [290, 200, 70, 1]), (64, [64], [520]),
+                                              (32, [3, 0, 8], [200, 70, 30]), (64, [1000], [511])])
 @pytest.mark.parametrize("bias", [False, True])
 def test_projection_with_rotation_and_cache_write(ops, dt, H, Hk, D, rot, inter, ps, starts, q_lens, bias):
+    check_projection_with_rotation_and_cache_write(ops, dt, H, Hk, D, rot, inter, ps, starts, q_lens, bias, 72)
+
+
+@pytest.mark.parametrize("dt", ["float32", "bfloat16"])
+@pytest.mark.parametrize("q_lens", [[100, 30], [20, 9], [300], [70, 200, 115]])
+def test_projection_with_rotation_and_cache_write_of_a_product_split_over_k(ops, dt, q_lens):
+    """The same with a width of 1,024, where the products of 17 to 511 rows are split over K
+    (8 to 32 tiles of 128 columns for 256 compute units) and the kernel that adds the ranges up
+    rotates and caches."""
+    starts = [5, 0, 64][:len(q_lens)]
+    check_projection_with_rotation_and_cache_write(ops, dt, 4, 2, 64, 64, False, 64, starts, q_lens, True, 1024)
+
+
+def check_projection_with_rotation_and_cache_write(ops, dt, H, Hk, D, rot, inter, ps, starts, q_lens, bias, E):
     """q, k and v from one product, rotated and cached.  Up to 16 bfloat16 rows the product's own
     kernel does all of it (with the weight's rows in paired order where a pair is (j, j + rot/2)),
-    up to 64 the kernel that adds the product's K ranges up, from 512 the tile kernel;
-    other numbers of rows, or 32-bit, run the product and the rotation kernel.  Both against float64 from
+    up to 511 the kernel that adds the product's K ranges up, from 512 the tile kernel;
+    32-bit runs the product and the rotation kernel.  Both against float64 from
     the weights in their natural order; and the two bfloat16 ways against each other."""
     from xyntetik_runner_amd.csrc.ops import paired_order
     torch.manual_seed(H * 100 + D + ps)
     tables, n_pages = scatter_pages([s + n for s, n in zip(starts, q_lens)], ps, 2)
     ctx = FakeCtx(starts, q_lens, tables, ps)
-    T, E, Q, K = sum(q_lens), 72, H * D, Hk * D
+    T, Q, K = sum(q_lens), H * D, Hk * D
     h = (torch.randn(T, E, device=DEV) * 0.5).to(DT[dt])
-    w = (torch.randn(Q + 2 * K, E, device=DEV) * 0.2).to(DT[dt])
+    w = (torch.randn(Q + 2 * K, E, device=DEV) * (0.2 if E < 500 else 0.05)).to(DT[dt])
     b = torch.randn(Q + 2 * K, device=DEV) * 0.3 if bias else None
     inv = (10000.0 ** (-torch.arange(rot // 2, dtype=torch.float64) * 2 / rot)).float().to(DEV) if rot else None
     paired = rot > 0 and not inter and rot % 16 == 0

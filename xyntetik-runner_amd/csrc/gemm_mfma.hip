@@ -998,7 +998,10 @@ static int launch_tile_variant(int variant, const GemmArgs& g, hipStream_t strea
     // (the loop that reads its fragments a k-step ahead is the faster one but for the 256x192 tile)
     if (variant == 12) return launch_tile_async<256, 128, 4, 2, 3, true>(g, stream);
     if (variant == 14) return launch_tile_async<256, 256, 4, 2, 2, true>(g, stream);
-    if (variant == 17) return launch_tile_async<128, 128, 2, 2, 2, true>(g, stream);
+    // (four slices in flight: with 65 to 512 rows these products are bound by how fast the weights
+    // arrive, and two slices, one of them in use, left a compute unit 32 KB on its way: the down
+    // product at 128 rows 46 -> 37 us, gate+up 72 -> 57, q/k/v at 512 rows 65 -> 45)
+    if (variant == 17) return launch_tile_async<128, 128, 2, 2, 4, false>(g, stream);
     if (variant == 26) return launch_tile_async<256, 192, 4, 2, 2>(g, stream);
     xr_set_error("gemm: unknown variant %d", variant);
     return XR_BAD_ARG;
@@ -1068,6 +1071,11 @@ extern "C" int xr_rope_table(void* cs, const int* positions, const float* inv_fr
     return XR_OK;
 }
 
+// From this many rows on the q/k/v product has tiles enough with K whole, and its tile kernel rotates
+// and caches its own result; with fewer rows the kernel that adds up its K ranges does.
+#define XR_ROPE_TILE_ROWS 512
+extern "C" int xr_rope_tile_rows() { return XR_ROPE_TILE_ROWS; }
+
 // epi: 0 store, 1 add into float out, 2 gated (w has 2N rows: gate rows then up rows; act: XR_ACT_*).
 // variant: 0 = choose by shape; 1 = skinny; 10..20 = tile shapes; 30, 31 = few rows with K split;
 //          +1000 = row tiles of one weight tile follow each other.
@@ -1119,9 +1127,10 @@ extern "C" int xr_gemm_bf16(void* out, const void* a, const void* w, const float
         }
     }
     g.rope.q_out = nullptr; g.rope.cs = nullptr;
-    // more than 64 rows: the tile kernel rotates and caches its own result, with the rows' cosines and
+    // many rows: the tile kernel rotates and caches its own result, with the rows' cosines and
     // sines from a table that a small kernel writes into the workspace first; K is then not split
-    const bool rope_direct = rope && M > 64;
+    // from XR_ROPE_TILE_ROWS rows on; below, the kernel that adds up the K ranges rotates and caches
+    const bool rope_direct = rope && M >= XR_ROPE_TILE_ROWS;
     if (rope) {
         XR_REQUIRE(variant == 0 && epi == EPI_STORE && !(norm && norm->xg),
                    "gemm: rotation and cache write are folded only into a plain product whose kernel the library chooses");
@@ -1243,7 +1252,11 @@ extern "C" int xr_gemm_bf16(void* out, const void* a, const void* w, const float
                 return rc != XR_OK ? rc : launch_tile_variant(cands[second].variant, g2, stream);
             }
             auto count_of = [&](int bm, int bn) { return ((M + bm - 1) / bm) * ((N + (sw ? bn / 2 : bn) - 1) / (sw ? bn / 2 : bn)); };
-            if (variant == 17 && count_of(128, 128) < 160) g.splits = pick_splits(count_of(128, 128));
+            if (variant == 17 && count_of(128, 128) < 160) {
+                g.splits = pick_splits(count_of(128, 128));
+                // the kernel that adds the ranges up takes whole rows and writes the norm that follows
+                if (g.splits > 1 && want_whole_norm) { g.norm_whole = 1; norm->ss_out_rows = -1; }
+            }
         }
     }
     if (variant == 1) {

@@ -169,6 +169,8 @@ class Ops:
         self.use_mfma = True
         self.fold_norms = True      # False: linear_add_rmsnorm always runs the norm's own kernel
         self.fuse_rope = True       # False: project_rope_kv_write always runs two kernels
+        self.ROPE_TILE_ROWS = int(lib.dll.xr_rope_tile_rows())
+        self.FINISH_ROWS = self.ROPE_TILE_ROWS - 1
 
     # -- checks -----------------------------------------------------------------
     @staticmethod
@@ -267,8 +269,8 @@ class Ops:
 
     # -- matrix product ---------------------------------------------------------
     GEMM_WORKSPACE_BYTES = 96 << 20
-    FINISH_ROWS = 64        # up to here a product's epilogue may be the kernel that adds its K ranges up
     ROPE_TILE_ROWS = 512    # from here the q/k/v product has tiles enough with K whole, and its tile kernel rotates and caches
+    FINISH_ROWS = 511       # up to here the kernel that adds a product's K ranges up rotates and caches (the library's own number)
 
     def _gemm_workspace(self, device):
         """Room for the sums of K ranges when a product with few rows is split (one buffer per process;
@@ -363,8 +365,9 @@ class Ops:
         With ``defer`` the caller says that what reads the result is a ``linear`` or
         ``linear_gated``: for at most 16 bfloat16 rows the product's kernel then also writes the
         weighted rows and their partial sums of squares, and an ``UnscaledRows`` comes back, whose
-        scale the next product applies.  From 17 to 64 rows the kernel that adds up the product's K
-        ranges takes whole rows and writes the finished norm.  In every other case the norm's own
+        scale the next product applies.  With more rows, where the product is split over K (always
+        from 17 to 64 rows, above that when its tiles are too few for the chip), the kernel that adds up
+        the K ranges takes whole rows and writes the finished norm.  In every other case the norm's own
         kernel runs.  A tensor comes back in both."""
         wt = w.data if isinstance(w, PackedWeight) else w
         rows = a.data if isinstance(a, UnscaledRows) else a
@@ -374,7 +377,7 @@ class Ops:
                 and residual.dtype == torch.float32 and self._mfma_ok(rows, wt))
         deferred = fits and defer and M <= UnscaledRows.MAX_ROWS
         # More rows: where the product is split over K (always from 17 to 64 rows, above that when
-        # its tiles are few and K is long), the kernel that adds the parts up takes whole rows and
+        # its tiles are too few for the chip), the kernel that adds the parts up takes whole rows and
         # writes the finished norm; the library says whether it did.
         whole = fits and M > UnscaledRows.MAX_ROWS and N % 4 == 0 and residual.stride(0) % 4 == 0
         if deferred or whole:
@@ -479,10 +482,10 @@ class Ops:
         ``w`` holds ``H`` query heads, then ``Hk`` key heads and ``Hk`` value heads (``Hk`` = 0 and
         no caches: queries alone); with ``paired`` its query and key rows are in ``paired_order``.
         Up to 16 bfloat16 rows (``h`` may be an ``UnscaledRows``) the product's kernel rotates and
-        stores its own result, up to 64 the kernel that adds the product's K ranges up does, from
+        stores its own result, up to 511 the kernel that adds the product's K ranges up does, from
         512 the tile kernel (with the rows' cosines and sines from a table made first), which
-        saves a kernel and the 32-bit copy of the projections; otherwise the product and
-        ``rope_kv_write`` run one after the other.  ``cs_table``: a callable that returns the
+        saves a kernel; in float32, and where the kernels' conditions on sizes do not hold, the
+        product and ``rope_kv_write`` run one after the other.  ``cs_table``: a callable that returns the
         step's ``rope_table`` (asked for only where the tile kernel rotates)."""
         rows = h.data if isinstance(h, UnscaledRows) else h
         wt = w.data if isinstance(w, PackedWeight) else w
