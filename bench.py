@@ -395,6 +395,11 @@ def main():
         for c, b in left_out:
             log(f"decode_b{b}_ctx{c}: left out, the cache of {b} such requests does not fit beside the weights "
                 f"or the context is beyond the model's {ctx_max}")
+        # short prompts (time to the first token's logits): steps of 128 and of 512 rows
+        for T in (128, 512):
+            short_s = measure_prefill(runner, cfg, T, repeats=5, seed=30 + T)
+            points[f"prefill_{T}_tokens_ms"] = round(short_s * 1e3, 3)
+            log(f"prefill {T} tokens: {short_s * 1e3:.2f} ms (the median of 5)")
         long_s = measure_prefill_in_portions(runner, cfg, long_T, 2048, seed=23)
         points[f"prefill_{long_T}_in_2048_portions"] = round(long_T / long_s, 1)
         log(f"prefill of {long_T} tokens in portions of 2048: {long_s * 1e3:.1f} ms, {long_T / long_s:.0f} tok/s")
