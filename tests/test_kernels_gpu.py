@@ -655,11 +655,10 @@ def ref_attention(q, k_seq, v_seq, starts, q_lens, scale, window):
         for i in range(n):
             p = s + i
             lo = max(0, p - window + 1) if window else 0
-            kk = k[lo:p + 1].repeat_interleave(H // Hk, dim=1)
-            vv = v[lo:p + 1].repeat_interleave(H // Hk, dim=1)
-            sc = torch.einsum("hd,thd->ht", q[t].double(), kk) * scale
+            qg = q[t].double().view(Hk, H // Hk, -1)            # query head h reads key/value head h // (H / Hk)
+            sc = torch.einsum("kgd,tkd->kgt", qg, k[lo:p + 1]) * scale
             pr = torch.softmax(sc, dim=-1)
-            outs.append(torch.einsum("ht,thd->hd", pr, vv))
+            outs.append(torch.einsum("kgt,tkd->kgd", pr, v[lo:p + 1]).reshape(H, -1))
             t += 1
     return torch.stack(outs)
 
@@ -669,7 +668,12 @@ def fill_cache(k_seq, v_seq, tables, n_pages, ps, dt):
     kc = torch.full((n_pages, Hk, ps, D), float("nan"), dtype=dt)
     vc = torch.full((n_pages, Hk, D, ps), float("nan"), dtype=dt)
     for b, (k, v) in enumerate(zip(k_seq, v_seq)):
-        for p in range(k.shape[0]):
+        full = k.shape[0] // ps                         # whole pages at once, the rest position by position
+        if full:
+            pages = torch.tensor(tables[b][:full], dtype=torch.long)
+            kc[pages] = k[:full * ps].to(dt).view(full, ps, Hk, D).permute(0, 2, 1, 3)
+            vc[pages] = v[:full * ps].to(dt).view(full, ps, Hk, D).permute(0, 2, 3, 1)
+        for p in range(full * ps, k.shape[0]):
             kc[tables[b][p // ps], :, p % ps, :] = k[p].to(dt)
             vc[tables[b][p // ps], :, :, p % ps] = v[p].to(dt)
     return kc.to(DEV), vc.to(DEV)
@@ -690,6 +694,9 @@ ATTN_CASES = [
     (6, 2, 48, 64, None, [5000], [1]),             # more than 64 pages: the page numbers are fetched again on the way
     (64, 8, 128, 64, None, [900, 0, 130], [1, 70, 3]),   # 8 query heads a key/value head: 4 tokens x 8 heads in a 32-row block
     (32, 32, 128, 64, None, [700, 0, 64], [1, 150, 2]),  # one query head a key/value head, 32 of them: 32 tokens in a block
+    (8, 2, 128, 64, None, [70001, 3], [1, 2]),           # a decoded token behind 70,000 keys (1,094 pages, 32 key ranges)
+    (8, 2, 128, 64, None, [66000], [40]),                # a prompt portion behind 66,000 keys (128-row items cut into key ranges)
+    (4, 1, 64, 32, 4096, [40000], [1]),                  # a window of 4,096 far into a long request
 ]
 
 
@@ -742,7 +749,10 @@ def test_attention(ops, dt, case):
     got = ops.attention(q.to(DEV).reshape(T, H * D).contiguous(), kc, vc, ctx, 0, H, Hk, D, ps, scale, window)
     got = got.cpu().reshape(T, H, D)
     assert torch.isfinite(got.float()).all(), "read a slot no request owns"
-    assert rel(got, want) < (3e-6 if dt == "float32" else 1.2e-2)
+    # 32-bit: 3e-6 of the largest output up to 4,096 keys; a row's sums over n keys are 32-bit running
+    # sums whose rounding grows with the root of n (the cases behind 66,000 and 70,000 keys: x 4)
+    tol32 = 3e-6 * max(1.0, math.sqrt(max(lens) / 4096))
+    assert rel(got, want) < (tol32 if dt == "float32" else 1.2e-2)
 
 
 def test_attention_items_longer_than_64_pages(ops):
