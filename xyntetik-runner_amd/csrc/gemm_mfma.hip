@@ -1197,8 +1197,8 @@ extern "C" int xr_gemm_bf16(void* out, const void* a, const void* w, const float
             // (relative to 256x256); a launch takes as many of these as its tiles make rounds of
             // 256.  When the last round of the best tile would leave most of the chip idle, the
             // columns of the full rounds go to that tile and the rest to a second launch with a
-            // smaller one (3 rounds + 1 of half-size tiles instead of 4).  If even the smallest
-            // tile does not fill the chip, K is split as well.
+            // smaller one (3 rounds + 1 of half-size tiles instead of 4).  A tile shape whose tiles
+            // are too few for the chip competes with K split among workgroups (below).
             // (The 256 compute units and the tiles' relative rates below are tuning measured on an
             // MI355X with the 8B shape's products, not limits: elsewhere they cost speed only.)
             struct Cand { int variant, bm, bn; double rate; };
@@ -1207,10 +1207,34 @@ extern "C" int xr_gemm_bf16(void* out, const void* a, const void* w, const float
             auto usable = [&](const Cand& c) { return !(sw && c.variant == 26); };
             auto count = [&](const Cand& c, int cols) { return ((M + c.bm - 1) / c.bm) * ((cols + width(c) - 1) / width(c)); };
             auto time_of = [&](const Cand& c, int cols) { return (double)((count(c, cols) + 255) / 256) * c.bm * c.bn / c.rate; };
-            int best = 0, second = -1, cols_first = N;
-            double t_best = time_of(cands[0], N);
-            for (int i = 1; i < 4; ++i)
-                if (usable(cands[i]) && time_of(cands[i], N) < t_best) { best = i; t_best = time_of(cands[i], N); }
+            // Times in seconds: a 256x256 tile's products over K columns take 65536 K x 0.5e-12 s at
+            // full rate (134 us at K = 4,096, measured 137).  A launch whose tiles are too few for the
+            // chip (under 160) may split K so that its workgroups make one round; the kernel that then
+            // adds the ranges up moves (ranges x their width + 2 x N) x M x 4 bytes at about 4.5 TB/s
+            // and costs a launch, and it writes the norm that follows, if one was asked for, which
+            // saves that kernel (11 us at 2,048 x 4,096).  Measured against this model at 256 to 1,024
+            // rows (us, model / measured): down at 512 rows in 256x128 tiles and 4 ranges 79 / 74-79, in
+            // 128x128 and 2 ranges 90 / 94, in 256x256 and 8 ranges 80 / 79; q/k/v at 256 rows in 256x128
+            // and 5 ranges 28 / 32, in 128x128 and 2 ranges 31 / 36.
+            const double unit = 0.5e-12;
+            auto seconds = [&](const Cand& c, int cols) { return time_of(c, cols) * K * unit; };
+            auto adding = [&](int ranges) {
+                return ((double)ranges * w_rows + 2.0 * N) * M * 4 / 4.5e12 + 3e-6 - (want_whole_norm ? 11e-6 : 0.0);
+            };
+            int best = 0, best_splits = 1, second = -1, cols_first = N;
+            double t_best = 1e30;
+            for (int i = 0; i < 4; ++i) {
+                if (!usable(cands[i])) continue;
+                const int c = count(cands[i], N);
+                double t = seconds(cands[i], N);
+                int sp = 1;
+                if (c < 160 && workspace && !rope_direct) {
+                    const int s2 = pick_splits(c);
+                    const double ts = (double)cands[i].bm * cands[i].bn / cands[i].rate * ((K + s2 - 1) / s2) * unit + adding(s2);
+                    if (s2 >= 2 && ts < t) { t = ts; sp = s2; }
+                }
+                if (t < t_best) { best = i; best_splits = sp; t_best = t; }
+            }
             for (int i = 0; i < 3; ++i) {
                 if (!usable(cands[i])) continue;
                 const int tm = (M + cands[i].bm - 1) / cands[i].bm, full = count(cands[i], N) / 256;
@@ -1218,28 +1242,8 @@ extern "C" int xr_gemm_bf16(void* out, const void* a, const void* w, const float
                 if (full < 1 || count(cands[i], N) % 256 == 0 || cols <= 0 || cols >= N) continue;
                 for (int j = i + 1; j < 4; ++j) {
                     if (!usable(cands[j]) || cols % width(cands[j])) continue;
-                    const double t = time_of(cands[i], cols) + time_of(cands[j], N - cols);
-                    if (t < 0.92 * t_best) { best = i; second = j; cols_first = cols; t_best = t; }   // (a second launch costs a little, too)
-                }
-            }
-            // Few large tiles and a long K (the down product): 256x256 tiles with K split in two or
-            // more, and the kernel that adds the parts up (which also writes the norm that follows,
-            // if one was asked for).  Times here are in products of a tile at full rate; the adding
-            // kernel moves (ranges + 2) x M x N x 4 bytes at about 4.5 TB/s, a tile does about
-            // 4 TFLOP/s.  Measured (2048 x 4096 x 14336): 264 us against 281 us with 256x128 tiles.
-            if (!sw && workspace && !rope_direct && count(cands[0], N) <= 128 && count(cands[0], N) >= 64) {
-                const int s2 = pick_splits(count(cands[0], N));
-                if (s2 >= 2) {
-                    const double unit = 0.5e-12;       // seconds per product-column of a 256x256 tile's row
-                    const double adding = ((double)(s2 + 2) * M * N * 4 / 4.5e12 + 3e-6) / unit;
-                    const double saved = want_whole_norm ? 11e-6 / unit : 0.0;
-                    const double t = 65536.0 * K / s2 + adding - saved;
-                    if (t < t_best * K) {
-                        g.m_fast = 1;
-                        g.splits = s2;
-                        if (want_whole_norm) { g.norm_whole = 1; norm->ss_out_rows = -1; }
-                        return launch_tile_variant(14, g, stream);
-                    }
+                    const double t = seconds(cands[i], cols) + seconds(cands[j], N - cols);
+                    if (t < 0.92 * t_best) { best = i; best_splits = 1; second = j; cols_first = cols; t_best = t; }   // (a second launch costs a little, too)
                 }
             }
             variant = cands[best].variant;
@@ -1251,11 +1255,10 @@ extern "C" int xr_gemm_bf16(void* out, const void* a, const void* w, const float
                 const int rc = launch_tile_variant(variant, g, stream);
                 return rc != XR_OK ? rc : launch_tile_variant(cands[second].variant, g2, stream);
             }
-            auto count_of = [&](int bm, int bn) { return ((M + bm - 1) / bm) * ((N + (sw ? bn / 2 : bn) - 1) / (sw ? bn / 2 : bn)); };
-            if (variant == 17 && count_of(128, 128) < 160) {
-                g.splits = pick_splits(count_of(128, 128));
+            if (best_splits > 1) {
+                g.splits = best_splits;
                 // the kernel that adds the ranges up takes whole rows and writes the norm that follows
-                if (g.splits > 1 && want_whole_norm) { g.norm_whole = 1; norm->ss_out_rows = -1; }
+                if (want_whole_norm) { g.norm_whole = 1; norm->ss_out_rows = -1; }
             }
         }
     }
