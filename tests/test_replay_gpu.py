@@ -268,6 +268,38 @@ def wide(models):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("which", ["A", "D"])
+def test_three_hundred_requests_decode_in_the_largest_recorded_step(models, which, dtype):
+    """300 requests with prompts of 1 to 6 tokens decode 5 tokens each side by side: the recorded step
+    for 512 rows (212 pad it), in which the q/k/v product is a tile product that rotates and caches its
+    own result from one table of the step's cosines and sines that all layers share inside the recording."""
+    from xyntetik_runner_amd.engine.batch import StepEntry
+    from xyntetik_runner_amd.engine.runner import ModelRunner
+    d, cfg, _, _, _ = models[which]
+    _, w = P.load_folder(d)
+    n, n_dec = 300, 5
+    rng = np.random.default_rng(8)
+    plen = [int(x) for x in rng.integers(1, 7, size=n)]
+    toks = [prompt_ids(plen[i] + n_dec, cfg["vocab_size"], 3000 + i) for i in range(n)]
+    runner = ModelRunner.from_folder(d, dtype=dtype, max_tokens=n * 64, page_size=16, max_requests=n)
+    poison(runner)
+    for g0 in range(0, n, 50):
+        runner.step([StepEntry(i, toks[i][:plen[i]], []) for i in range(g0, g0 + 50)])
+    got = {i: [] for i in range(n)}
+    for k in range(n_dec):
+        out = runner.step([StepEntry(i, [toks[i][plen[i] + k]], [0]) for i in range(n)]).cpu().numpy()
+        for i in range(n):
+            got[i].append(out[i])
+    assert runner.graphs.captures == 1 and runner.graphs.replays == n_dec - 1
+    for i in range(n):
+        rows = np.stack(got[i])
+        want = P.forward(cfg, w, toks[i], all_at_once=True)[plen[i]:]
+        assert np.isfinite(rows).all() and np.abs(rows).max() > 0
+        mx, mean = logit_error(rows, want)
+        assert mx <= TOL[dtype][0] and mean <= TOL[dtype][1], (which, dtype, i, plen[i], mx, mean)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("n_live", [20, 40, 64])
 @pytest.mark.parametrize("which", list(WIDE))
 def test_many_requests_decode_through_recorded_steps(wide, which, n_live, dtype):
