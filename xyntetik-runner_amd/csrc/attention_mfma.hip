@@ -151,45 +151,10 @@ _Pragma("unroll")                                                               
                 for (int e = 0; e < 16; ++e) o[d][e] *= corr;                                            \
         }
 
-// Writing a row's result: the final output, or the partial result of a key range.
-#define ATTN_WRITE_OUT(SLOT)                                                                         \
-    const float inv = l > 0.f ? 1.0f / l : 0.f;                                                          \
-    if (!row_ok) return;                                                                                 \
-    if ((SLOT) < 0) {                                                                                    \
-        bf16_t* op = a.out + ((size_t)t * a.H + h) * HD;                                                 \
-_Pragma("unroll")                                                                                        \
-        for (int d = 0; d < DB; ++d)                                                                     \
-_Pragma("unroll")                                                                                        \
-            for (int e4 = 0; e4 < 4; ++e4) {                                                             \
-                const int dd = d * 32 + e4 * 8 + lg * 4;                                                 \
-                if (dd < HD) {                                                                           \
-                    uint2 w = make_uint2(pack2(o[d][e4 * 4 + 0] * inv, o[d][e4 * 4 + 1] * inv),          \
-                                         pack2(o[d][e4 * 4 + 2] * inv, o[d][e4 * 4 + 3] * inv));         \
-                    *reinterpret_cast<uint2*>(op + dd) = w;                                              \
-                }                                                                                        \
-            }                                                                                            \
-        return;                                                                                          \
-    }                                                                                                    \
-    float* po = a.part_o + (((size_t)(SLOT) * a.Hk + kvh) * ROWS + lr) * HD;                             \
-_Pragma("unroll")                                                                                        \
-    for (int d = 0; d < DB; ++d)                                                                         \
-_Pragma("unroll")                                                                                        \
-        for (int e4 = 0; e4 < 4; ++e4) {                                                                 \
-            const int dd = d * 32 + e4 * 8 + lg * 4;                                                     \
-            if (dd < HD)                                                                                 \
-                *reinterpret_cast<float4*>(po + dd) = make_float4(o[d][e4 * 4 + 0] * inv, o[d][e4 * 4 + 1] * inv, \
-                                                                  o[d][e4 * 4 + 2] * inv, o[d][e4 * 4 + 3] * inv); \
-        }                                                                                                \
-    if (lg == 0) {                                                                                       \
-        float* pm = a.part_ml + (((size_t)(SLOT) * a.Hk + kvh) * ROWS + lr) * 2;                         \
-        pm[0] = m;                                                                                       \
-        pm[1] = l;                                                                                       \
-    }
-
 // ------------------------------------------------------------------------------ workgroup kernel
 // Long prompt portions: a set of 4 waves takes 128 consecutive rows of one request and
 // key/value head (wave w the rows row0 + 32 w ..) and a range of keys (a workgroup is one such
-// set, or two that halve the range between them: CTA_SETS below).  The K tile
+// set, or two that halve the range between them: CtaShape::SETS below).  The K tile
 // [32 keys][HD] and the V^T tile [HD][32 keys] are copied once into LDS for all four waves,
 // by asynchronous copies, two tiles at a time into the places of the two tiles before the ones
 // being worked on (4 tiles in LDS; measured at head size 128, a prompt of 2,048 tokens: a barrier
@@ -208,74 +173,127 @@ constexpr int KSTR = CK_POW2 ? CK : CK + 1;                 // chunks between ke
 constexpr int NKC = 32 * KSTR;                              // chunks of a K tile
 constexpr int NVC = DB * 32 * 4;                            // chunks of a V^T tile
 constexpr int CTA_ROWS = 128;
-constexpr int CTA_LOADS = (NKC + NVC + 255) / 256;          // copies per lane and tile
-constexpr int STAGE_CHUNKS = CTA_LOADS * 256;
 constexpr int CTA_STAGES = 4;                               // tiles in LDS (copied two at a time)
-// Two sets of four waves share an item where LDS has room for two rings: the first set takes the
-// first half of the item's tiles, the second set the rest, and their results are combined through
-// LDS at the end.  A compute unit then has two waves a SIMD from ONE item, and the items, which
-// start longest first, follow one another on it: a causal prompt's blocks see 1 to n keys, and with
-// one set an item (two items to a unit, a long one beside a short one) the long one ran on alone,
-// one wave a SIMD, for most of its time (2,048 tokens, 8 key/value heads: 70 us, now 5x).
-constexpr int CTA_SETS = 2 * CTA_STAGES * STAGE_CHUNKS * 16 <= 144 * 1024 ? 2 : 1;
-constexpr int CTA_THREADS = 256 * CTA_SETS;
-constexpr int CTA_RING_BYTES = CTA_SETS * CTA_STAGES * STAGE_CHUNKS * 16;
-constexpr int CTA_COMBINE_BYTES = CTA_SETS == 2 ? 4 * ROWS * (HD + 4 + 2) * 4 : 0;
-constexpr int CTA_LDS_BYTES = CTA_RING_BYTES > CTA_COMBINE_BYTES ? CTA_RING_BYTES : CTA_COMBINE_BYTES;
-static_assert(CTA_LDS_BYTES <= 160 * 1024, "the tiles do not fit into LDS");
 
-__global__ __launch_bounds__(CTA_THREADS, CTA_SETS == 2 ? 1 : 2) void k_attn_cta(AttnArgs a) {
-    extern __shared__ uint4 lds_all[];                      // [CTA_SETS][CTA_STAGES][STAGE_CHUNKS]
-    const int tid = threadIdx.x & 255, lane = tid & 63, wave = tid >> 6;       // within the set
-    const int set = __builtin_amdgcn_readfirstlane((int)threadIdx.x >> 8);
-    uint4* lds = lds_all + set * CTA_STAGES * STAGE_CHUNKS;
+// RB: 32-row blocks a wave takes.  1 is what is built: four waves a set, two waves a SIMD.  With 2 (two
+// waves a set with 64 rows each, one wave a SIMD, the output accumulators in the upper half of the
+// register file) every K and V^T fragment read from LDS serves two products, and it gives the same
+// bits; compiled as it stands it is slower (2,048 rows behind 6,144 keys: 447 us against 316), because
+// a lone wave has nothing to cover its own waits for LDS and at the barriers.
+//
+// Two sets share an item where LDS has room for two rings: the first set takes the first half of the
+// item's tiles, the second set the rest, and their results are combined through LDS at the end.  A
+// compute unit then has two waves a SIMD from ONE item, and the items, which start longest first,
+// follow one another on it: a causal prompt's blocks see 1 to n keys, and with one set an item (two
+// items to a unit, a long one beside a short one) the long one ran on alone, one wave a SIMD, for most
+// of its time (2,048 tokens, 8 key/value heads: 70 us, now 63).
+template <int RB> struct CtaShape {
+    static constexpr int SET_WAVES = 4 / RB;
+    static constexpr int SET_THREADS = 64 * SET_WAVES;
+    static constexpr int LOADS = (NKC + NVC + SET_THREADS - 1) / SET_THREADS;     // copies per lane and tile
+    static constexpr int STAGE = LOADS * SET_THREADS;                               // chunks of a tile's place in LDS
+    static constexpr int SETS = 2 * CTA_STAGES * STAGE * 16 <= 144 * 1024 ? 2 : 1;
+    static constexpr int THREADS = SET_THREADS * SETS;
+    static constexpr int RING_BYTES = SETS * CTA_STAGES * STAGE * 16;
+    static constexpr int COMBINE_BYTES = SETS == 2 ? 4 * ROWS * (HD + 4 + 2) * 4 : 0;
+    static constexpr int LDS_BYTES = RING_BYTES > COMBINE_BYTES ? RING_BYTES : COMBINE_BYTES;
+    static_assert(LDS_BYTES <= 160 * 1024, "the tiles do not fit into LDS");
+};
+
+// a row block's result: the final output, or the partial result of a key range
+__device__ inline void cta_write_out(const AttnArgs& a, const f32x16 (&o)[DB], float m, float l, bool row_ok, int t, int h,
+                                     int kvh, int lr, int lg, int slot) {
+    const float inv = l > 0.f ? 1.0f / l : 0.f;
+    if (!row_ok) return;
+    if (slot < 0) {
+        bf16_t* op = a.out + ((size_t)t * a.H + h) * HD;
+#pragma unroll
+        for (int d = 0; d < DB; ++d)
+#pragma unroll
+            for (int e4 = 0; e4 < 4; ++e4) {
+                const int dd = d * 32 + e4 * 8 + lg * 4;
+                if (dd < HD) {
+                    uint2 w = make_uint2(pack2(o[d][e4 * 4 + 0] * inv, o[d][e4 * 4 + 1] * inv),
+                                         pack2(o[d][e4 * 4 + 2] * inv, o[d][e4 * 4 + 3] * inv));
+                    *reinterpret_cast<uint2*>(op + dd) = w;
+                }
+            }
+        return;
+    }
+    float* po = a.part_o + (((size_t)slot * a.Hk + kvh) * ROWS + lr) * HD;
+#pragma unroll
+    for (int d = 0; d < DB; ++d)
+#pragma unroll
+        for (int e4 = 0; e4 < 4; ++e4) {
+            const int dd = d * 32 + e4 * 8 + lg * 4;
+            if (dd < HD)
+                *reinterpret_cast<float4*>(po + dd) = make_float4(o[d][e4 * 4 + 0] * inv, o[d][e4 * 4 + 1] * inv,
+                                                                  o[d][e4 * 4 + 2] * inv, o[d][e4 * 4 + 3] * inv);
+        }
+    if (lg == 0) {
+        float* pm = a.part_ml + (((size_t)slot * a.Hk + kvh) * ROWS + lr) * 2;
+        pm[0] = m;
+        pm[1] = l;
+    }
+}
+
+template <int RB>
+__global__ __launch_bounds__(CtaShape<RB>::THREADS, 1) void k_attn_cta(AttnArgs a) {
+    using SH = CtaShape<RB>;
+    constexpr int SET_THREADS = SH::SET_THREADS, LOADS = SH::LOADS, STAGE = SH::STAGE, SETS = SH::SETS;
+    extern __shared__ uint4 lds_all[];                      // [SETS][CTA_STAGES][STAGE]
+    const int tid = threadIdx.x % SET_THREADS, lane = tid & 63, wave = tid >> 6;       // within the set
+    const int set = __builtin_amdgcn_readfirstlane((int)threadIdx.x / SET_THREADS);
+    uint4* lds = lds_all + set * CTA_STAGES * STAGE;
     // Items come longest first, and workgroups start in the order of their numbers: an item's
     // key/value heads are numbered side by side, so that the longest items of every head start
     // first.  (With 8 key/value heads a head's items then also run on one of the 8 dies and share
     // its L2.)
-    // (One set, two workgroups to a unit, the second 256 numbers later: when all run at once, the
-    // second half of the numbers is taken in reverse, so that a unit gets a long and a short item.)
     unsigned wg = blockIdx.x;
-    if (CTA_SETS == 1 && gridDim.x <= 512 && wg >= (gridDim.x + 1) / 2) wg = gridDim.x - 1 - (wg - (gridDim.x + 1) / 2);
+    if (SETS == 1 && gridDim.x <= 512 && wg >= (gridDim.x + 1) / 2) wg = gridDim.x - 1 - (wg - (gridDim.x + 1) / 2);
     const int item_no = (int)(wg / (unsigned)a.Hk);
     const int kvh = (int)wg - item_no * a.Hk;
     const int* it = a.cta_items + (size_t)item_no * ITEM_INTS;
-    const int req = it[0], row0 = it[1] + wave * ROWS;
-    const int slot = it[4] < 0 ? -1 : it[4] + wave;
+    const int req = it[0];
     const int q0 = it[5], q_len = it[6], start = it[7];
     // the set's share of the item's keys; both sets go through the loop as often as the first
     const int nt_item = (it[3] - it[2] + 31) >> 5;
-    const int nt_first = CTA_SETS == 2 ? (nt_item + 1) >> 1 : nt_item;
+    const int nt_first = SETS == 2 ? (nt_item + 1) >> 1 : nt_item;
     const int kbeg = it[2] + set * nt_first * 32;
-    const int kend = (set == 0 && CTA_SETS == 2 && it[2] + nt_first * 32 < it[3]) ? it[2] + nt_first * 32 : it[3];
+    const int kend = (set == 0 && SETS == 2 && it[2] + nt_first * 32 < it[3]) ? it[2] + nt_first * 32 : it[3];
     const int G = a.H / a.Hk;
     const int lr = lane & 31, lg = lane >> 5;
     const int seq_len = start + q_len;
     const int* bt = a.block_table + (size_t)req * a.table_stride;
 
-    // this lane's query row
-    const int rho = row0 + lr;
-    const int tok = rho / G, hg = rho - tok * G;
-    const bool row_ok = tok < q_len;
-    const int t = q0 + tok, h = kvh * G + hg;
-    const int pos = start + tok;
-    const int lo = (a.window > 0 && pos - a.window + 1 > 0) ? pos - a.window + 1 : 0;
-
-    bf16x8 qf[KD];
-    {
-        const bf16_t* qp = a.q + ((size_t)(row_ok ? t : q0) * a.H + h) * HD + lg * 8;
+    // this lane's query rows, one in each of the wave's row blocks
+    int slot_[RB], t_[RB], h_[RB], pos_[RB], lo_[RB];
+    bool ok_[RB];
+    bf16x8 qf[RB][KD];
 #pragma unroll
-        for (int kd = 0; kd < KD; ++kd) qf[kd] = as_bf16x8(keep_if(row_ok, ldg16(qp + kd * 16)));
+    for (int rb = 0; rb < RB; ++rb) {
+        const int blk = wave * RB + rb;
+        const int rho = it[1] + blk * ROWS + lr;
+        const int tok = rho / G, hg = rho - tok * G;
+        slot_[rb] = it[4] < 0 ? -1 : it[4] + blk;
+        ok_[rb] = tok < q_len;
+        t_[rb] = q0 + tok;
+        h_[rb] = kvh * G + hg;
+        pos_[rb] = start + tok;
+        lo_[rb] = (a.window > 0 && pos_[rb] - a.window + 1 > 0) ? pos_[rb] - a.window + 1 : 0;
+        const bf16_t* qp = a.q + ((size_t)(ok_[rb] ? t_[rb] : q0) * a.H + h_[rb]) * HD + lg * 8;
+#pragma unroll
+        for (int kd = 0; kd < KD; ++kd) qf[rb][kd] = as_bf16x8(keep_if(ok_[rb], ldg16(qp + kd * 16)));
     }
-    const int ra = lr >> 3, rg = (lr >> 2) & 1, rb = lr & 3;
-    const int key_off = 16 * (ra >> 1) + 8 * rg + 4 * (ra & 1) + rb;
+    const int ra = lr >> 3, rg = (lr >> 2) & 1, rb4 = lr & 3;
+    const int key_off = 16 * (ra >> 1) + 8 * rg + 4 * (ra & 1) + rb4;
 
     // the pieces this lane copies for every tile
-    int src_off[CTA_LOADS], src_key[CTA_LOADS];
-    bool src_is_k[CTA_LOADS];
+    int src_off[LOADS], src_key[LOADS];
+    bool src_is_k[LOADS];
 #pragma unroll
-    for (int i = 0; i < CTA_LOADS; ++i) {
-        const int q = i * 256 + tid;
+    for (int i = 0; i < LOADS; ++i) {
+        const int q = i * SET_THREADS + tid;
         src_is_k[i] = q < NKC;
         if (q < NKC) {
             const int r = q / KSTR, cs = q - r * KSTR;
@@ -295,10 +313,10 @@ __global__ __launch_bounds__(CTA_THREADS, CTA_SETS == 2 ? 1 : 2) void k_attn_cta
     // Where every lane's piece exists in every whole tile and a copy instruction brings pieces of
     // keys only or of values only (head sizes 64, 128 and 256), a whole tile of an existing page
     // is copied from two bases that all lanes share, each lane adding a fixed 32-bit offset.
-    constexpr bool CTA_FAST = CK_POW2 && NKC % 256 == 0 && NVC % 256 == 0 && HD % 32 == 0;
-    uint32_t fast_off[CTA_LOADS];
+    constexpr bool CTA_FAST = CK_POW2 && NKC % SET_THREADS == 0 && NVC % SET_THREADS == 0 && HD % 32 == 0;
+    uint32_t fast_off[LOADS];
 #pragma unroll
-    for (int i = 0; i < CTA_LOADS; ++i) fast_off[i] = (uint32_t)src_off[i] * 2u;
+    for (int i = 0; i < LOADS; ++i) fast_off[i] = (uint32_t)src_off[i] * 2u;
 
     // page numbers of the item's keys, one per lane, 64 pages at a time
     int pages_base = kbeg >> a.page_shift;
@@ -329,54 +347,64 @@ __global__ __launch_bounds__(CTA_THREADS, CTA_SETS == 2 ? 1 : 2) void k_attn_cta
         const size_t pb_ = (size_t)(pg_ < 0 ? 0 : pg_) * a.Hk + kvh;                                     \
         const bf16_t* kb_ = kc + (pb_ * a.page_size + (kt_ & a.page_mask)) * HD;                         \
         const bf16_t* vb_ = vc + pb_ * HD * a.page_size + (kt_ & a.page_mask);                           \
-        const uint32_t dst_ = __builtin_amdgcn_readfirstlane(lds_base + (uint32_t)(((ti_ % CTA_STAGES) * STAGE_CHUNKS + wave * 64) * 16)); \
+        const uint32_t dst_ = __builtin_amdgcn_readfirstlane(lds_base + (uint32_t)(((ti_ % CTA_STAGES) * STAGE + wave * 64) * 16)); \
         if (CTA_FAST && pg_ >= 0 && kt_ + 32 <= seq_len) {                                               \
-            _Pragma("unroll") for (int i = 0; i < CTA_LOADS; ++i)                                        \
-                lds_dma16_base(i * 256 < NKC ? kb_ : vb_, fast_off[i], dst_ + i * 256 * 16);             \
+            _Pragma("unroll") for (int i = 0; i < LOADS; ++i)                                            \
+                lds_dma16_base(i * SET_THREADS < NKC ? kb_ : vb_, fast_off[i], dst_ + i * SET_THREADS * 16); \
         } else {                                                                                         \
-            _Pragma("unroll") for (int i = 0; i < CTA_LOADS; ++i) {                                      \
-                const bool ok_ = pg_ >= 0 && kt_ + src_key[i] < seq_len;                                 \
-                const bf16_t* p_ = ok_ ? (src_is_k[i] ? kb_ : vb_) + src_off[i] : zero_src;              \
-                lds_dma16(p_, dst_ + i * 256 * 16);                                                      \
+            _Pragma("unroll") for (int i = 0; i < LOADS; ++i) {                                          \
+                const bool okc_ = pg_ >= 0 && kt_ + src_key[i] < seq_len;                                \
+                const bf16_t* p_ = okc_ ? (src_is_k[i] ? kb_ : vb_) + src_off[i] : zero_src;             \
+                lds_dma16(p_, dst_ + i * SET_THREADS * 16);                                              \
             }                                                                                            \
         }                                                                                                \
     }
 
-    f32x16 o[DB];
+    f32x16 o_[RB][DB];
+    float m_[RB], l_[RB];      // m in units of log2
+    int pmin_[RB], lmax_[RB], pmax_[RB], lmin_[RB];
 #pragma unroll
-    for (int d = 0; d < DB; ++d)
+    for (int rb = 0; rb < RB; ++rb) {
 #pragma unroll
-        for (int e = 0; e < 16; ++e) o[d][e] = 0.f;
-    float m = -INFINITY, l = 0.f;      // m in units of log2
-    const float c2 = a.scale * 1.44269504088896340736f;
-    // what the rows of this wave can see: keys [lo_min, pos_max]; keys in [lo_max, pos_min] by all
-    int pos_min = row_ok ? pos : 0x7fffffff, lo_max = row_ok ? lo : 0;
-    int pos_max = row_ok ? pos : -1, lo_min = row_ok ? lo : 0x7fffffff;
+        for (int d = 0; d < DB; ++d)
 #pragma unroll
-    for (int o_ = 32; o_ > 0; o_ >>= 1) {
-        pos_min = min(pos_min, __shfl_xor(pos_min, o_, 64));
-        lo_max = max(lo_max, __shfl_xor(lo_max, o_, 64));
-        pos_max = max(pos_max, __shfl_xor(pos_max, o_, 64));
-        lo_min = min(lo_min, __shfl_xor(lo_min, o_, 64));
+            for (int e = 0; e < 16; ++e) o_[rb][d][e] = 0.f;
+        m_[rb] = -INFINITY;
+        l_[rb] = 0.f;
+        // what the rows of this block can see: keys [lo_min, pos_max]; keys in [lo_max, pos_min] by all
+        int pos_min = ok_[rb] ? pos_[rb] : 0x7fffffff, lo_max = ok_[rb] ? lo_[rb] : 0;
+        int pos_max = ok_[rb] ? pos_[rb] : -1, lo_min = ok_[rb] ? lo_[rb] : 0x7fffffff;
+#pragma unroll
+        for (int x = 32; x > 0; x >>= 1) {
+            pos_min = min(pos_min, __shfl_xor(pos_min, x, 64));
+            lo_max = max(lo_max, __shfl_xor(lo_max, x, 64));
+            pos_max = max(pos_max, __shfl_xor(pos_max, x, 64));
+            lo_min = min(lo_min, __shfl_xor(lo_min, x, 64));
+        }
+        pmin_[rb] = pos_min; lmax_[rb] = lo_max; pmax_[rb] = pos_max; lmin_[rb] = lo_min;
     }
+    const float c2 = a.scale * 1.44269504088896340736f;
 
     // The tiles are copied and waited for two at a time: the workgroup meets at a barrier, and the
     // copies' addresses are worked out, every second tile (two tiles take a wave over 2 us, more
     // than a copy from L2 needs to land).
-    static_assert(CTA_STAGES % 2 == 0 && CTA_LOADS * 2 < 64, "the tiles in LDS come in pairs");
+    static_assert(CTA_STAGES % 2 == 0 && LOADS * 2 < 64, "the tiles in LDS come in pairs");
 #pragma unroll
     for (int st = 0; st < CTA_STAGES - 2; ++st) CTA_ISSUE(st)
     for (int ti = 0; ti < nt_first; ++ti) {
         if ((ti & 1) == 0) {
             // tiles ti and ti+1 have landed when at most the CTA_STAGES-4 younger ones are on their way
-            wait_vmcnt<CTA_LOADS * (CTA_STAGES - 4)>();
+            wait_vmcnt<LOADS * (CTA_STAGES - 4)>();
             __builtin_amdgcn_s_barrier();                // for every wave; and tiles ti-2, ti-1 are no longer read
             CTA_ISSUE(ti + CTA_STAGES - 2)               // into their places (zeros past the end)
             CTA_ISSUE(ti + CTA_STAGES - 1)
         }
         const int kt = kbeg + ti * 32;
-        if (ti >= nt || kt > pos_max || kt + 32 <= lo_min) continue; // nothing here for this wave's rows
-        const uint4* Ks = lds + (ti % CTA_STAGES) * STAGE_CHUNKS;
+        bool any = false;
+#pragma unroll
+        for (int rb = 0; rb < RB; ++rb) any = any || !(kt > pmax_[rb] || kt + 32 <= lmin_[rb]);
+        if (ti >= nt || !any) continue;                  // nothing here for this wave's rows
+        const uint4* Ks = lds + (ti % CTA_STAGES) * STAGE;
         const uint4* Vs = Ks + NKC;
         uint4 kf[KD], vf[2][DB];
 #pragma unroll
@@ -402,74 +430,96 @@ __global__ __launch_bounds__(CTA_THREADS, CTA_SETS == 2 ? 1 : 2) void k_attn_cta
                 }
             }
         }
-        f32x16 s;
+        f32x16 s_[RB];
 #pragma unroll
-        for (int e = 0; e < 16; ++e) s[e] = 0.f;
+        for (int rb = 0; rb < RB; ++rb)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) s_[rb][e] = 0.f;
 #pragma unroll
         for (int kd = 0; kd < KD; ++kd)
-            s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16x8(kf[kd]), qf[kd], s, 0, 0, 0);
-        float p[16];
-        float corr;
-        ATTN_SOFTMAX_STEP(kt, kend)
 #pragma unroll
-        for (int j = 0; j < 2; ++j) {
-            uint4 pk = make_uint4(pack2(p[8 * j + 0], p[8 * j + 1]), pack2(p[8 * j + 2], p[8 * j + 3]),
-                                  pack2(p[8 * j + 4], p[8 * j + 5]), pack2(p[8 * j + 6], p[8 * j + 7]));
-            const bf16x8 pf = as_bf16x8(pk);
+            for (int rb = 0; rb < RB; ++rb)
+                s_[rb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16x8(kf[kd]), qf[rb][kd], s_[rb], 0, 0, 0);
 #pragma unroll
-            for (int d = 0; d < DB; ++d)
-                o[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16x8(vf[j][d]), pf, o[d], 0, 0, 0);
+        for (int rb = 0; rb < RB; ++rb) {
+            f32x16& s = s_[rb];
+            f32x16 (&o)[DB] = o_[rb];
+            float& m = m_[rb];
+            float& l = l_[rb];
+            const bool row_ok = ok_[rb];
+            const int pos = pos_[rb], lo = lo_[rb], pos_min = pmin_[rb], lo_max = lmax_[rb];
+            float p[16];
+            float corr;
+            ATTN_SOFTMAX_STEP(kt, kend)
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                uint4 pk = make_uint4(pack2(p[8 * j + 0], p[8 * j + 1]), pack2(p[8 * j + 2], p[8 * j + 3]),
+                                      pack2(p[8 * j + 4], p[8 * j + 5]), pack2(p[8 * j + 6], p[8 * j + 7]));
+                const bf16x8 pf = as_bf16x8(pk);
+#pragma unroll
+                for (int d = 0; d < DB; ++d)
+                    o[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16x8(vf[j][d]), pf, o[d], 0, 0, 0);
+            }
         }
     }
 #undef CTA_ISSUE
     wait_vmcnt<0>();                                     // the trailing copies of zeros
-    l += __shfl_xor(l, 32, 64);                          // the row's sum from its two lanes
+#pragma unroll
+    for (int rb = 0; rb < RB; ++rb) l_[rb] += __shfl_xor(l_[rb], 32, 64);      // the row's sum from its two lanes
 
-    if (CTA_SETS == 2) {
+    if (SETS == 2) {
         // the second set hands its rows' maxima, sums and unnormalised outputs to the first
         __syncthreads();                                 // the rings are free
-        float* xo = reinterpret_cast<float*>(lds_all);   // [4 waves][ROWS][HD + 4]
-        float* xml = xo + 4 * ROWS * (HD + 4);           // [4 waves][ROWS][2]
-        float* mine = xo + (wave * ROWS + lr) * (HD + 4);
+        float* xo = reinterpret_cast<float*>(lds_all);   // [4 row blocks][ROWS][HD + 4]
+        float* xml = xo + 4 * ROWS * (HD + 4);           // [4 row blocks][ROWS][2]
         if (set == 1) {
+#pragma unroll
+            for (int rb = 0; rb < RB; ++rb) {
+                float* mine = xo + ((wave * RB + rb) * ROWS + lr) * (HD + 4);
+#pragma unroll
+                for (int d = 0; d < DB; ++d)
+#pragma unroll
+                    for (int e4 = 0; e4 < 4; ++e4) {
+                        const int dd = d * 32 + e4 * 8 + lg * 4;
+                        if (dd < HD)
+                            *reinterpret_cast<float4*>(mine + dd) = make_float4(o_[rb][d][e4 * 4 + 0], o_[rb][d][e4 * 4 + 1],
+                                                                                o_[rb][d][e4 * 4 + 2], o_[rb][d][e4 * 4 + 3]);
+                    }
+                if (lg == 0) {
+                    xml[((wave * RB + rb) * ROWS + lr) * 2] = m_[rb];
+                    xml[((wave * RB + rb) * ROWS + lr) * 2 + 1] = l_[rb];
+                }
+            }
+        }
+        __syncthreads();
+        if (set == 1) return;
+#pragma unroll
+        for (int rb = 0; rb < RB; ++rb) {
+            const float* mine = xo + ((wave * RB + rb) * ROWS + lr) * (HD + 4);
+            const float m1 = xml[((wave * RB + rb) * ROWS + lr) * 2], l1 = xml[((wave * RB + rb) * ROWS + lr) * 2 + 1];
+            const float mn = fmaxf(m_[rb], m1);
+            const float f0 = m_[rb] == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(m_[rb] - mn);
+            const float f1 = m1 == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(m1 - mn);
+            l_[rb] = l_[rb] * f0 + l1 * f1;
+            m_[rb] = mn;
 #pragma unroll
             for (int d = 0; d < DB; ++d)
 #pragma unroll
                 for (int e4 = 0; e4 < 4; ++e4) {
                     const int dd = d * 32 + e4 * 8 + lg * 4;
-                    if (dd < HD)
-                        *reinterpret_cast<float4*>(mine + dd) = make_float4(o[d][e4 * 4 + 0], o[d][e4 * 4 + 1],
-                                                                            o[d][e4 * 4 + 2], o[d][e4 * 4 + 3]);
+                    if (dd < HD) {
+                        const float4 x = *reinterpret_cast<const float4*>(mine + dd);
+                        o_[rb][d][e4 * 4 + 0] = o_[rb][d][e4 * 4 + 0] * f0 + x.x * f1;
+                        o_[rb][d][e4 * 4 + 1] = o_[rb][d][e4 * 4 + 1] * f0 + x.y * f1;
+                        o_[rb][d][e4 * 4 + 2] = o_[rb][d][e4 * 4 + 2] * f0 + x.z * f1;
+                        o_[rb][d][e4 * 4 + 3] = o_[rb][d][e4 * 4 + 3] * f0 + x.w * f1;
+                    }
                 }
-            if (lg == 0) {
-                xml[(wave * ROWS + lr) * 2] = m;
-                xml[(wave * ROWS + lr) * 2 + 1] = l;
-            }
         }
-        __syncthreads();
-        if (set == 1) return;
-        const float m1 = xml[(wave * ROWS + lr) * 2], l1 = xml[(wave * ROWS + lr) * 2 + 1];
-        const float mn = fmaxf(m, m1);
-        const float f0 = m == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(m - mn);
-        const float f1 = m1 == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(m1 - mn);
-        l = l * f0 + l1 * f1;
-        m = mn;
-#pragma unroll
-        for (int d = 0; d < DB; ++d)
-#pragma unroll
-            for (int e4 = 0; e4 < 4; ++e4) {
-                const int dd = d * 32 + e4 * 8 + lg * 4;
-                if (dd < HD) {
-                    const float4 x = *reinterpret_cast<const float4*>(mine + dd);
-                    o[d][e4 * 4 + 0] = o[d][e4 * 4 + 0] * f0 + x.x * f1;
-                    o[d][e4 * 4 + 1] = o[d][e4 * 4 + 1] * f0 + x.y * f1;
-                    o[d][e4 * 4 + 2] = o[d][e4 * 4 + 2] * f0 + x.z * f1;
-                    o[d][e4 * 4 + 3] = o[d][e4 * 4 + 3] * f0 + x.w * f1;
-                }
-            }
     }
-
-    ATTN_WRITE_OUT(slot)
+#pragma unroll
+    for (int rb = 0; rb < RB; ++rb)
+        cta_write_out(a, o_[rb], m_[rb], l_[rb], ok_[rb], t_[rb], h_[rb], kvh, lr, lg, slot_[rb]);
 }
 
 // ------------------------------------------------------------------------------ streaming kernel
@@ -817,15 +867,15 @@ extern "C" int xr_attention_mfma(void* out, const void* q, const void* k_cache, 
     a.part_o = part_o; a.part_ml = part_ml; a.n_items = n_items; a.H = H; a.Hk = Hk;
     a.page_shift = shift; a.page_mask = page_size - 1; a.page_size = page_size; a.scale = scale; a.window = window;
     if (n_cta_items > 0) {
-        constexpr int smem = CTA_LDS_BYTES;
+        constexpr int smem = CtaShape<1>::LDS_BYTES;
         static bool attr_set = false;
         if (!attr_set) {
-            hipError_t e = hipFuncSetAttribute((const void*)k_attn_cta, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+            hipError_t e = hipFuncSetAttribute((const void*)k_attn_cta<1>, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
             if (e != hipSuccess) (void)hipGetLastError();     // or the next launch's check would report this refusal
             XR_REQUIRE(e == hipSuccess, "attention: %d bytes of LDS refused: %s", smem, hipGetErrorString(e));
             attr_set = true;
         }
-        k_attn_cta<<<dim3((unsigned)n_cta_items * (unsigned)Hk), CTA_THREADS, smem, stream>>>(a);
+        k_attn_cta<1><<<dim3((unsigned)n_cta_items * (unsigned)Hk), CtaShape<1>::THREADS, smem, stream>>>(a);
         XR_CHECK_LAUNCH("attention_cta");
     }
     if (n_items > 0) {
