@@ -25,11 +25,11 @@ from typing import Dict, List, Tuple
 
 def read_trace(folder: str) -> List[Tuple[int, int, str, int]]:
     """(start ns, end ns, kernel name, grid size) of every dispatch, in order of start."""
-    files = sorted(glob.glob(os.path.join(folder, "**", "*kernel_trace.csv"), recursive=True))
+    files = sorted(glob.glob(os.path.join(folder, "**", "*kernel_trace.csv"), recursive=True), key=os.path.getmtime)
     if not files:
         raise SystemExit(f"no *kernel_trace.csv under {folder}")
     rows = []
-    with open(files[-1], newline="") as f:
+    with open(files[-1], newline="") as f:               # the newest, if the folder holds several runs
         for r in csv.DictReader(f):
             rows.append((int(r["Start_Timestamp"]), int(r["End_Timestamp"]), r["Kernel_Name"], int(r.get("Grid_Size_X") or 0)))
     rows.sort()
