@@ -116,6 +116,42 @@ def test_linear_bf16_mfma(ops, M, N, K):
                        a.double() @ w.double().T + b.double()) < 1e-5
 
 
+@pytest.mark.parametrize("variant", [51, 55])
+@pytest.mark.parametrize("M,N,K", [(65, 100, 192), (300, 333, 256), (513, 520, 1024), (256, 256, 4096)])
+def test_four_wave_tile_kernels(ops, variant, M, N, K):
+    """The 256x256 and 256x128 tiles' kernels with four waves and a written order of instructions, by
+    name (they refuse what they do not take): rows and columns that fill no tile, plain and packed
+    weights, a bias, adding into the output, the gated epilogue; against the eight-wave kernel of
+    the same tile the sums are the same to the bit (same products in the same order)."""
+    from xyntetik_runner_amd.csrc.ops import KernelError
+    eight_waves = 114 if variant == 51 else 112
+    a = (torch.randn(M, K, device=DEV) * 0.5).bfloat16()
+    w = (torch.randn(N, K, device=DEV) * 0.1).bfloat16()
+    b = torch.randn(N, device=DEV) * 0.1
+    want = a.double() @ w.double().T + b.double()
+    for wt in (w, ops.pack_weight(w)):
+        got = ops.linear(a, wt, bias=b, out_dtype=torch.float32, variant=variant)
+        assert rel(got, want) < 1e-5
+        assert torch.equal(got, ops.linear(a, wt, bias=b, out_dtype=torch.float32, variant=eight_waves))
+        assert rel(ops.linear(a, wt, bias=b, variant=variant), want) < 6e-3
+    base = torch.randn(M, N, device=DEV)
+    out = base.clone()
+    ops.linear(a, w, out=out, accumulate=True, variant=variant)
+    assert rel(out, base.double() + a.double() @ w.double().T) < 1e-5
+    w2 = (torch.randn(2 * N, K, device=DEV) * 0.1).bfloat16()
+    b2 = torch.randn(2 * N, device=DEV) * 0.1
+    r = a.double() @ w2.double().T + b2.double()
+    want = r[:, :N] / (1 + torch.exp(-r[:, :N])) * r[:, N:]
+    for wt in (w2, ops.pack_weight(w2, gated=True)):
+        assert rel(ops.linear_swiglu(a, wt, bias=b2, variant=variant), want) < 6e-3
+    # what they do not take is refused by name, and taken by the eight-wave kernel when the tile is asked for
+    a2 = (torch.randn(M, 72, device=DEV) * 0.5).bfloat16()
+    w3 = (torch.randn(N, 72, device=DEV) * 0.1).bfloat16()
+    with pytest.raises(KernelError, match="four-wave"):
+        ops.linear(a2, w3, variant=variant)
+    assert rel(ops.linear(a2, w3, out_dtype=torch.float32, variant=14 if variant == 51 else 12), a2.double() @ w3.double().T) < 1e-5
+
+
 @pytest.mark.parametrize("M", [8, 40, 300])
 def test_gated_product_with_gates_far_from_zero(ops, M):
     """Gate values of -200 and +200 through the fused epilogues: the weight-streaming kernel's
@@ -328,11 +364,12 @@ def _unpack(data, N, K):
 
 
 def test_long_products_with_few_tiles_are_split_over_k(ops):
-    """2048 x 4096 x 14336 (a down product): 128 tiles of 256x256 would fill half the chip, so K is
-    split in two and a second kernel adds the halves into the residual stream; asked for the
-    norm that follows, that kernel writes it too and the norm's own kernel is not launched."""
+    """1024 x 4096 x 14336 (a down product): 128 tiles of 256x128 (or 64 of 256x256) would fill half
+    the chip or less, so K is split and a second kernel adds the ranges into the residual stream;
+    asked for the norm that follows, that kernel writes it too and the norm's own kernel is not
+    launched."""
     torch.manual_seed(11)
-    M, N, K = 2048, 4096, 14336
+    M, N, K = 1024, 4096, 14336
     a = (torch.randn(M, K, device=DEV) * 0.3).bfloat16()
     w = (torch.randn(N, K, device=DEV) * 0.05).bfloat16()
     pw = ops.pack_weight(w)
@@ -580,7 +617,16 @@ def test_projection_with_rotation_and_cache_write_of_a_product_split_over_k(ops,
     check_projection_with_rotation_and_cache_write(ops, dt, 4, 2, 64, 64, False, 64, starts, q_lens, True, 1024)
 
 
-def check_projection_with_rotation_and_cache_write(ops, dt, H, Hk, D, rot, inter, ps, starts, q_lens, bias, E):
+@pytest.mark.parametrize("variant", [51, 55, 114, 112])
+@pytest.mark.parametrize("H,Hk,D,rot,inter", [(4, 2, 64, 64, False), (3, 1, 48, 32, False), (2, 1, 80, 80, True), (5, 1, 128, 128, False)])
+def test_projection_with_rotation_in_the_tile_kernels_by_name(ops, variant, H, Hk, D, rot, inter):
+    """From 512 rows the tile kernel rotates and caches its own result: the four-wave kernels of the
+    256x256 and 256x128 tiles (16 and 8 tiles of 32x32 a wave) and the eight-wave ones, by name, with
+    heads that straddle the waves' tiles."""
+    check_projection_with_rotation_and_cache_write(ops, "bfloat16", H, Hk, D, rot, inter, 16, [5, 0], [530, 70], True, 256, variant=variant)
+
+
+def check_projection_with_rotation_and_cache_write(ops, dt, H, Hk, D, rot, inter, ps, starts, q_lens, bias, E, variant=0):
     """q, k and v from one product, rotated and cached.  Up to 16 bfloat16 rows the product's own
     kernel does all of it (with the weight's rows in paired order where a pair is (j, j + rot/2)),
     up to 511 the kernel that adds the product's K ranges up, from 512 the tile kernel;
@@ -621,7 +667,8 @@ def check_projection_with_rotation_and_cache_write(ops, dt, H, Hk, D, rot, inter
         try:
             q = ops.project_rope_kv_write(h, ops.pack_weight(wp), bp, kc, vc, ctx.positions, ctx.req_of_token,
                                           ctx.block_table(0), inv, H, Hk, D, rot, inter, 1.0, ps, paired=paired,
-                                          cs_table=step_table if fuse not in (True, False) and rot else None)
+                                          cs_table=step_table if fuse not in (True, False) and rot else None,
+                                          variant=variant if fuse else 0)
         finally:
             ops.fuse_rope = True
         assert q.dtype == DT[dt] and rel(q.cpu().reshape(T, H, D), want_q) < tol

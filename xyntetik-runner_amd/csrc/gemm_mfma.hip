@@ -24,6 +24,8 @@
 // pages (RopeFuse), so that a decode step launches 6 kernels a layer.
 // The reference's float-weight "GEMM" is a multi-column matvec (src/kernels.cu:116-144);
 // its tensor-core kernels (:856) exist for quantised weights only.
+#include <type_traits>
+
 #include "common.h"
 #include "async_copy.h"
 
@@ -65,7 +67,7 @@ struct GemmArgs {
     int out_bf16;      // storage of out
     int epi;
     int act;           // the gate's activation (XR_ACT_*), with EPI_GATED
-    int m_fast;        // tile order of the asynchronous kernel: 1 = consecutive workgroups share a weight tile
+    int m_fast;        // tile order of the asynchronous kernel: 1 = consecutive workgroups share a weight tile, 2 = by XCD
     int splits;        // > 1: K is cut into this many ranges, each workgroup writes raw sums to `partial`
     int k_per_split;   // columns per range (a multiple of 64)
     float* partial;    // [splits][M][rows of w]
@@ -185,34 +187,57 @@ __device__ inline void rope_store(const RopeFuse& rp, int tok, int nn, float val
 // lane and their addresses.)  mode: 0 store float, 1 add into float, 2 store bfloat16.
 // A wave's LDS accesses are served in order, so it needs no barrier for an area of its own.
 constexpr int STAGE_FLOATS = 32 * (64 + 4);      // a wave's area: 32 rows of 64 columns, rows 16 bytes apart in the banks
+// What write_tiles will add to (mode 1), fetched ahead: a lane's 4 floats of each of its 4 NT rows.
+// The stores of one tile and the loads of the next may be the same memory for all the compiler
+// knows, so loads left inside write_tiles wait for each store before them, one trip to memory
+// after the other (measured: the down product of 2,048 rows 240 us against 194 without adding).
+template <int NT>
+__device__ inline void load_old(float4 (&old)[4 * NT], const void* dst, int ld, int m_base, int M, int col_base, int col_end, int lane) {
+    constexpr int CPR = 8 * NT, RPI = 64 / CPR;
+    const int ch = lane % CPR, col = col_base + ch * 4;
+    const float* const dst32 = (const float*)dst + ((size_t)m_base * ld + col_base);
+    const uint32_t lane_off = (uint32_t)((lane / CPR) * ld + ch * 4);
+#pragma unroll
+    for (int it = 0; it < 4 * NT; ++it) {
+        const int m = m_base + it * RPI + lane / CPR;
+        old[it] = (m < M && col < col_end) ? *reinterpret_cast<const float4*>(dst32 + lane_off + (uint32_t)(it * RPI * ld)) : make_float4(0.f, 0.f, 0.f, 0.f);
+    }
+}
+
 template <int NT>
 __device__ inline void write_tiles(float* stage, const f32x16 (&t)[NT], void* dst, int ld, int mode,
-                                   int m_base, int M, int col_base, int col_end, int lane) {
+                                   int m_base, int M, int col_base, int col_end, int lane, const float4* old = nullptr) {
     constexpr int SW = 32 * NT, LD = SW + 4, CPR = SW / 4, RPI = 64 / CPR;
     const int lr = lane & 31, lg = lane >> 5;
 #pragma unroll
     for (int n = 0; n < NT; ++n)
 #pragma unroll
         for (int e = 0; e < 16; ++e) stage[((e / 4) * 8 + lg * 4 + (e % 4)) * LD + n * 32 + lr] = t[n][e];
+    // one address for the tile's corner, which all lanes share, and a 32-bit offset per lane from it
     const int ch = lane % CPR, col = col_base + ch * 4;
+    const size_t corner = (size_t)m_base * ld + col_base;
+    bf16_t* const dst16 = (bf16_t*)dst + corner;
+    float* const dst32 = (float*)dst + corner;
+    const uint32_t lane_off = (uint32_t)((lane / CPR) * ld + ch * 4);
 #pragma unroll
     for (int it = 0; it < 32 / RPI; ++it) {
         const int row = it * RPI + lane / CPR, m = m_base + row;
         const float4 x = *reinterpret_cast<const float4*>(stage + row * LD + ch * 4);
         if (m >= M || col >= col_end) continue;
-        const size_t o = (size_t)m * ld + col;
+        const uint32_t o = lane_off + (uint32_t)(it * RPI * ld);
         if (mode == 2) {
             uint2 v;
             v.x = pack_bf16x2(x.x, x.y);
             v.y = pack_bf16x2(x.z, x.w);
-            *reinterpret_cast<uint2*>((bf16_t*)dst + o) = v;
+            *reinterpret_cast<uint2*>(dst16 + o) = v;
         } else {
-            float4* q = reinterpret_cast<float4*>((float*)dst + o);
+            float4* q = reinterpret_cast<float4*>(dst32 + o);
             float4 y = x;
-            if (mode == 1) { const float4 old = *q; y.x += old.x; y.y += old.y; y.z += old.z; y.w += old.w; }
+            if (mode == 1) { const float4 o4 = old ? old[it] : *q; y.x += o4.x; y.y += o4.y; y.z += o4.z; y.w += o4.w; }
             *q = y;
         }
     }
+    __builtin_amdgcn_sched_barrier(0);               // (tile by tile: no tile's addresses wait in registers for another's stores)
 }
 
 // The cosines and sines a product of many rows needs to rotate its own result, once for all
@@ -355,12 +380,37 @@ __device__ inline int w_row_of(int r, int bx, int N, int epi, int& out_col) {
 // 16 consecutive rows must fall into 16 different 16-byte bank groups.  Two rows of 128 bytes
 // (8 chunks) fill the banks, so the shift counts pairs of rows.  (The counter of LDS bank
 // conflicts reads zero with this, and half the active cycles with a shift by the row number.)
-template <int CH> __device__ inline int swz(int r) { static_assert(CH == 8, "rows of 8 chunks"); return (r >> 1) & 7; }
+// (Rows of 64 bytes, 4 chunks: four rows fill the banks, and the shift counts fours of rows.)
+template <int CH> __device__ inline int swz(int r) {
+    static_assert(CH == 8 || CH == 4, "rows of 8 or of 4 chunks");
+    return CH == 8 ? (r >> 1) & 7 : (r >> 2) & 3;
+}
 
-template <int BM, int BN, int WARPS_M, int WARPS_N, int STAGES, bool PIPE = false>
-__global__ __launch_bounds__(64 * WARPS_M * WARPS_N) void k_gemm_tile_async(GemmArgs g) {
+// f(integral_constant<int, I>) for I = FROM .. TO-1, each call with its index a constant
+template <int FROM, int TO, class F>
+__device__ __forceinline__ void static_for(F&& f) {
+    if constexpr (FROM < TO) {
+        f(std::integral_constant<int, FROM>{});
+        static_for<FROM + 1, TO>(f);
+    }
+}
+
+// waits until at most `slices` slices of LOADS copies each are still on their way (a number the
+// unrolled loops around the call make a constant)
+template <int LOADS> __device__ inline void wait_slices(int slices) {
+    static_assert(LOADS * 3 < 64, "the counter holds 6 bits");
+    if (slices <= 0) wait_vmcnt<0>();
+    else if (slices == 1) wait_vmcnt<LOADS>();
+    else if (slices == 2) wait_vmcnt<LOADS * 2>();
+    else wait_vmcnt<LOADS * 3>();
+}
+
+template <int BM, int BN, int WARPS_M, int WARPS_N, int STAGES, int PIPE = 0, int BK = 64>
+__device__ __forceinline__ void gemm_tile(const GemmArgs& g, const int item, uint4* lds) {
     constexpr int WAVES = WARPS_M * WARPS_N;
-    constexpr int BK = 64, CH = BK / 8, RPL = 64 / CH;  // chunks of a row; rows that one load instruction covers
+    constexpr int CH = BK / 8, RPL = 64 / CH;           // chunks of a row; rows that one load instruction covers
+    constexpr int KS = BK / 16;                         // k-steps of a slice
+    static_assert(BK == 64 || BK == 32, "slices of 64 or of 32 columns");
     constexpr int WM = BM / WARPS_M, WN = BN / WARPS_N;
     constexpr int TM = WM / 32, TN = WN / 32;
     constexpr int ROWS = BM + BN;                       // rows of one stage: activations, then weights
@@ -368,9 +418,9 @@ __global__ __launch_bounds__(64 * WARPS_M * WARPS_N) void k_gemm_tile_async(Gemm
     static_assert(ROWS % (RPL * WAVES) == 0, "stage does not divide among waves");
     static_assert(LOADS * STAGES < 64, "too many loads in flight for the counter");
     constexpr int BUF = ROWS * CH;                      // chunks per stage
-    extern __shared__ uint4 lds[];                      // [STAGES][BUF]
-
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+                                                        // lds: [STAGES][BUF]
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);     // (the same in all lanes: what follows from it stays in scalar registers)
     const int wm0 = (wave / WARPS_N) * WM, wn0 = (wave % WARPS_N) * WN;
     // Workgroups are numbered along M first (m_fast) or along N first.  Consecutive
     // workgroups go to different XCDs, so with 8 row tiles each XCD keeps one activation tile
@@ -379,9 +429,25 @@ __global__ __launch_bounds__(64 * WARPS_M * WARPS_N) void k_gemm_tile_async(Gemm
     constexpr int BN_OUT_S = BN / 2;
     const int bn_out = g.epi == EPI_GATED ? BN_OUT_S : BN;
     const int tiles_n = (g.col1 - g.col0 + bn_out - 1) / bn_out;
-    const int tile_ = (int)(blockIdx.x / g.splits), split_ = (int)(blockIdx.x % g.splits);
-    const int bm_ = g.m_fast ? tile_ % tiles_m : tile_ / tiles_n;
-    const int bx = g.col0 / bn_out + (g.m_fast ? tile_ / tiles_m : tile_ % tiles_n);
+    const int tile_ = __builtin_amdgcn_readfirstlane(item / g.splits), split_ = __builtin_amdgcn_readfirstlane(item % g.splits);
+    // (the divisions are done in vector registers; their results go back to scalar ones)
+    // m_fast 2 (the column tiles are a multiple of 8, the row tiles at most 8): workgroup i runs on
+    // XCD i % 8, and each XCD takes every 8th column tile with all its row tiles, row tiles first, so
+    // a weight tile is fetched from memory by one XCD alone, and the XCD's 32 workgroups of a moment
+    // share 4 weight tiles and the activation tiles in its L2.  (Measured on the 8B shape's prompt
+    // step of 2,048 rows against m_fast 1: 29.4 -> 27.9 ms.  With 32 row tiles, in groups of 8 x 4
+    // tiles an XCD, it lost: 8192 x 28672 x 4096 in 1,776 us against 1,456.)
+    int bm_v, bn_v;
+    if (g.m_fast == 2) {
+        const int l = tile_ >> 3;
+        bm_v = l % tiles_m;
+        bn_v = (l / tiles_m) * 8 + (tile_ & 7);
+    } else {
+        bm_v = g.m_fast ? tile_ % tiles_m : tile_ / tiles_n;
+        bn_v = g.m_fast ? tile_ / tiles_m : tile_ % tiles_n;
+    }
+    const int bm_ = __builtin_amdgcn_readfirstlane(bm_v);
+    const int bx = __builtin_amdgcn_readfirstlane(g.col0 / bn_out + bn_v);
     const int k_begin = split_ * g.k_per_split;
     const int k_end = (k_begin + g.k_per_split) < g.K ? (k_begin + g.k_per_split) : g.K;
     const int m0 = bm_ * BM;
@@ -410,9 +476,10 @@ __global__ __launch_bounds__(64 * WARPS_M * WARPS_N) void k_gemm_tile_async(Gemm
             const int n = w_row_of<BN, WN>(row - BM, bx, g.N, g.epi, oc);
             const bool ok = oc < g.N && n < n_rows;
             if (g.w_packed) {
-                // row n % 16 of group n / 16; the slice's 64 columns are 2 blocks, chunk c the
+                // row n % 16 of group n / 16; a slice of 64 columns is 2 blocks, chunk c the
                 // (c % 4)-th of its row in block c / 4; a slice further on is 2 blocks = 1024 elements on,
-                // so one copy instruction of a wave (8 rows) reads two runs of 512 bytes
+                // so one copy instruction of a wave (8 rows) reads two runs of 512 bytes (a slice of 32
+                // columns is one block, and a copy instruction reads all 1024 bytes of it)
                 if (ok) p = g.w + (size_t)(n >> 4) * kblocks * 512 + (c >> 2) * 512 + (n & 15) * 32 + (c & 3) * 8;
                 step = BK * 16;
             } else if (ok) {
@@ -457,7 +524,127 @@ __global__ __launch_bounds__(64 * WARPS_M * WARPS_N) void k_gemm_tile_async(Gemm
 
     const int nk = (k_end - k_begin + BK - 1) / BK;
     const int lr = lane & 31, lg = lane >> 5;
-    if constexpr (PIPE) {
+    if constexpr (PIPE == 2) {
+        // The order of instructions is written out: a k-step is TM*TN slots, each one product
+        // followed by at most Q other instructions (a fragment read for the next k-step, a copy of
+        // a later slice), and nothing moves from slot to slot.  Every slice is whole here (the
+        // host sees to it), rows that do not exist are read from a row that does (their results
+        // are never stored), so a copy is a base that all lanes share, which moves on from slice
+        // to slice in scalar registers, and a fixed offset per lane.
+        constexpr int LA = BM / (RPL * WAVES);                    // the first LA copies of a slice bring activations
+        static_assert(BM % (RPL * WAVES) == 0 && LA < LOADS, "a copy instruction would straddle the operands");
+        static_assert(KS % 2 == 0, "the two sets of fragments alternate");
+        constexpr int DPK = TM * TN / 2;                          // copies issued in one k-step
+        constexpr int RS = TM * TN / (TM + TN) > 0 ? TM * TN / (TM + TN) : 1;     // a read every RS slots
+        constexpr int DS = TM * TN / DPK > 0 ? TM * TN / DPK : 1;                 // a copy every DS slots
+        constexpr int DSTEPS = (LOADS + DPK - 1) / DPK;           // k-steps that issue a slice's copies
+        static_assert(DSTEPS <= KS, "a slice's copies must be out before the next barrier");
+        uint32_t off[LOADS];
+        int oc0;
+        const int n_base = w_row_of<BN, WN>(0, bx, g.N, g.epi, oc0);
+#pragma unroll
+        for (int i = 0; i < LOADS; ++i) {
+            const int row = (i * WAVES + wave) * RPL + lane / CH;
+            const int c = (lane % CH) ^ swz<CH>(row);
+            if (i < LA) {
+                const int m = m0 + row < g.M ? row : g.M - 1 - m0;
+                off[i] = (uint32_t)(m * g.lda + c * 8) * 2u;
+            } else {
+                int oc;
+                int n = w_row_of<BN, WN>(row - BM, bx, g.N, g.epi, oc);
+                if (!(oc < g.N && n < n_rows)) n = n_base;
+                off[i] = g.w_packed ? (uint32_t)(((n >> 4) - (n_base >> 4)) * (int)kblocks * 512 + (c >> 2) * 512 + (n & 15) * 32 + (c & 3) * 8) * 2u
+                                    : (uint32_t)((n - n_base) * g.K + c * 8) * 2u;
+            }
+        }
+        const bf16_t* a_nxt = g.a + (size_t)m0 * g.lda + k_begin;
+        const bf16_t* w_nxt = g.w_packed ? g.w + (size_t)(n_base >> 4) * kblocks * 512 + (size_t)k_begin * 16
+                                         : g.w + (size_t)n_base * g.K + k_begin;
+        const int w_step = g.w_packed ? BK * 16 : BK;
+        bf16x8 af[2][TM], wf[2][TN];
+#define LONE_COPY(DI, DST)                                                                           \
+    lds_dma16_base((DI) < LA ? a_nxt : w_nxt, off[DI], lds_wave + (uint32_t)((DST) * BUF * 16 + (DI) * WAVES * 64 * 16));
+// one k-step: the products of fragment set F; if RD, the reads of k-step RD_KS of the slice in
+// buffer RD_BUF into the other set; if PART >= 0, copies PART*DPK .. of the next slice into buffer DST
+#define LONE_KSTEP(F, RD, RD_BUF, RD_KS, PART, DST)                                                  \
+    {                                                                                                \
+        const uint4* A_ = lds + (RD_BUF) * BUF;                                                      \
+        const uint4* W_ = A_ + BM * CH;                                                              \
+        const int c_ = (RD_KS) * 2 + lg;                                                             \
+        _Pragma("unroll") for (int t = 0; t < TM * TN; ++t) {                                        \
+            acc[t / TN][t % TN] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[F][t / TN], wf[F][t % TN], acc[t / TN][t % TN], 0, 0, 0); \
+            if ((RD) && t % RS == 0 && t / RS < TM + TN) {                                           \
+                const int q = t / RS;                                                                \
+                if (q < TM) {                                                                        \
+                    const int r = wm0 + q * 32 + lr;                                                 \
+                    af[(F) ^ 1][q] = as_bf16x8(A_[r * CH + (c_ ^ swz<CH>(r))]);                      \
+                } else {                                                                             \
+                    const int r = wn0 + (q - TM) * 32 + lr;                                          \
+                    wf[(F) ^ 1][q - TM] = as_bf16x8(W_[r * CH + (c_ ^ swz<CH>(r))]);                 \
+                }                                                                                    \
+            }                                                                                        \
+            if ((PART) >= 0 && t % DS == DS - 1 && t / DS < DPK) {                                   \
+                const int di = (PART) * DPK + t / DS;                                                \
+                if (di < LOADS) LONE_COPY(di, DST)                                                   \
+            }                                                                                        \
+            __builtin_amdgcn_sched_barrier(0);                                                       \
+        }                                                                                            \
+        if ((PART) == DSTEPS - 1) { a_nxt += BK; w_nxt += w_step; }                                                 \
+    }
+// the last k-step of the slice in buffer SB, behind the barrier that frees this buffer and
+// certifies the next slice, and the other k-steps of the slice after it
+#define LONE_ROUND(SB, SBN, COPY, WAITN)                                                             \
+    {                                                                                                \
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");                                           \
+        wait_slices<LOADS>(WAITN);                                                                   \
+        __builtin_amdgcn_s_barrier();                                                                \
+        __builtin_amdgcn_sched_barrier(0);                                                           \
+        LONE_KSTEP((KS - 1) & 1, true, SBN, 0, (COPY) ? 0 : -1, SB)                                  \
+        _Pragma("unroll") for (int ks = 0; ks < KS - 1; ++ks)                                        \
+            LONE_KSTEP(ks & 1, true, SBN, ks + 1, (COPY) && ks + 1 < DSTEPS ? ks + 1 : -1, SB)       \
+    }
+#pragma unroll
+        for (int st = 0; st < STAGES; ++st) {
+#pragma unroll
+            for (int i = 0; i < LOADS; ++i) LONE_COPY(i, st)
+            a_nxt += BK;
+            w_nxt += w_step;
+        }
+        wait_vmcnt<LOADS * (STAGES - 1)>();              // slice 0 has landed
+        __builtin_amdgcn_s_barrier();
+        {
+            const uint4* A_ = lds;
+            const uint4* W_ = A_ + BM * CH;
+#pragma unroll
+            for (int i = 0; i < TM; ++i) {
+                const int r = wm0 + i * 32 + lr;
+                af[0][i] = as_bf16x8(A_[r * CH + (lg ^ swz<CH>(r))]);
+            }
+#pragma unroll
+            for (int j = 0; j < TN; ++j) {
+                const int r = wn0 + j * 32 + lr;
+                wf[0][j] = as_bf16x8(W_[r * CH + (lg ^ swz<CH>(r))]);
+            }
+        }
+#pragma unroll
+        for (int ks = 0; ks < KS - 1; ++ks) LONE_KSTEP(ks & 1, true, 0, ks + 1, -1, 0)
+        int sb = 0;                                      // the buffer of slice s
+        for (int s_ = 0; s_ < nk - STAGES; ++s_) {
+            const int sbn = sb + 1 == STAGES ? 0 : sb + 1;
+            LONE_ROUND(sb, sbn, true, STAGES - 2)
+            sb = sbn;
+        }
+#pragma unroll
+        for (int r_ = 0; r_ < STAGES - 1; ++r_) {        // the slices after which nothing is copied
+            const int sbn = sb + 1 == STAGES ? 0 : sb + 1;
+            LONE_ROUND(sb, sbn, false, STAGES - 2 - r_)
+            sb = sbn;
+        }
+        LONE_KSTEP((KS - 1) & 1, false, 0, 0, -1, 0)
+#undef LONE_ROUND
+#undef LONE_KSTEP
+#undef LONE_COPY
+    } else if constexpr (PIPE == 1) {
         // The fragments of k-step ks+1 are read into a second set of registers before the
         // products of k-step ks are issued, also across the edge of a slice.  A buffer is free
         // for the slice STAGES further on as soon as every wave has left its slice (the barrier
@@ -483,17 +670,18 @@ __global__ __launch_bounds__(64 * WARPS_M * WARPS_N) void k_gemm_tile_async(Gemm
         }                                                                                            \
     }
         READ_FRAGS(0, 0, 0)
+        constexpr int PARTS = KS > 2 ? 3 : KS;
         for (int kt = 0; kt < nk; ++kt) {
 #pragma unroll
-            for (int ks = 0; ks < 4; ++ks) {
-                if (ks < 3) {
-                    if (ks < 2 && kt > 0) ASYNC_ISSUE_PART(kt + STAGES - 1, ks + 1, 3)
+            for (int ks = 0; ks < KS; ++ks) {
+                if (ks < KS - 1) {
+                    if (ks < PARTS - 1 && kt > 0) ASYNC_ISSUE_PART(kt + STAGES - 1, ks + 1, PARTS)
                     READ_FRAGS(kt % STAGES, ks + 1, (ks + 1) & 1)
                 } else {
                     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // this wave no longer reads slice kt ...
                     wait_vmcnt<LOADS * (STAGES - 2)>();                  // ... and its share of slice kt+1 has landed
                     __builtin_amdgcn_s_barrier();
-                    ASYNC_ISSUE_PART(kt + STAGES, 0, 3)                  // into the buffer of slice kt
+                    ASYNC_ISSUE_PART(kt + STAGES, 0, PARTS)              // into the buffer of slice kt
                     READ_FRAGS((kt + 1) % STAGES, 0, 0)
                 }
 #pragma unroll
@@ -541,13 +729,21 @@ __global__ __launch_bounds__(64 * WARPS_M * WARPS_N) void k_gemm_tile_async(Gemm
 #undef ASYNC_ISSUE
 #undef ASYNC_ISSUE_PART
     wait_vmcnt<0>();                                     // the trailing loads of zeros
+    // What the write-out derives from the lane's number is computed here, from a copy the compiler
+    // cannot trace back: values kept in registers through the loop were spilled, and a reload
+    // between the stores waits for every store before it (one counter for loads and stores).
+    int lane_after = lane;
+    asm volatile("" : "+v"(lane_after));
+    {
+    const int lane = lane_after, lr = lane & 31, lg = lane >> 5;
 
     // where 4 columns a lane may be written, the results go through LDS, each wave through an area
     // of its own, once no wave reads operands there any more
     static_assert((size_t)STAGES * ROWS * CH * 16 >= (size_t)WAVES * STAGE_FLOATS * 4, "no room for the waves' output areas");
     float* stage = reinterpret_cast<float*>(lds) + wave * STAGE_FLOATS;
     constexpr int NTP = TN % 2 == 0 ? 2 : 1;             // tiles written together
-    if (g.vec_out || g.rope.cs) __builtin_amdgcn_s_barrier();
+    const bool rotate = g.rope.cs != nullptr;
+    if (g.vec_out || rotate) __builtin_amdgcn_s_barrier();
 
     if (g.splits > 1 || g.raw) {
         // raw sums of this K range, by weight row: the epilogue belongs to k_gemm_finish
@@ -620,26 +816,32 @@ __global__ __launch_bounds__(64 * WARPS_M * WARPS_N) void k_gemm_tile_async(Gemm
             }
         return;
     }
-    if (g.vec_out || g.rope.cs) {
+    if (g.vec_out || rotate) {
+        // (tile by tile through a recursion of templates: a loop that the compiler declines to unroll,
+        // as it does one with 16 rotations in it, would index the accumulators at run time, and
+        // they would live in memory)
+        const bool adding = !rotate && g.epi == EPI_ACCUM;
+        float4 old[2][4 * NTP];                     // what the tiles of this round and of the next are added to
+        if (adding) load_old<NTP>(old[0], g.out, g.ldo, m0 + wm0, g.M, bx * BN + wn0, g.N, lane);
+        static_for<0, TM * (TN / NTP)>([&](auto idx) {
+            constexpr int i = decltype(idx)::value / (TN / NTP), j = decltype(idx)::value % (TN / NTP) * NTP;
+            constexpr int nxt = decltype(idx)::value + 1, ni = nxt / (TN / NTP), nj = nxt % (TN / NTP) * NTP;
+            if (adding && nxt < TM * (TN / NTP))
+                load_old<NTP>(old[nxt & 1], g.out, g.ldo, m0 + wm0 + ni * 32, g.M, bx * BN + wn0 + nj * 32, g.N, lane);
+            f32x16 t[NTP];
 #pragma unroll
-        for (int i = 0; i < TM; ++i)
+            for (int n = 0; n < NTP; ++n) {
+                const int col = bx * BN + wn0 + (j + n) * 32 + lr;
+                const float b = g.bias && col < g.N ? g.bias[col] : 0.f;
 #pragma unroll
-            for (int j = 0; j < TN; j += NTP) {
-                f32x16 t[NTP];
-#pragma unroll
-                for (int n = 0; n < NTP; ++n) {
-                    const int col = bx * BN + wn0 + (j + n) * 32 + lr;
-                    const float b = g.bias && col < g.N ? g.bias[col] : 0.f;
-#pragma unroll
-                    for (int e = 0; e < 16; ++e) t[n][e] = acc[i][j + n][e] + b;
-                }
-                if (g.rope.cs) {
-                    rope_tiles<NTP>(stage, t, g.rope, m0 + wm0 + i * 32, g.M, bx * BN + wn0 + j * 32, g.N, lane);
-                    continue;
-                }
-                write_tiles<NTP>(stage, t, g.out, g.ldo, g.epi == EPI_ACCUM ? 1 : (g.out_bf16 ? 2 : 0),
-                                 m0 + wm0 + i * 32, g.M, bx * BN + wn0 + j * 32, g.N, lane);
+                for (int e = 0; e < 16; ++e) t[n][e] = acc[i][j + n][e] + b;
             }
+            if (rotate)
+                rope_tiles<NTP>(stage, t, g.rope, m0 + wm0 + i * 32, g.M, bx * BN + wn0 + j * 32, g.N, lane);
+            else
+                write_tiles<NTP>(stage, t, g.out, g.ldo, g.epi == EPI_ACCUM ? 1 : (g.out_bf16 ? 2 : 0),
+                                 m0 + wm0 + i * 32, g.M, bx * BN + wn0 + j * 32, g.N, lane, adding ? old[decltype(idx)::value & 1] : nullptr);
+        });
         return;
     }
 #pragma unroll
@@ -655,6 +857,16 @@ __global__ __launch_bounds__(64 * WARPS_M * WARPS_N) void k_gemm_tile_async(Gemm
                 if (m < g.M) store_out(g, m, n, acc[i][j][e] + b);
             }
         }
+    }
+}
+
+// One workgroup a tile and K range.  (Workgroups that stay and take every 256th tile were measured
+// too, with the tiles assigned in turn or taken from a counter: no faster, and what the compiler then
+// keeps in registers from tile to tile it spills.)
+template <int BM, int BN, int WARPS_M, int WARPS_N, int STAGES, int PIPE = 0, int BK = 64>
+__global__ __launch_bounds__(64 * WARPS_M * WARPS_N) void k_gemm_tile_async(GemmArgs g) {
+    extern __shared__ uint4 lds[];
+    gemm_tile<BM, BN, WARPS_M, WARPS_N, STAGES, PIPE, BK>(g, (int)blockIdx.x, lds);
 }
 
 // Sums the K ranges of a split product in a fixed order and applies the epilogue.
@@ -749,16 +961,19 @@ __global__ __launch_bounds__(1024) void k_gemm_finish_norm(GemmArgs g) {
     }
 }
 
-template <int BM, int BN, int WM_, int WN_, int ST, bool PIPE = false>
+// (what a launcher answers when its kernel does not take the product and another one must)
+#define XR_NOT_TAKEN -1000
+
+template <int BM, int BN, int WM_, int WN_, int ST, int PIPE = 0, int BK = 64>
 static int launch_tile_async(GemmArgs g, hipStream_t stream) {
     if (g.epi == EPI_GATED && (BN / WN_ / 32) % 2) {
         xr_set_error("gemm: a %dx%d tile cannot pair gate and up columns", BM, BN);
         return XR_BAD_ARG;
     }
-    size_t smem = (size_t)ST * (BM + BN) * 8 * 16;
+    size_t smem = (size_t)ST * (BM + BN) * (BK / 8) * 16;
     static bool attr_set = false;
     if (!attr_set) {
-        hipError_t e = hipFuncSetAttribute((const void*)k_gemm_tile_async<BM, BN, WM_, WN_, ST, PIPE>,
+        hipError_t e = hipFuncSetAttribute((const void*)k_gemm_tile_async<BM, BN, WM_, WN_, ST, PIPE, BK>,
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
         if (e != hipSuccess) {
             (void)hipGetLastError();             // or the next launch's check would report this refusal
@@ -775,6 +990,7 @@ static int launch_tile_async(GemmArgs g, hipStream_t stream) {
     }
     unsigned tiles_n = (unsigned)((g.col1 - g.col0 + n_out_tile - 1) / n_out_tile), tiles_m = (unsigned)((g.M + BM - 1) / BM);
     unsigned tiles = tiles_n * tiles_m;
+    if (g.m_fast == 2 && (tiles_n % 8 || tiles_m > 8)) g.m_fast = 1;
     if (g.splits < 1 || !g.partial || g.col0 > 0 || g.col1 < g.N) g.splits = 1;
     if (g.splits > 1) {
         int slices = (g.K + 63) / 64;
@@ -783,6 +999,16 @@ static int launch_tile_async(GemmArgs g, hipStream_t stream) {
         g.splits = (slices + per - 1) / per;            // no empty range
     }
     if (g.splits == 1) g.k_per_split = ((g.K + 63) / 64) * 64;
+    if (PIPE == 2) {
+        // the loop with its instructions in a written order: whole slices only, at least ST of them
+        // in every K range, and every lane's piece within 4 GB of the tile's first
+        const int last = g.K - (g.splits - 1) * g.k_per_split;
+        const size_t span = (size_t)(g.epi == EPI_GATED ? g.N + BN : BN) + 16;
+        if (g.K % BK || last < ST * BK || g.k_per_split < ST * BK || (size_t)BM * g.lda * 2 >= (1ull << 32) ||
+            span * (size_t)(((g.K + 31) / 32) * 32) * 2 >= (1ull << 32)) {
+            return XR_NOT_TAKEN;
+        }
+    }
     if (g.raw && (!g.partial || g.col0 > 0 || g.col1 < g.N)) {
         xr_set_error("gemm: no room for the raw sums of a product whose epilogue is a kernel of its own");
         return XR_BAD_ARG;
@@ -794,7 +1020,7 @@ static int launch_tile_async(GemmArgs g, hipStream_t stream) {
         const void* base = raw_out ? (const void*)g.partial : (const void*)g.out;
         g.vec_out = g.N % 4 == 0 && ld % 4 == 0 && ((uintptr_t)base % 16) == 0 && (!raw_out || ((size_t)g.M * ld) % 4 == 0);
     }
-    k_gemm_tile_async<BM, BN, WM_, WN_, ST, PIPE><<<tiles * g.splits, 64 * WM_ * WN_, smem, stream>>>(g);
+    k_gemm_tile_async<BM, BN, WM_, WN_, ST, PIPE, BK><<<tiles * g.splits, 64 * WM_ * WN_, smem, stream>>>(g);
     XR_CHECK_LAUNCH("gemm_tile_async");
     if (g.norm_whole) {
         k_gemm_finish_norm<<<(unsigned)g.M, 1024, 0, stream>>>(g);
@@ -996,8 +1222,30 @@ __global__ __launch_bounds__(64 * KSW) void k_gemm_skinny(GemmArgs g) {
 
 static int launch_tile_variant(int variant, const GemmArgs& g, hipStream_t stream) {
     // (the loop that reads its fragments a k-step ahead is the faster one but for the 256x192 tile)
-    if (variant == 12) return launch_tile_async<256, 128, 4, 2, 3, true>(g, stream);
-    if (variant == 14) return launch_tile_async<256, 256, 4, 2, 2, true>(g, stream);
+    // Two kernels for the 256x256 and the 256x128 tile: four waves, one a SIMD, each with a quarter of
+    // the tile and the order of its instructions written out (PIPE 2), where the product allows it
+    // (whole slices of K, enough of them, no rotation), else eight waves and the loop that reads its
+    // fragments a k-step ahead.  Measured at 2,048 rows (us, eight waves / four): gate+up 489 / 419,
+    // the down product 221 / 194, the output product 69 / 61; 8192 x 28672 x 4096: 1,611 / 1,417.
+    // (A product that rotates its result keeps the eight waves unless the four are asked for by name:
+    // the rotation is work for the vector units, where four waves with 16 tiles each took 148 us for the
+    // q/k/v product of 2,048 rows against 118 in 256x192 tiles with eight.)
+    if ((variant == 12 && !g.rope.cs) || variant == 55) {
+        const int rc = launch_tile_async<256, 128, 2, 2, 3, 2, 64>(g, stream);
+        if (rc != XR_NOT_TAKEN) return rc;
+    }
+    if (variant == 12) return launch_tile_async<256, 128, 4, 2, 3, 1>(g, stream);
+    if ((variant == 14 && !g.rope.cs) || variant == 51) {
+        const int rc = launch_tile_async<256, 256, 2, 2, 2, 2, 64>(g, stream);
+        if (rc != XR_NOT_TAKEN) return rc;
+    }
+    if (variant == 14) return launch_tile_async<256, 256, 4, 2, 2, 1>(g, stream);
+    if (variant == 112) return launch_tile_async<256, 128, 4, 2, 3, 1>(g, stream);     // (the eight-wave kernels by name, for tests)
+    if (variant == 114) return launch_tile_async<256, 256, 4, 2, 2, 1>(g, stream);
+    if (variant == 51 || variant == 55) {
+        xr_set_error("gemm: the four-wave kernel does not take K %d in %d ranges, lda %d, or a rotation", g.K, g.splits, g.lda);
+        return XR_BAD_ARG;
+    }
     // (four slices in flight: with 65 to 512 rows these products are bound by how fast the weights
     // arrive, and two slices, one of them in use, left a compute unit 32 KB on its way: the down
     // product at 128 rows 46 -> 37 us, gate+up 72 -> 57, q/k/v at 512 rows 65 -> 45)
@@ -1132,8 +1380,8 @@ extern "C" int xr_gemm_bf16(void* out, const void* a, const void* w, const float
     // from XR_ROPE_TILE_ROWS rows on; below, the kernel that adds up the K ranges rotates and caches
     const bool rope_direct = rope && M >= XR_ROPE_TILE_ROWS;
     if (rope) {
-        XR_REQUIRE(variant == 0 && epi == EPI_STORE && !(norm && norm->xg),
-                   "gemm: rotation and cache write are folded only into a plain product whose kernel the library chooses");
+        XR_REQUIRE((variant == 0 || (rope_direct && variant >= 10 && variant < 200)) && epi == EPI_STORE && !(norm && norm->xg),
+                   "gemm: rotation and cache write are folded only into a plain product whose kernel the library chooses (or, with many rows, a tile kernel named)");
         if (rope_direct) {
             XR_REQUIRE(rope->cs_table || (workspace && (size_t)M * (rope->rot / 2 + 1) * sizeof(float2) <= workspace_bytes),
                        "gemm: rotation after a product of %d rows needs a workspace for its table", M);
@@ -1171,6 +1419,7 @@ extern "C" int xr_gemm_bf16(void* out, const void* a, const void* w, const float
             }
         }
     }
+    if (variant >= 2000) { g.m_fast = 2; variant -= 2000; }
     if (variant >= 1000) { g.m_fast = 1; variant -= 1000; }
     const bool sw = epi == EPI_GATED;
     const int w_rows = epi == EPI_GATED ? 2 * N : N;
@@ -1201,14 +1450,18 @@ extern "C" int xr_gemm_bf16(void* out, const void* a, const void* w, const float
             // are too few for the chip competes with K split among workgroups (below).
             // (The 256 compute units and the tiles' relative rates below are tuning measured on an
             // MI355X with the 8B shape's products, not limits: elsewhere they cost speed only.)
-            struct Cand { int variant, bm, bn; double rate; };
-            const Cand cands[4] = {{14, 256, 256, 1.0}, {26, 256, 192, 0.93}, {12, 256, 128, 0.90}, {17, 128, 128, 0.74}};
+            // (rate: of the tile's products, relative to 256x256; fixed: seconds a round beside them.  At
+            // 2,048 rows a round of 256x256 tiles took 107 us with K = 4,096 and 191 with 7,168, one of
+            // 256x128 tiles 61 us with K = 4,096 and 194 with 14,336, one of 256x192 tiles 118.)
+            struct Cand { int variant, bm, bn; double rate, fixed; };
+            const double four = rope_direct ? 0.85 : 1.0;        // (the eight-wave kernels of these tiles, which a rotating product takes)
+            const Cand cands[4] = {{14, 256, 256, 1.0 * four, 0.0}, {26, 256, 192, 0.73, 8e-6}, {12, 256, 128, 1.0 * four, 8e-6},
+                                   {17, 128, 128, 0.63, 0.0}};
             auto width = [&](const Cand& c) { return sw ? c.bn / 2 : c.bn; };
             auto usable = [&](const Cand& c) { return !(sw && c.variant == 26); };
             auto count = [&](const Cand& c, int cols) { return ((M + c.bm - 1) / c.bm) * ((cols + width(c) - 1) / width(c)); };
-            auto time_of = [&](const Cand& c, int cols) { return (double)((count(c, cols) + 255) / 256) * c.bm * c.bn / c.rate; };
-            // Times in seconds: a 256x256 tile's products over K columns take 65536 K x 0.5e-12 s at
-            // full rate (134 us at K = 4,096, measured 137).  A launch whose tiles are too few for the
+            // Times in seconds: a 256x256 tile's products over K columns take 65536 K x 0.4e-12 s at
+            // full rate (107 us at K = 4,096, as measured).  A launch whose tiles are too few for the
             // chip (under 160) may split K so that its workgroups make one round; the kernel that then
             // adds the ranges up moves (ranges x their width + 2 x N) x M x 4 bytes at about 4.5 TB/s
             // and costs a launch, and it writes the norm that follows, if one was asked for, which
@@ -1216,8 +1469,10 @@ extern "C" int xr_gemm_bf16(void* out, const void* a, const void* w, const float
             // rows (us, model / measured): down at 512 rows in 256x128 tiles and 4 ranges 79 / 74-79, in
             // 128x128 and 2 ranges 90 / 94, in 256x256 and 8 ranges 80 / 79; q/k/v at 256 rows in 256x128
             // and 5 ranges 28 / 32, in 128x128 and 2 ranges 31 / 36.
-            const double unit = 0.5e-12;
-            auto seconds = [&](const Cand& c, int cols) { return time_of(c, cols) * K * unit; };
+            const double unit = 0.4e-12;
+            auto seconds = [&](const Cand& c, int cols) {
+                return (double)((count(c, cols) + 255) / 256) * ((double)c.bm * c.bn / c.rate * K * unit + c.fixed);
+            };
             auto adding = [&](int ranges) {
                 return ((double)ranges * w_rows + 2.0 * N) * M * 4 / 4.5e12 + 3e-6 - (want_whole_norm ? 11e-6 : 0.0);
             };
@@ -1230,7 +1485,7 @@ extern "C" int xr_gemm_bf16(void* out, const void* a, const void* w, const float
                 int sp = 1;
                 if (c < 160 && workspace && !rope_direct) {
                     const int s2 = pick_splits(c);
-                    const double ts = (double)cands[i].bm * cands[i].bn / cands[i].rate * ((K + s2 - 1) / s2) * unit + adding(s2);
+                    const double ts = (double)cands[i].bm * cands[i].bn / cands[i].rate * ((K + s2 - 1) / s2) * unit + cands[i].fixed + adding(s2);
                     if (s2 >= 2 && ts < t) { t = ts; sp = s2; }
                 }
                 if (t < t_best) { best = i; best_splits = sp; t_best = t; }
@@ -1247,7 +1502,7 @@ extern "C" int xr_gemm_bf16(void* out, const void* a, const void* w, const float
                 }
             }
             variant = cands[best].variant;
-            g.m_fast = 1;
+            g.m_fast = 2;                      // (where the tiles' counts allow, else 1: the launcher sees to it)
             if (second >= 0) {
                 GemmArgs g2 = g;
                 g.col1 = cols_first;

@@ -475,7 +475,7 @@ class Ops:
 
     def project_rope_kv_write(self, h, w, bias, k_cache, v_cache, positions, req_of_token, block_table,
                               inv_freq, H: int, Hk: int, D: int, rot: int, interleaved: bool, mscale: float,
-                              page_size: int, paired: bool = False, cs_table=None) -> torch.Tensor:
+                              page_size: int, paired: bool = False, cs_table=None, variant: int = 0) -> torch.Tensor:
         """``[q | k | v] = h @ w^T (+ bias)``, queries and keys rotated, keys and values written
         to their pages; returns the rotated queries ``[T, H*D]`` in the compute dtype.
 
@@ -486,7 +486,8 @@ class Ops:
         512 the tile kernel (with the rows' cosines and sines from a table made first), which
         saves a kernel; in float32, and where the kernels' conditions on sizes do not hold, the
         product and ``rope_kv_write`` run one after the other.  ``cs_table``: a callable that returns the
-        step's ``rope_table`` (asked for only where the tile kernel rotates)."""
+        step's ``rope_table`` (asked for only where the tile kernel rotates).  ``variant``: a tile kernel
+        by number instead of the library's choice (tests; from 512 rows on)."""
         rows = h.data if isinstance(h, UnscaledRows) else h
         wt = w.data if isinstance(w, PackedWeight) else w
         T, Q, KV = rows.shape[0], H * D, Hk * D
@@ -513,7 +514,7 @@ class Ops:
             table = cs_table() if (cs_table is not None and T >= self.ROPE_TILE_ROWS and rot > 0) else None
             rp.cs_table = _ptr(table)
             self.lib.check(self.lib.xr_gemm_bf16(None, rows.data_ptr(), wt.data_ptr(), _ptr(bias), T, w.shape[0],
-                                                 rows.shape[1], rows.stride(0), w.shape[0], XR_F32, 0, 0, 0,
+                                                 rows.shape[1], rows.stride(0), w.shape[0], XR_F32, 0, 0, variant,
                                                  1 if isinstance(w, PackedWeight) else 0,
                                                  *self._gemm_workspace(rows.device),
                                                  C.addressof(norm) if norm is not None else None,
