@@ -116,15 +116,15 @@ def test_linear_bf16_mfma(ops, M, N, K):
                        a.double() @ w.double().T + b.double()) < 1e-5
 
 
-@pytest.mark.parametrize("variant", [51, 55])
-@pytest.mark.parametrize("M,N,K", [(65, 100, 192), (300, 333, 256), (513, 520, 1024), (256, 256, 4096)])
+@pytest.mark.parametrize("variant", [51, 55, 58])
+@pytest.mark.parametrize("M,N,K", [(65, 100, 256), (300, 333, 256), (513, 520, 1024), (256, 256, 4096)])
 def test_four_wave_tile_kernels(ops, variant, M, N, K):
-    """The 256x256 and 256x128 tiles' kernels with four waves and a written order of instructions, by
-    name (they refuse what they do not take): rows and columns that fill no tile, plain and packed
+    """The 256x256, 256x128 and 128x128 tiles' kernels with four waves and a written order of instructions,
+    by name (they refuse what they do not take): rows and columns that fill no tile, plain and packed
     weights, a bias, adding into the output, the gated epilogue; against the eight-wave kernel of
     the same tile the sums are the same to the bit (same products in the same order)."""
     from xyntetik_runner_amd.csrc.ops import KernelError
-    eight_waves = 114 if variant == 51 else 112
+    eight_waves = {51: 114, 55: 112, 58: 117}[variant]            # (the same tile with the other loop)
     a = (torch.randn(M, K, device=DEV) * 0.5).bfloat16()
     w = (torch.randn(N, K, device=DEV) * 0.1).bfloat16()
     b = torch.randn(N, device=DEV) * 0.1
@@ -149,7 +149,7 @@ def test_four_wave_tile_kernels(ops, variant, M, N, K):
     w3 = (torch.randn(N, 72, device=DEV) * 0.1).bfloat16()
     with pytest.raises(KernelError, match="four-wave"):
         ops.linear(a2, w3, variant=variant)
-    assert rel(ops.linear(a2, w3, out_dtype=torch.float32, variant=14 if variant == 51 else 12), a2.double() @ w3.double().T) < 1e-5
+    assert rel(ops.linear(a2, w3, out_dtype=torch.float32, variant={51: 14, 55: 12, 58: 17}[variant]), a2.double() @ w3.double().T) < 1e-5
 
 
 @pytest.mark.parametrize("M", [8, 40, 300])

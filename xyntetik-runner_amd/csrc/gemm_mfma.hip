@@ -534,9 +534,10 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, const int item, uin
         constexpr int LA = BM / (RPL * WAVES);                    // the first LA copies of a slice bring activations
         static_assert(BM % (RPL * WAVES) == 0 && LA < LOADS, "a copy instruction would straddle the operands");
         static_assert(KS % 2 == 0, "the two sets of fragments alternate");
-        constexpr int DPK = TM * TN / 2;                          // copies issued in one k-step
-        constexpr int RS = TM * TN / (TM + TN) > 0 ? TM * TN / (TM + TN) : 1;     // a read every RS slots
-        constexpr int DS = TM * TN / DPK > 0 ? TM * TN / DPK : 1;                 // a copy every DS slots
+        constexpr int SLOTS = TM * TN, READS = TM + TN;
+        // copies issued in one k-step: one every other slot, or what brings a slice's copies out in KS-1 k-steps
+        constexpr int DPK = SLOTS / 2 > (LOADS + KS - 2) / (KS - 1) ? SLOTS / 2 : (LOADS + KS - 2) / (KS - 1);
+        constexpr int DOFF = SLOTS / DPK > 1 ? SLOTS / DPK - 1 : 0;               // (copies in the slots between the reads)
         constexpr int DSTEPS = (LOADS + DPK - 1) / DPK;           // k-steps that issue a slice's copies
         static_assert(DSTEPS <= KS, "a slice's copies must be out before the next barrier");
         uint32_t off[LOADS];
@@ -571,21 +572,24 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, const int item, uin
         const uint4* A_ = lds + (RD_BUF) * BUF;                                                      \
         const uint4* W_ = A_ + BM * CH;                                                              \
         const int c_ = (RD_KS) * 2 + lg;                                                             \
-        _Pragma("unroll") for (int t = 0; t < TM * TN; ++t) {                                        \
+        _Pragma("unroll") for (int t = 0; t < SLOTS; ++t) {                                          \
             acc[t / TN][t % TN] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[F][t / TN], wf[F][t % TN], acc[t / TN][t % TN], 0, 0, 0); \
-            if ((RD) && t % RS == 0 && t / RS < TM + TN) {                                           \
-                const int q = t / RS;                                                                \
-                if (q < TM) {                                                                        \
-                    const int r = wm0 + q * 32 + lr;                                                 \
-                    af[(F) ^ 1][q] = as_bf16x8(A_[r * CH + (c_ ^ swz<CH>(r))]);                      \
-                } else {                                                                             \
-                    const int r = wn0 + (q - TM) * 32 + lr;                                          \
-                    wf[(F) ^ 1][q - TM] = as_bf16x8(W_[r * CH + (c_ ^ swz<CH>(r))]);                 \
+            _Pragma("unroll") for (int q = 0; q < READS; ++q) {             /* read q in slot q SLOTS / READS */ \
+                if ((RD) && q * SLOTS / READS == t) {                                                \
+                    if (q < TM) {                                                                    \
+                        const int r = wm0 + q * 32 + lr;                                             \
+                        af[(F) ^ 1][q] = as_bf16x8(A_[r * CH + (c_ ^ swz<CH>(r))]);                  \
+                    } else {                                                                         \
+                        const int r = wn0 + (q - TM) * 32 + lr;                                      \
+                        wf[(F) ^ 1][q - TM] = as_bf16x8(W_[r * CH + (c_ ^ swz<CH>(r))]);             \
+                    }                                                                                \
                 }                                                                                    \
             }                                                                                        \
-            if ((PART) >= 0 && t % DS == DS - 1 && t / DS < DPK) {                                   \
-                const int di = (PART) * DPK + t / DS;                                                \
-                if (di < LOADS) LONE_COPY(di, DST)                                                   \
+            _Pragma("unroll") for (int d = 0; d < DPK; ++d) {               /* copy d in slot d SLOTS / DPK (+ DOFF) */ \
+                if ((PART) >= 0 && d * SLOTS / DPK + DOFF == t) {                                    \
+                    const int di = (PART) * DPK + d;                                                 \
+                    if (di < LOADS) LONE_COPY(di, DST)                                               \
+                }                                                                                    \
             }                                                                                        \
             __builtin_amdgcn_sched_barrier(0);                                                       \
         }                                                                                            \
@@ -1242,14 +1246,19 @@ static int launch_tile_variant(int variant, const GemmArgs& g, hipStream_t strea
     if (variant == 14) return launch_tile_async<256, 256, 4, 2, 2, 1>(g, stream);
     if (variant == 112) return launch_tile_async<256, 128, 4, 2, 3, 1>(g, stream);     // (the eight-wave kernels by name, for tests)
     if (variant == 114) return launch_tile_async<256, 256, 4, 2, 2, 1>(g, stream);
-    if (variant == 51 || variant == 55) {
-        xr_set_error("gemm: the four-wave kernel does not take K %d in %d ranges, lda %d, or a rotation", g.K, g.splits, g.lda);
-        return XR_BAD_ARG;
-    }
     // (four slices in flight: with 65 to 512 rows these products are bound by how fast the weights
     // arrive, and two slices, one of them in use, left a compute unit 32 KB on its way: the down
     // product at 128 rows 46 -> 37 us, gate+up 72 -> 57, q/k/v at 512 rows 65 -> 45)
-    if (variant == 17) return launch_tile_async<128, 128, 2, 2, 4, false>(g, stream);
+    // (the written order also where the weights' arrival bounds the kernel: little, 1-2%)
+    if ((variant == 17 && !g.rope.cs) || variant == 58) {
+        const int rc = launch_tile_async<128, 128, 2, 2, 4, 2, 64>(g, stream);
+        if (rc != XR_NOT_TAKEN) return rc;
+    }
+    if (variant == 17 || variant == 117) return launch_tile_async<128, 128, 2, 2, 4, false>(g, stream);
+    if (variant == 51 || variant == 55 || variant == 58) {
+        xr_set_error("gemm: the four-wave kernel does not take K %d in %d ranges, lda %d, or a rotation", g.K, g.splits, g.lda);
+        return XR_BAD_ARG;
+    }
     if (variant == 26) return launch_tile_async<256, 192, 4, 2, 2>(g, stream);
     xr_set_error("gemm: unknown variant %d", variant);
     return XR_BAD_ARG;
@@ -1543,7 +1552,9 @@ extern "C" int xr_gemm_bf16(void* out, const void* a, const void* w, const float
         // (four slices in flight instead of three: the gate and up product 50.6 -> 47.0 us at 64 rows,
         // the others as before; five, 256 weight rows a tile, or twice the K ranges for two
         // workgroups a compute unit gain nothing or lose)
-        return launch_tile_async<64, 128, 2, 2, 4>(g, stream);
+        // (with the order of instructions written out where the product allows: decode at batch 64 7.43 -> 7.31 ms)
+        const int rc = launch_tile_async<64, 128, 2, 2, 4, 2, 64>(g, stream);
+        return rc != XR_NOT_TAKEN ? rc : launch_tile_async<64, 128, 2, 2, 4>(g, stream);
     }
     return launch_tile_variant(variant, g, stream);
 }
