@@ -274,45 +274,64 @@ __device__ inline void rope_tiles(float* stage, const f32x16 (&t)[NT], const Rop
         const int sec = col < Q ? 0 : 1;
         const int rel = col - (sec ? Q : 0);
         const int hs = rel / rp.D, c = rel - hs * rp.D;
+        constexpr int ITS = 32 / RPI;
+        const int hi = (c >> 3) & 1, j0 = (c >> 4) * 8 + (c & 7);           // (paired order)
+        // everything the rows' stores need from memory first (cosines and sines, the keys' places),
+        // then the arithmetic and the stores: a load behind a store waits for that store, since
+        // they may be the same memory for all the compiler knows, and one trip to memory after the
+        // other was most of this function's time
+        float2 f[ITS][4];
+        size_t kdst[ITS];
 #pragma unroll
-        for (int it = 0; it < 32 / RPI; ++it) {
+        for (int it = 0; it < ITS; ++it) {
+            const int m = m_base + it * RPI + lane / CPR;
+            if (m >= M) continue;
+            if (c < rp.rot) {
+                const float2* cs = rp.cs + (size_t)m * half;
+                if (rp.interleaved) {
+#pragma unroll
+                    for (int e = 0; e < 4; e += 2)
+                        if (c + e < rp.rot) f[it][e] = cs[(c + e) >> 1];
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) f[it][e] = cs[j0 + e];
+                }
+            }
+            if (sec == 1) {
+                const PageRef pr = page_of(rp.block_table, rp.table_stride, rp.req_of_token[m], rp.positions[m], rp.page_shift, rp.page_mask);
+                kdst[it] = (((size_t)pr.page * rp.Hk + hs) * rp.page_size + pr.off) * rp.D;
+            }
+        }
+#pragma unroll
+        for (int it = 0; it < ITS; ++it) {
             const int row = it * RPI + lane / CPR, m = m_base + row;
             if (m >= M) continue;
             const float4 x = *reinterpret_cast<const float4*>(stage + row * LD + ch * 4);
             float o[4] = {x.x, x.y, x.z, x.w};
             int d0 = c;
             if (c < rp.rot) {
-                const float2* cs = rp.cs + (size_t)m * half;
                 if (rp.interleaved) {
 #pragma unroll
                     for (int e = 0; e < 4; e += 2)
                         if (c + e < rp.rot) {
-                            const float2 f = cs[(c + e) >> 1];
                             const float x0 = o[e], x1 = o[e + 1];
-                            o[e] = x0 * f.x - x1 * f.y;
-                            o[e + 1] = x0 * f.y + x1 * f.x;
+                            o[e] = x0 * f[it][e].x - x1 * f[it][e].y;
+                            o[e + 1] = x0 * f[it][e].y + x1 * f[it][e].x;
                         }
                 } else {
-                    const int hi = (c >> 3) & 1, j0 = (c >> 4) * 8 + (c & 7);
                     const float4 y = *reinterpret_cast<const float4*>(stage + row * LD + (ch ^ 2) * 4);
                     const float pv[4] = {y.x, y.y, y.z, y.w};
 #pragma unroll
                     for (int e = 0; e < 4; ++e) {
-                        const float2 f = cs[j0 + e];
                         const float x0 = hi ? pv[e] : o[e], x1 = hi ? o[e] : pv[e];
-                        o[e] = hi ? x0 * f.y + x1 * f.x : x0 * f.x - x1 * f.y;
+                        o[e] = hi ? x0 * f[it][e].y + x1 * f[it][e].x : x0 * f[it][e].x - x1 * f[it][e].y;
                     }
                     d0 = j0 + hi * half;
                 }
             }
             const uint2 w = make_uint2(pack_bf16x2(o[0], o[1]), pack_bf16x2(o[2], o[3]));
-            if (sec == 0) {
-                *reinterpret_cast<uint2*>(rp.q_out + ((size_t)m * rp.H + hs) * rp.D + d0) = w;
-            } else {
-                const int pos = rp.positions[m];
-                const PageRef pr = page_of(rp.block_table, rp.table_stride, rp.req_of_token[m], pos, rp.page_shift, rp.page_mask);
-                *reinterpret_cast<uint2*>(rp.k_cache + (((size_t)pr.page * rp.Hk + hs) * rp.page_size + pr.off) * rp.D + d0) = w;
-            }
+            if (sec == 0) *reinterpret_cast<uint2*>(rp.q_out + ((size_t)m * rp.H + hs) * rp.D + d0) = w;
+            else *reinterpret_cast<uint2*>(rp.k_cache + kdst[it] + d0) = w;
         }
     }
     if (col_base + SW > Q + KV && KV > 0) {
@@ -1232,8 +1251,8 @@ static int launch_tile_variant(int variant, const GemmArgs& g, hipStream_t strea
     // fragments a k-step ahead.  Measured at 2,048 rows (us, eight waves / four): gate+up 489 / 419,
     // the down product 221 / 194, the output product 69 / 61; 8192 x 28672 x 4096: 1,611 / 1,417.
     // (A product that rotates its result keeps the eight waves unless the four are asked for by name:
-    // the rotation is work for the vector units, where four waves with 16 tiles each took 148 us for the
-    // q/k/v product of 2,048 rows against 118 in 256x192 tiles with eight.)
+    // the rotation is work for the vector units, where four waves with 16 tiles each took 128 us for the
+    // q/k/v product of 2,048 rows against 115 in 256x192 tiles with eight.)
     if ((variant == 12 && !g.rope.cs) || variant == 55) {
         const int rc = launch_tile_async<256, 128, 2, 2, 3, 2, 64>(g, stream);
         if (rc != XR_NOT_TAKEN) return rc;
