@@ -5,7 +5,9 @@
 //     computes a BM x BN tile; both operands are copied from memory straight into LDS in
 //     64-wide K slices (16-byte chunks, XOR-swizzled so that fragment reads do not collide),
 //     several slices ahead, and fed to v_mfma_f32_32x32x16_bf16.  With few tiles K is split
-//     over workgroups and k_gemm_finish adds the parts in a fixed order.
+//     over workgroups and k_gemm_finish adds the parts in a fixed order.  Three main loops:
+//     four waves with the order of their instructions written out (what serves, where K is
+//     whole slices), and two with eight waves for the rest.
 //   * k_gemm_skinny: M <= 16 (decoding).  The product is bound by reading the weights
 //     once, so each wave streams 16 weight rows straight from memory into MFMA fragments
 //     (v_mfma_f32_16x16x32_bf16, weights as the A operand, tokens as the B operand) with
@@ -384,9 +386,11 @@ __device__ inline int w_row_of(int r, int bx, int N, int epi, int& out_col) {
 // kt, slices kt+1 .. kt+STAGES-1 are on their way, with no registers and no LDS-write
 // instructions spent on them.  A lane whose piece lies outside the matrices reads from a
 // block of zeros instead, so every slice issues the same number of loads and one counter
-// wait (vmcnt) tells when a slice has landed.  Two main loops: in the plain one a k-step reads
-// its fragments and multiplies; with PIPE the fragments of k-step ks+1 (also the next slice's
-// first) are read into a second set of registers before the products of k-step ks are issued.
+// wait (vmcnt) tells when a slice has landed.  Three main loops (PIPE): in the plain one (0) a
+// k-step reads its fragments and multiplies; in the second (1) the fragments of k-step ks+1 (also
+// the next slice's first) are read into a second set of registers before the products of k-step ks
+// are issued; the third (2) is the second with the order of its instructions written out, slot by
+// slot, for waves that have a SIMD to themselves (described where it stands).
 // Measured on MI355X (8192 x 28672 x 4096, random data): a compute unit is given its operands
 // at up to 50 bytes a cycle from L2 and reads LDS at 190, the matrix cores alone do 1.8 PFLOP/s
 // (the clock falls from 2.4 to 1.8-2.0 GHz under them); a 256x256 tile spent 115 us in its loop
