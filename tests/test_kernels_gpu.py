@@ -117,7 +117,7 @@ def test_linear_bf16_mfma(ops, M, N, K):
 
 
 @pytest.mark.parametrize("variant", [51, 55, 58])
-@pytest.mark.parametrize("M,N,K", [(65, 100, 256), (300, 333, 256), (513, 520, 1024), (256, 256, 4096)])
+@pytest.mark.parametrize("M,N,K", [(65, 100, 256), (300, 333, 256), (513, 520, 1024), (256, 256, 4096), (300, 1352, 256)])
 def test_four_wave_tile_kernels(ops, variant, M, N, K):
     """The 256x256, 256x128 and 128x128 tiles' kernels with four waves and a written order of instructions,
     by name (they refuse what they do not take): rows and columns that fill no tile, plain and packed
@@ -133,6 +133,10 @@ def test_four_wave_tile_kernels(ops, variant, M, N, K):
         got = ops.linear(a, wt, bias=b, out_dtype=torch.float32, variant=variant)
         assert rel(got, want) < 1e-5
         assert torch.equal(got, ops.linear(a, wt, bias=b, out_dtype=torch.float32, variant=eight_waves))
+        # the same tiles in the other orders of workgroups (side by side along the rows; by XCD, with
+        # column tiles that are no multiple of 8: workgroups without a tile leave)
+        for order in (1000, 2000):
+            assert torch.equal(got, ops.linear(a, wt, bias=b, out_dtype=torch.float32, variant=order + variant))
         assert rel(ops.linear(a, wt, bias=b, variant=variant), want) < 6e-3
     base = torch.randn(M, N, device=DEV)
     out = base.clone()

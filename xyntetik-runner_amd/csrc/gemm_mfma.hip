@@ -454,10 +454,11 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, const int item, uin
     const int tiles_n = (g.col1 - g.col0 + bn_out - 1) / bn_out;
     const int tile_ = __builtin_amdgcn_readfirstlane(item / g.splits), split_ = __builtin_amdgcn_readfirstlane(item % g.splits);
     // (the divisions are done in vector registers; their results go back to scalar ones)
-    // m_fast 2 (the column tiles are a multiple of 8, the row tiles at most 8): workgroup i runs on
-    // XCD i % 8, and each XCD takes every 8th column tile with all its row tiles, row tiles first, so
-    // a weight tile is fetched from memory by one XCD alone, and the XCD's 32 workgroups of a moment
-    // share 4 weight tiles and the activation tiles in its L2.  (Measured on the 8B shape's prompt
+    // m_fast 2 (at most 8 row tiles): workgroup i runs on XCD i % 8, and each XCD takes every 8th
+    // column tile with all its row tiles, row tiles first, so a weight tile is fetched from memory by
+    // one XCD alone, and the XCD's 32 workgroups of a moment share 4 weight tiles and the activation
+    // tiles in its L2.  (Where the column tiles are no multiple of 8 the launch has workgroups for 8
+    // equal shares, and those of a share's missing column leave at once.)  (Measured on the 8B shape's prompt
     // step of 2,048 rows against m_fast 1: 29.4 -> 27.9 ms.  With 32 row tiles, in groups of 8 x 4
     // tiles an XCD, it lost: 8192 x 28672 x 4096 in 1,776 us against 1,456.)
     int bm_v, bn_v;
@@ -465,6 +466,7 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, const int item, uin
         const int l = tile_ >> 3;
         bm_v = l % tiles_m;
         bn_v = (l / tiles_m) * 8 + (tile_ & 7);
+        if (bn_v >= tiles_n) return;
     } else {
         bm_v = g.m_fast ? tile_ % tiles_m : tile_ / tiles_n;
         bn_v = g.m_fast ? tile_ / tiles_m : tile_ % tiles_n;
@@ -1017,7 +1019,8 @@ static int launch_tile_async(GemmArgs g, hipStream_t stream) {
     }
     unsigned tiles_n = (unsigned)((g.col1 - g.col0 + n_out_tile - 1) / n_out_tile), tiles_m = (unsigned)((g.M + BM - 1) / BM);
     unsigned tiles = tiles_n * tiles_m;
-    if (g.m_fast == 2 && (tiles_n % 8 || tiles_m > 8)) g.m_fast = 1;
+    if (g.m_fast == 2 && (tiles_m > 8 || tiles_n < 8)) g.m_fast = 1;
+    if (g.m_fast == 2) tiles = 8 * tiles_m * ((tiles_n + 7) / 8);
     if (g.splits < 1 || !g.partial || g.col0 > 0 || g.col1 < g.N) g.splits = 1;
     if (g.splits > 1) {
         int slices = (g.K + 63) / 64;
