@@ -278,14 +278,19 @@ __device__ inline void rope_tiles(float* stage, const f32x16 (&t)[NT], const Rop
         const int hs = rel / rp.D, c = rel - hs * rp.D;
         constexpr int ITS = 32 / RPI;
         const int hi = (c >> 3) & 1, j0 = (c >> 4) * 8 + (c & 7);           // (paired order)
-        // everything the rows' stores need from memory first (cosines and sines, the keys' places),
-        // then the arithmetic and the stores: a load behind a store waits for that store, since
-        // they may be the same memory for all the compiler knows, and one trip to memory after the
-        // other was most of this function's time
-        float2 f[ITS][4];
-        size_t kdst[ITS];
+        // what the rows' stores need from memory first (cosines and sines, the keys' places), then
+        // the arithmetic and the stores, four rows of the lane at a time (all eight are more
+        // registers than the eight-wave 256x256 kernel has): a load behind a store waits for that
+        // store, since they may be the same memory for all the compiler knows, and one trip to
+        // memory after the other was most of this function's time
+        constexpr int HB = ITS < 4 ? ITS : 4;
+        static_assert(ITS % HB == 0, "the lane's rows come in fours");
 #pragma unroll
-        for (int it = 0; it < ITS; ++it) {
+        for (int it0 = 0; it0 < ITS; it0 += HB) {
+        float2 f[HB][4];
+        size_t kdst[HB];
+#pragma unroll
+        for (int it = it0; it < it0 + HB; ++it) {
             const int m = m_base + it * RPI + lane / CPR;
             if (m >= M) continue;
             if (c < rp.rot) {
@@ -293,19 +298,19 @@ __device__ inline void rope_tiles(float* stage, const f32x16 (&t)[NT], const Rop
                 if (rp.interleaved) {
 #pragma unroll
                     for (int e = 0; e < 4; e += 2)
-                        if (c + e < rp.rot) f[it][e] = cs[(c + e) >> 1];
+                        if (c + e < rp.rot) f[it - it0][e] = cs[(c + e) >> 1];
                 } else {
 #pragma unroll
-                    for (int e = 0; e < 4; ++e) f[it][e] = cs[j0 + e];
+                    for (int e = 0; e < 4; ++e) f[it - it0][e] = cs[j0 + e];
                 }
             }
             if (sec == 1) {
                 const PageRef pr = page_of(rp.block_table, rp.table_stride, rp.req_of_token[m], rp.positions[m], rp.page_shift, rp.page_mask);
-                kdst[it] = (((size_t)pr.page * rp.Hk + hs) * rp.page_size + pr.off) * rp.D;
+                kdst[it - it0] = (((size_t)pr.page * rp.Hk + hs) * rp.page_size + pr.off) * rp.D;
             }
         }
 #pragma unroll
-        for (int it = 0; it < ITS; ++it) {
+        for (int it = it0; it < it0 + HB; ++it) {
             const int row = it * RPI + lane / CPR, m = m_base + row;
             if (m >= M) continue;
             const float4 x = *reinterpret_cast<const float4*>(stage + row * LD + ch * 4);
@@ -317,8 +322,8 @@ __device__ inline void rope_tiles(float* stage, const f32x16 (&t)[NT], const Rop
                     for (int e = 0; e < 4; e += 2)
                         if (c + e < rp.rot) {
                             const float x0 = o[e], x1 = o[e + 1];
-                            o[e] = x0 * f[it][e].x - x1 * f[it][e].y;
-                            o[e + 1] = x0 * f[it][e].y + x1 * f[it][e].x;
+                            o[e] = x0 * f[it - it0][e].x - x1 * f[it - it0][e].y;
+                            o[e + 1] = x0 * f[it - it0][e].y + x1 * f[it - it0][e].x;
                         }
                 } else {
                     const float4 y = *reinterpret_cast<const float4*>(stage + row * LD + (ch ^ 2) * 4);
@@ -326,14 +331,15 @@ __device__ inline void rope_tiles(float* stage, const f32x16 (&t)[NT], const Rop
 #pragma unroll
                     for (int e = 0; e < 4; ++e) {
                         const float x0 = hi ? pv[e] : o[e], x1 = hi ? o[e] : pv[e];
-                        o[e] = hi ? x0 * f[it][e].y + x1 * f[it][e].x : x0 * f[it][e].x - x1 * f[it][e].y;
+                        o[e] = hi ? x0 * f[it - it0][e].y + x1 * f[it - it0][e].x : x0 * f[it - it0][e].x - x1 * f[it - it0][e].y;
                     }
                     d0 = j0 + hi * half;
                 }
             }
             const uint2 w = make_uint2(pack_bf16x2(o[0], o[1]), pack_bf16x2(o[2], o[3]));
             if (sec == 0) *reinterpret_cast<uint2*>(rp.q_out + ((size_t)m * rp.H + hs) * rp.D + d0) = w;
-            else *reinterpret_cast<uint2*>(rp.k_cache + kdst[it] + d0) = w;
+            else *reinterpret_cast<uint2*>(rp.k_cache + kdst[it - it0] + d0) = w;
+        }
         }
     }
     if (col_base + SW > Q + KV && KV > 0) {
