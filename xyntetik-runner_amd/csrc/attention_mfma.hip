@@ -25,6 +25,8 @@
 // with 8 fixed slices for decoding).  Page sizes are powers of two from 16; a key that does
 // not exist (past the request's end, or in a page the window has given back) is copied from
 // a block of zeros, and the words of V^T past the end in the last tile are masked on use.
+#include <type_traits>
+
 #include "common.h"
 #include "async_copy.h"
 
@@ -156,12 +158,12 @@ _Pragma("unroll")                                                               
 // key/value head (wave w the rows row0 + 32 w ..) and a range of keys (a workgroup is one such
 // set, or two that halve the range between them: CtaShape::SETS below).  The K tile
 // [32 keys][HD] and the V^T tile [HD][32 keys] are copied once into LDS for all four waves,
-// by asynchronous copies, two tiles at a time into the places of the two tiles before the ones
-// being worked on (4 tiles in LDS; measured at head size 128, a prompt of 2,048 tokens: a barrier
-// and a round of address arithmetic every tile with three tiles ahead 73 us, every second tile
-// 71 us), instead of once per wave from
-// the caches; each wave then works as above with its fragments read from LDS.  A wave skips
-// the tiles that none of its rows can see, but takes part in every copy and barrier.
+// by asynchronous copies, two places of a ring of four at a time, into the two that were read
+// last (measured at head size 128, a prompt of 2,048 tokens: a barrier and a round of address
+// arithmetic every tile with three tiles ahead 73 us, every second tile 71 us), instead of
+// once per wave from the caches; each wave then works as above with its fragments read from
+// LDS.  A wave skips the tiles that none of its rows can see, but takes part in every copy and
+// barrier.
 //
 // LDS places are 16-byte chunks.  K: row r (key kt + r) has its chunk c at r * KSTR + c',
 // c' = c ^ (r mod CK) where CK is a power of two, else c with rows one chunk apart more
@@ -173,25 +175,25 @@ constexpr int KSTR = CK_POW2 ? CK : CK + 1;                 // chunks between ke
 constexpr int NKC = 32 * KSTR;                              // chunks of a K tile
 constexpr int NVC = DB * 32 * 4;                            // chunks of a V^T tile
 constexpr int CTA_ROWS = 128;
-constexpr int CTA_STAGES = 4;                               // tiles in LDS (copied two at a time)
+constexpr int CTA_STAGES = 4;                               // places in the ring (filled two at a time)
 
-// RB: 32-row blocks a wave takes.  1 is what is built: four waves a set, two waves a SIMD.  With 2 (two
-// waves a set with 64 rows each, one wave a SIMD, the output accumulators in the upper half of the
-// register file) every K and V^T fragment read from LDS serves two products, and it gives the same
-// bits; compiled as it stands it is slower (2,048 rows behind 6,144 keys: 447 us against 316), because
-// a lone wave has nothing to cover its own waits for LDS and at the barriers.
+// Four waves a set, each with one 32-row block, two waves a SIMD.  (Two blocks a wave, 64 rows, one
+// wave a SIMD and the output accumulators in the upper half of the register file, so that every K
+// and V^T fragment read from LDS serves two products, was built with a loop that finished a tile
+// before it began the next: the same bits, and slower, 2,048 rows behind 6,144 keys 447 us against
+// 316, because a lone wave has nothing to cover its own waits for LDS and at the barriers.)
 //
 // Two sets share an item where LDS has room for two rings: the first set takes the first half of the
 // item's tiles, the second set the rest, and their results are combined through LDS at the end.  A
 // compute unit then has two waves a SIMD from ONE item, and the items, which start longest first,
 // follow one another on it: a causal prompt's blocks see 1 to n keys, and with one set an item (two
 // items to a unit, a long one beside a short one) the long one ran on alone, one wave a SIMD, for most
-// of its time (2,048 tokens, 8 key/value heads: 70 us, now 63).
-template <int RB> struct CtaShape {
-    static constexpr int SET_WAVES = 4 / RB;
+// of its time (2,048 tokens, 8 key/value heads: 70 us against 63).
+struct CtaShape {
+    static constexpr int SET_WAVES = 4;
     static constexpr int SET_THREADS = 64 * SET_WAVES;
-    static constexpr int LOADS = (NKC + NVC + SET_THREADS - 1) / SET_THREADS;     // copies per lane and tile
-    static constexpr int STAGE = LOADS * SET_THREADS;                               // chunks of a tile's place in LDS
+    static constexpr int LOADS = (NKC + NVC + SET_THREADS - 1) / SET_THREADS;     // copies per lane and place
+    static constexpr int STAGE = LOADS * SET_THREADS;                               // chunks of a place in LDS
     static constexpr int SETS = 2 * CTA_STAGES * STAGE * 16 <= 144 * 1024 ? 2 : 1;
     static constexpr int THREADS = SET_THREADS * SETS;
     static constexpr int RING_BYTES = SETS * CTA_STAGES * STAGE * 16;
@@ -237,12 +239,205 @@ __device__ inline void cta_write_out(const AttnArgs& a, const f32x16 (&o)[DB], f
     }
 }
 
-template <int RB>
-__global__ __launch_bounds__(CtaShape<RB>::THREADS, 1) void k_attn_cta(AttnArgs a) {
-    using SH = CtaShape<RB>;
+// f(integral_constant<int, I>) for I = FROM .. TO-1, each call with its index a constant
+template <int FROM, int TO, class F>
+__device__ __forceinline__ void static_for(F&& f) {
+    if constexpr (FROM < TO) {
+        f(std::integral_constant<int, FROM>{});
+        static_for<FROM + 1, TO>(f);
+    }
+}
+
+__device__ __forceinline__ uint4 lds_read16(uint32_t byte_addr) {
+    typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+    const u32x4 x = *reinterpret_cast<const __attribute__((address_space(3))) u32x4*>(byte_addr);
+    return make_uint4(x[0], x[1], x[2], x[3]);
+}
+
+// What a wave's tile loop needs of its lane and of its rows, set up once an item.
+struct CtaWave {
+    uint32_t kbase;             // LDS byte address of this lane's K fragment of k-step 0 in place 0 of the set's ring
+    uint32_t vbase[2];          // and of its V^T fragments of channels 0-31, keys 0-15 and 16-31
+    bf16x8 qf[KD];
+    float c2;
+    int pos, lo, lg;
+    bool row_ok;
+    int kbeg, kend, nt, seq_len;
+    int pos_min, pos_max, lo_min, lo_max;       // the same in every lane, in scalar registers
+    __device__ __forceinline__ bool sees(int t) const {          // does any row of the wave see a key of tile t
+        const int kt = kbeg + t * 32;
+        return t >= 0 && t < nt && !(kt > pos_max || kt + 32 <= lo_min);
+    }
+    __device__ __forceinline__ bool whole(int t) const {         // does every row see all of it
+        const int kt = kbeg + t * 32;
+        return kt + 32 <= kend && kt + 31 <= pos_min && kt >= lo_max;
+    }
+};
+
+// The softmax of a whole tile cut into 18 pieces (the maximum over the lane's scores; the exchange, the
+// reference and the factor; the 16 weights) and dealt to the NS product slots of a step by their cost
+// in cycles of the vector unit (an exponential is a quarter-rate instruction).
+template <int NS> struct CtaPlan {
+    static constexpr int WA = 32, WB = 44, WP = 26, TOTAL = WA + WB + 16 * WP;
+    static constexpr int slot_of(int piece) {
+        const int before = piece == 0 ? 0 : piece == 1 ? WA : WA + WB + (piece - 2) * WP;
+        return before * NS / TOTAL;
+    }
+};
+
+// One step of a wave: the score product of tile v, the softmax of tile v-1 and the value product of
+// tile v-2, which do not depend on each other.  K of tile v and V^T of tile v-2 lie in place v mod 4 of
+// the ring.  In the middle of an item (cta_step_whole: tile v-1 seen whole by all the wave's rows, tiles
+// v and v-2 there) the three are written as NS slots, each one product, the fragment read of the
+// product AHEAD slots on and a piece of the softmax, and the compiler keeps the slots apart: the matrix
+// unit then works on one tile while the vector unit works on another, in one wave, where the loop that
+// finished a tile before it began the next had each unit wait for the other (counters: the matrix unit
+// busy 36% of the cycles, the vector unit 40%, both at once 10%).  At an item's edges (cta_step_edge)
+// the three run one after the other, each if its tile is there.  The two kinds of step are the bodies
+// of loops of their own, not two branches of one loop: where two branches that both write the output
+// accumulators meet, the compiler kept a second copy of those 64 registers and spilled.
+struct CtaFrags {
+    uint32_t kb, vb[2];
+    template <int STAGE> __device__ __forceinline__ CtaFrags(const CtaWave& w, int v, std::integral_constant<int, STAGE>) {
+        const uint32_t st = (uint32_t)(v & (CTA_STAGES - 1)) * (STAGE * 16);
+        kb = w.kbase + st;
+        vb[0] = w.vbase[0] + st + NKC * 16;
+        vb[1] = w.vbase[1] + st + NKC * 16;
+    }
+    // (k-step kd of a K row: 32 bytes on, or, where the chunks of a row are swapped about by the
+    // row's number, the address with kd's bits flipped: one register for all k-steps)
+    template <int K> __device__ __forceinline__ uint4 get() const {
+        if constexpr (K < KD) return lds_read16(CK_POW2 ? kb ^ (uint32_t)(K << 5) : kb + (uint32_t)(K << 5));
+        else return lds_read16(vb[(K - KD) / DB] + ((K - KD) % DB) * 128 * 16);
+    }
+};
+
+template <int STAGE>
+__device__ __forceinline__ void cta_step_whole(const CtaWave& w, int v, f32x16& s_new, const f32x16& s_cur,
+                                               uint4 (&pf_new)[2], const uint4 (&pf_old)[2], f32x16 (&o)[DB], float& m, float& l) {
+    constexpr int NS = KD + 2 * DB, AHEAD = 3 < NS ? 3 : NS;
+    const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    const CtaFrags f(w, v, std::integral_constant<int, STAGE>{});
+    const f32x16& s = s_cur;
+    uint4 fr[NS];
+    static_for<0, AHEAD>([&](auto kc) { fr[decltype(kc)::value] = f.template get<decltype(kc)::value>(); });
+    float mt = 0.f, mn = 0.f, corr = 1.f, rs = 0.f, pe = 0.f;
+    uint32_t pk[8];
+    __builtin_amdgcn_sched_barrier(0);
+    static_for<0, NS>([&](auto kc) {
+        constexpr int k = decltype(kc)::value;
+        if constexpr (k + AHEAD < NS) fr[k + AHEAD] = f.template get<k + AHEAD>();
+        if constexpr (k == 0) s_new = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16x8(fr[k]), w.qf[k], zero, 0, 0, 0);
+        else if constexpr (k < KD) s_new = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16x8(fr[k]), w.qf[k], s_new, 0, 0, 0);
+        else {
+            constexpr int j = (k - KD) / DB, d = (k - KD) % DB;
+            o[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16x8(fr[k]), as_bf16x8(pf_old[j]), o[d], 0, 0, 0);
+        }
+        static_for<0, 18>([&](auto pc) {
+            constexpr int piece = decltype(pc)::value;
+            if constexpr (CtaPlan<NS>::slot_of(piece) == k) {
+                if constexpr (piece == 0) {
+                    mt = fmaxf(s[0], s[15]);        // the compiler's own instruction reads s first
+                    mt = max3(mt, s[1], s[2]);
+#pragma unroll
+                    for (int e = 3; e < 15; e += 2) mt = max3(mt, s[e], s[e + 1]);
+                } else if constexpr (piece == 1) {
+                    mt = max_across_halves(mt);
+                    mn = mt * w.c2 > m + MAX_SLACK ? mt * w.c2 : m;
+                    corr = __builtin_amdgcn_exp2f(m - mn);
+                    asm volatile("" : "+v"(corr));
+                } else {
+                    // (each piece ends in a statement the compiler may not move: it would otherwise
+                    // put off all the weights, which nothing in this step reads, to behind the step's
+                    // last branch, and the vector unit's work would again follow the matrix unit's)
+                    constexpr int e = piece - 2;
+                    const float x = __builtin_amdgcn_exp2f(fmaf(s[e], w.c2, -mn));
+                    rs += x;
+                    asm volatile("" : "+v"(rs));
+                    if constexpr (e % 2 == 1) {
+                        pk[e / 2] = pack2(pe, x);
+                        asm volatile("" : "+v"(pk[e / 2]));
+                    } else pe = x;
+                }
+            }
+        });
+        __builtin_amdgcn_sched_barrier(0);
+    });
+    pf_new[0] = make_uint4(pk[0], pk[1], pk[2], pk[3]);
+    pf_new[1] = make_uint4(pk[4], pk[5], pk[6], pk[7]);
+    l = fmaf(l, corr, rs);
+    m = mn;
+    if (__any(corr != 1.0f)) {
+#pragma unroll
+        for (int d = 0; d < DB; ++d)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) o[d][e] *= corr;
+    }
+}
+
+template <int STAGE>
+__device__ __forceinline__ void cta_step_edge(const CtaWave& w, int v, f32x16& s_new, const f32x16& s_cur,
+                                              uint4 (&pf_new)[2], const uint4 (&pf_old)[2], f32x16 (&o)[DB], float& m, float& l) {
+    constexpr int NS = KD + 2 * DB;
+    const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    const CtaFrags f(w, v, std::integral_constant<int, STAGE>{});
+    const int lg = w.lg;
+    if (w.sees(v)) {
+        uint4 kf[KD];
+        static_for<0, KD>([&](auto kc) { kf[decltype(kc)::value] = f.template get<decltype(kc)::value>(); });
+        s_new = zero;
+#pragma unroll
+        for (int kd = 0; kd < KD; ++kd) s_new = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16x8(kf[kd]), w.qf[kd], s_new, 0, 0, 0);
+    }
+    __builtin_amdgcn_sched_barrier(0);           // (one after the other: their fragments do not wait in registers side by side)
+    if (w.sees(v - 2)) {
+        uint4 vf[2 * DB];
+        static_for<KD, NS>([&](auto kc) { vf[decltype(kc)::value - KD] = f.template get<decltype(kc)::value>(); });
+        const int kt = w.kbeg + (v - 2) * 32;
+        if (kt + 32 > w.seq_len) {             // the request's last tile: slots past its end hold old data
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                const int k8 = kt + 16 * j + 8 * lg;
+                uint32_t mk[4];
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                    mk[e] = (k8 + 2 * e < w.seq_len ? 0x0000FFFFu : 0u) | (k8 + 2 * e + 1 < w.seq_len ? 0xFFFF0000u : 0u);
+#pragma unroll
+                for (int d = 0; d < DB; ++d) {
+                    uint4& x = vf[j * DB + d];
+                    x.x &= mk[0]; x.y &= mk[1]; x.z &= mk[2]; x.w &= mk[3];
+                }
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int d = 0; d < DB; ++d)
+                o[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16x8(vf[j * DB + d]), as_bf16x8(pf_old[j]), o[d], 0, 0, 0);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    if (w.sees(v - 1)) {
+        const f32x16& s = s_cur;
+        const int kt = w.kbeg + (v - 1) * 32;
+        const bool row_ok = w.row_ok;
+        const int pos = w.pos, lo = w.lo, pos_min = w.pos_min, lo_max = w.lo_max;
+        const float c2 = w.c2;
+        float p[16];
+        float corr;
+        ATTN_SOFTMAX_STEP(kt, w.kend)
+        pf_new[0] = make_uint4(pack2(p[0], p[1]), pack2(p[2], p[3]), pack2(p[4], p[5]), pack2(p[6], p[7]));
+        pf_new[1] = make_uint4(pack2(p[8], p[9]), pack2(p[10], p[11]), pack2(p[12], p[13]), pack2(p[14], p[15]));
+    }
+}
+
+// The kernel.  A place of the ring holds K of tile v beside V^T of tile v-2, which is what step v reads.
+__global__ __launch_bounds__(CtaShape::THREADS, 1) void k_attn_cta(AttnArgs a) {
+    using SH = CtaShape;
     constexpr int SET_THREADS = SH::SET_THREADS, LOADS = SH::LOADS, STAGE = SH::STAGE, SETS = SH::SETS;
+    static_assert(CTA_STAGES == 4, "the steps below name the four places of the ring");
     extern __shared__ uint4 lds_all[];                      // [SETS][CTA_STAGES][STAGE]
-    const int tid = threadIdx.x % SET_THREADS, lane = tid & 63, wave = tid >> 6;       // within the set
+    const int tid = threadIdx.x % SET_THREADS, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);                          // within the set
     const int set = __builtin_amdgcn_readfirstlane((int)threadIdx.x / SET_THREADS);
     uint4* lds = lds_all + set * CTA_STAGES * STAGE;
     // Items come longest first, and workgroups start in the order of their numbers: an item's
@@ -255,70 +450,78 @@ __global__ __launch_bounds__(CtaShape<RB>::THREADS, 1) void k_attn_cta(AttnArgs 
     const int kvh = (int)wg - item_no * a.Hk;
     const int* it = a.cta_items + (size_t)item_no * ITEM_INTS;
     const int req = it[0];
-    const int q0 = it[5], q_len = it[6], start = it[7];
-    // the set's share of the item's keys; both sets go through the loop as often as the first
+    const int q_len = it[6], start = it[7];
     const int nt_item = (it[3] - it[2] + 31) >> 5;
     const int nt_first = SETS == 2 ? (nt_item + 1) >> 1 : nt_item;
     const int kbeg = it[2] + set * nt_first * 32;
     const int kend = (set == 0 && SETS == 2 && it[2] + nt_first * 32 < it[3]) ? it[2] + nt_first * 32 : it[3];
     const int G = a.H / a.Hk;
-    const int lr = lane & 31, lg = lane >> 5;
     const int seq_len = start + q_len;
     const int* bt = a.block_table + (size_t)req * a.table_stride;
+    const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) void*)lds;
 
-    // this lane's query rows, one in each of the wave's row blocks
-    int slot_[RB], t_[RB], h_[RB], pos_[RB], lo_[RB];
-    bool ok_[RB];
-    bf16x8 qf[RB][KD];
-#pragma unroll
-    for (int rb = 0; rb < RB; ++rb) {
-        const int blk = wave * RB + rb;
-        const int rho = it[1] + blk * ROWS + lr;
+    CtaWave w;
+    {
+        const int lr = lane & 31, lg = lane >> 5;
+        const int rho = it[1] + wave * ROWS + lr;
         const int tok = rho / G, hg = rho - tok * G;
-        slot_[rb] = it[4] < 0 ? -1 : it[4] + blk;
-        ok_[rb] = tok < q_len;
-        t_[rb] = q0 + tok;
-        h_[rb] = kvh * G + hg;
-        pos_[rb] = start + tok;
-        lo_[rb] = (a.window > 0 && pos_[rb] - a.window + 1 > 0) ? pos_[rb] - a.window + 1 : 0;
-        const bf16_t* qp = a.q + ((size_t)(ok_[rb] ? t_[rb] : q0) * a.H + h_[rb]) * HD + lg * 8;
+        const bool row_ok = tok < q_len;
+        w.row_ok = row_ok;
+        w.pos = start + tok;
+        w.lo = (a.window > 0 && w.pos - a.window + 1 > 0) ? w.pos - a.window + 1 : 0;
+        w.lg = lg;
+        const bf16_t* qp = a.q + ((size_t)(row_ok ? it[5] + tok : it[5]) * a.H + kvh * G + hg) * HD + lg * 8;
 #pragma unroll
-        for (int kd = 0; kd < KD; ++kd) qf[rb][kd] = as_bf16x8(keep_if(ok_[rb], ldg16(qp + kd * 16)));
+        for (int kd = 0; kd < KD; ++kd) w.qf[kd] = as_bf16x8(keep_if(row_ok, ldg16(qp + kd * 16)));
+        const int ra = lr >> 3, rg = (lr >> 2) & 1, rb4 = lr & 3;
+        const int key_off = 16 * (ra >> 1) + 8 * rg + 4 * (ra & 1) + rb4;
+        // (with swapped chunks a row is a power of two long and the ring begins at a multiple of it:
+        // the chunk's number within the row is the address's low bits, and k-step kd flips bits of it)
+        w.kbase = lds_base + (uint32_t)(key_off * KSTR + (CK_POW2 ? (lg ^ (key_off & (CK - 1))) : lg)) * 16u;
+#pragma unroll
+        for (int j = 0; j < 2; ++j) w.vbase[j] = lds_base + (uint32_t)(lr * 4 + ((2 * j + lg) ^ ((lr >> 2) & 3))) * 16u;
     }
-    const int ra = lr >> 3, rg = (lr >> 2) & 1, rb4 = lr & 3;
-    const int key_off = 16 * (ra >> 1) + 8 * rg + 4 * (ra & 1) + rb4;
 
-    // the pieces this lane copies for every tile
-    int src_off[LOADS], src_key[LOADS];
-    bool src_is_k[LOADS];
-#pragma unroll
-    for (int i = 0; i < LOADS; ++i) {
-        const int q = i * SET_THREADS + tid;
-        src_is_k[i] = q < NKC;
+    // The pieces this lane copies for every place of the ring.  Where every lane's piece exists in every
+    // whole tile and a copy instruction brings pieces of keys only or of values only (head sizes 64, 128
+    // and 256), a whole tile of an existing page is copied from two bases that all lanes share, each
+    // lane adding a fixed 32-bit offset.
+    constexpr bool CTA_FAST = CK_POW2 && NKC % SET_THREADS == 0 && NVC % SET_THREADS == 0 && HD % 32 == 0;
+    auto piece = [&](int i, int tid_, int& off, int& key, bool& is_k) {
+        const int q = i * SET_THREADS + tid_;
+        is_k = q < NKC;
         if (q < NKC) {
             const int r = q / KSTR, cs = q - r * KSTR;
             const int c = CK_POW2 ? (cs ^ (r & (CK - 1))) : cs;
-            src_off[i] = r * HD + c * 8;
-            src_key[i] = cs < CK ? r : (1 << 30);           // the spare chunk of a row stays zero
+            off = r * HD + c * 8;
+            key = cs < CK ? r : (1 << 30);                  // the spare chunk of a row stays zero
         } else {
-            const int v = q - NKC, d = v >> 2, c = (v & 3) ^ ((d >> 2) & 3);
-            src_off[i] = d * a.page_size + c * 8;
-            src_key[i] = (v < NVC && d < HD) ? c * 8 : (1 << 30);
+            const int vv = q - NKC, d = vv >> 2, c = (vv & 3) ^ ((d >> 2) & 3);
+            off = d * a.page_size + c * 8;
+            key = (vv < NVC && d < HD) ? c * 8 : (1 << 30);
+        }
+    };
+    constexpr int N_OFF = CTA_FAST ? LOADS : 1;
+    uint32_t fast_off[N_OFF];
+    if (CTA_FAST) {
+#pragma unroll
+        for (int n = 0; n < N_OFF; ++n) {
+            int off, key;
+            bool is_k;
+            piece(n, tid, off, key, is_k);
+            fast_off[n] = (uint32_t)off * 2u;
         }
     }
     const bf16_t* __restrict__ kc = a.kc;
     const bf16_t* __restrict__ vc = a.vc;
+    // a page's bytes (of all its key/value heads), and this head's part of page 0
+    const uint32_t page_bytes = (uint32_t)a.Hk * (uint32_t)a.page_size * (HD * 2);
+    const char* const kc_head = reinterpret_cast<const char*>(kc) + (size_t)kvh * a.page_size * (HD * 2);
+    const char* const vc_head = reinterpret_cast<const char*>(vc) + (size_t)kvh * a.page_size * (HD * 2);
     const bf16_t* zero_src = reinterpret_cast<const bf16_t*>(xr_zero_chunk);
-    const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) void*)lds;
-    // Where every lane's piece exists in every whole tile and a copy instruction brings pieces of
-    // keys only or of values only (head sizes 64, 128 and 256), a whole tile of an existing page
-    // is copied from two bases that all lanes share, each lane adding a fixed 32-bit offset.
-    constexpr bool CTA_FAST = CK_POW2 && NKC % SET_THREADS == 0 && NVC % SET_THREADS == 0 && HD % 32 == 0;
-    uint32_t fast_off[LOADS];
-#pragma unroll
-    for (int i = 0; i < LOADS; ++i) fast_off[i] = (uint32_t)src_off[i] * 2u;
 
-    // page numbers of the item's keys, one per lane, 64 pages at a time
+    // page numbers of the item's keys, one per lane, 64 pages at a time, from the page of the older of
+    // the two tiles a place holds (pages hold at least 32 positions: the newer is at most 2 pages on)
     int pages_base = kbeg >> a.page_shift;
     int my_page;
     {
@@ -328,52 +531,69 @@ __global__ __launch_bounds__(CtaShape<RB>::THREADS, 1) void k_attn_cta(AttnArgs 
         my_page = in ? my_page : -1;
     }
     const int nt = kend > kbeg ? (kend - kbeg + 31) >> 5 : 0;
-    // a tile lies within one page (pages hold at least 32 positions, tiles begin at multiples of 32)
-#define CTA_ISSUE(TI)                                                                                    \
+    // place u of the ring: K of tile u, V^T of tile u-2 (zeros for tiles that do not exist)
+    // Place u of the ring: K of tile u and V^T of tile u-2.  A tile that does not exist (before the first,
+    // past the set's last) is never read and is not copied.  Where every copy instruction brings pieces
+    // of keys only or of values only, a tile that exists is copied whole, the slots past the request's
+    // end with it: they lie in the tile's page, the scores of their keys are never looked at (the softmax
+    // chooses, it does not multiply) and their values are masked where they are used.  Else (a head size
+    // with spare chunks in LDS) each piece that exists is copied from where it lies and the others from
+    // a block of zeros.
+#define STEPS_ISSUE(UI)                                                                                  \
     {                                                                                                    \
-        const int ti_ = (TI);                                                                            \
-        const int kt_ = kbeg + ti_ * 32;                                                                 \
-        int pg_ = -1;                                                                                    \
-        if (ti_ < nt) {                                                                                  \
-            if ((kt_ >> a.page_shift) - pages_base >= 64) {                                              \
-                pages_base = kt_ >> a.page_shift;                                                        \
-                const int pi = pages_base + lane;                                                        \
-                const bool in = ((long)pi << a.page_shift) < seq_len;                                    \
-                my_page = bt[in ? pi : 0];                                                               \
-                my_page = in ? my_page : -1;                                                             \
-            }                                                                                            \
-            pg_ = __builtin_amdgcn_readlane(my_page, __builtin_amdgcn_readfirstlane((kt_ >> a.page_shift) - pages_base)); \
+        const int u_ = (UI);                                                                             \
+        const int ktk_ = kbeg + u_ * 32, ktv_ = ktk_ - 64;                                               \
+        const uint32_t dst_ = __builtin_amdgcn_readfirstlane(lds_base + (uint32_t)(((u_ & (CTA_STAGES - 1)) * STAGE + wave * 64) * 16)); \
+        const bool k_there_ = u_ < nt && ktk_ < seq_len, v_there_ = u_ >= 2 && u_ - 2 < nt && ktv_ < seq_len; \
+        if (k_there_ && (ktk_ >> a.page_shift) - pages_base >= 64) {                                     \
+            pages_base = (u_ >= 2 ? ktv_ : ktk_) >> a.page_shift;                                        \
+            const int pi = pages_base + lane;                                                            \
+            const bool in = ((long)pi << a.page_shift) < seq_len;                                        \
+            my_page = bt[in ? pi : 0];                                                                   \
+            my_page = in ? my_page : -1;                                                                 \
         }                                                                                                \
-        const size_t pb_ = (size_t)(pg_ < 0 ? 0 : pg_) * a.Hk + kvh;                                     \
-        const bf16_t* kb_ = kc + (pb_ * a.page_size + (kt_ & a.page_mask)) * HD;                         \
-        const bf16_t* vb_ = vc + pb_ * HD * a.page_size + (kt_ & a.page_mask);                           \
-        const uint32_t dst_ = __builtin_amdgcn_readfirstlane(lds_base + (uint32_t)(((ti_ % CTA_STAGES) * STAGE + wave * 64) * 16)); \
-        if (CTA_FAST && pg_ >= 0 && kt_ + 32 <= seq_len) {                                               \
-            _Pragma("unroll") for (int i = 0; i < LOADS; ++i)                                            \
-                lds_dma16_base(i * SET_THREADS < NKC ? kb_ : vb_, fast_off[i], dst_ + i * SET_THREADS * 16); \
+        if (CTA_FAST) {                                                                                  \
+            if (k_there_) {                                                                              \
+                const int pg_ = __builtin_amdgcn_readlane(my_page, (ktk_ >> a.page_shift) - pages_base); \
+                const char* kb_ = kc_head + (size_t)(uint32_t)pg_ * page_bytes + (uint32_t)(ktk_ & a.page_mask) * (HD * 2); \
+                _Pragma("unroll") for (int i = 0; i < LOADS; ++i)                                        \
+                    if (i * SET_THREADS < NKC) lds_dma16_base(kb_, fast_off[i % N_OFF], dst_ + i * SET_THREADS * 16); \
+            }                                                                                            \
+            if (v_there_) {                                                                              \
+                const int pg_ = __builtin_amdgcn_readlane(my_page, (ktv_ >> a.page_shift) - pages_base); \
+                const char* vb_ = vc_head + (size_t)(uint32_t)pg_ * page_bytes + (uint32_t)(ktv_ & a.page_mask) * 2; \
+                _Pragma("unroll") for (int i = 0; i < LOADS; ++i)                                        \
+                    if (i * SET_THREADS >= NKC) lds_dma16_base(vb_, fast_off[i % N_OFF], dst_ + i * SET_THREADS * 16); \
+            }                                                                                            \
         } else {                                                                                         \
+            const int pgk_ = k_there_ ? __builtin_amdgcn_readlane(my_page, __builtin_amdgcn_readfirstlane((ktk_ >> a.page_shift) - pages_base)) : -1; \
+            const int pgv_ = v_there_ ? __builtin_amdgcn_readlane(my_page, __builtin_amdgcn_readfirstlane((ktv_ >> a.page_shift) - pages_base)) : -1; \
+            const size_t pbk_ = (size_t)(pgk_ < 0 ? 0 : pgk_) * a.Hk + kvh;                              \
+            const size_t pbv_ = (size_t)(pgv_ < 0 ? 0 : pgv_) * a.Hk + kvh;                              \
+            const bf16_t* kb_ = kc + (pbk_ * a.page_size + (ktk_ & a.page_mask)) * HD;                   \
+            const bf16_t* vb_ = vc + pbv_ * HD * a.page_size + (ktv_ & a.page_mask);                     \
             _Pragma("unroll") for (int i = 0; i < LOADS; ++i) {                                          \
-                const bool okc_ = pg_ >= 0 && kt_ + src_key[i] < seq_len;                                \
-                const bf16_t* p_ = okc_ ? (src_is_k[i] ? kb_ : vb_) + src_off[i] : zero_src;             \
+                int tid_ = tid, off_, key_;                                                              \
+                bool isk_;                                                                               \
+                asm volatile("" : "+v"(tid_));            /* (worked out here, not kept in registers throughout) */ \
+                piece(i, tid_, off_, key_, isk_);                                                        \
+                const bool okc_ = isk_ ? (pgk_ >= 0 && ktk_ + key_ < seq_len) : (pgv_ >= 0 && ktv_ + key_ < seq_len); \
+                const bf16_t* p_ = okc_ ? (isk_ ? kb_ : vb_) + off_ : zero_src;                          \
                 lds_dma16(p_, dst_ + i * SET_THREADS * 16);                                              \
             }                                                                                            \
         }                                                                                                \
     }
 
-    f32x16 o_[RB][DB];
-    float m_[RB], l_[RB];      // m in units of log2
-    int pmin_[RB], lmax_[RB], pmax_[RB], lmin_[RB];
+    f32x16 o[DB];
 #pragma unroll
-    for (int rb = 0; rb < RB; ++rb) {
+    for (int d = 0; d < DB; ++d)
 #pragma unroll
-        for (int d = 0; d < DB; ++d)
-#pragma unroll
-            for (int e = 0; e < 16; ++e) o_[rb][d][e] = 0.f;
-        m_[rb] = -INFINITY;
-        l_[rb] = 0.f;
-        // what the rows of this block can see: keys [lo_min, pos_max]; keys in [lo_max, pos_min] by all
-        int pos_min = ok_[rb] ? pos_[rb] : 0x7fffffff, lo_max = ok_[rb] ? lo_[rb] : 0;
-        int pos_max = ok_[rb] ? pos_[rb] : -1, lo_min = ok_[rb] ? lo_[rb] : 0x7fffffff;
+        for (int e = 0; e < 16; ++e) o[d][e] = 0.f;
+    float m = -INFINITY, l = 0.f;           // m in units of log2
+    {
+        // what the wave's rows can see: keys [lo_min, pos_max]; keys in [lo_max, pos_min] by all
+        int pos_min = w.row_ok ? w.pos : 0x7fffffff, lo_max = w.row_ok ? w.lo : 0;
+        int pos_max = w.row_ok ? w.pos : -1, lo_min = w.row_ok ? w.lo : 0x7fffffff;
 #pragma unroll
         for (int x = 32; x > 0; x >>= 1) {
             pos_min = min(pos_min, __shfl_xor(pos_min, x, 64));
@@ -381,145 +601,118 @@ __global__ __launch_bounds__(CtaShape<RB>::THREADS, 1) void k_attn_cta(AttnArgs 
             pos_max = max(pos_max, __shfl_xor(pos_max, x, 64));
             lo_min = min(lo_min, __shfl_xor(lo_min, x, 64));
         }
-        pmin_[rb] = pos_min; lmax_[rb] = lo_max; pmax_[rb] = pos_max; lmin_[rb] = lo_min;
+        w.pos_min = __builtin_amdgcn_readfirstlane(pos_min); w.lo_max = __builtin_amdgcn_readfirstlane(lo_max);
+        w.pos_max = __builtin_amdgcn_readfirstlane(pos_max); w.lo_min = __builtin_amdgcn_readfirstlane(lo_min);
     }
-    const float c2 = a.scale * 1.44269504088896340736f;
+    w.c2 = a.scale * 1.44269504088896340736f;
+    w.kbeg = kbeg; w.kend = kend; w.nt = nt; w.seq_len = seq_len;
 
-    // The tiles are copied and waited for two at a time: the workgroup meets at a barrier, and the
-    // copies' addresses are worked out, every second tile (two tiles take a wave over 2 us, more
-    // than a copy from L2 needs to land).
-    static_assert(CTA_STAGES % 2 == 0 && LOADS * 2 < 64, "the tiles in LDS come in pairs");
-#pragma unroll
-    for (int st = 0; st < CTA_STAGES - 2; ++st) CTA_ISSUE(st)
-    for (int ti = 0; ti < nt_first; ++ti) {
-        if ((ti & 1) == 0) {
-            // tiles ti and ti+1 have landed when at most the CTA_STAGES-4 younger ones are on their way
-            wait_vmcnt<LOADS * (CTA_STAGES - 4)>();
-            __builtin_amdgcn_s_barrier();                // for every wave; and tiles ti-2, ti-1 are no longer read
-            CTA_ISSUE(ti + CTA_STAGES - 2)               // into their places (zeros past the end)
-            CTA_ISSUE(ti + CTA_STAGES - 1)
-        }
-        const int kt = kbeg + ti * 32;
-        bool any = false;
-#pragma unroll
-        for (int rb = 0; rb < RB; ++rb) any = any || !(kt > pmax_[rb] || kt + 32 <= lmin_[rb]);
-        if (ti >= nt || !any) continue;                  // nothing here for this wave's rows
-        const uint4* Ks = lds + (ti % CTA_STAGES) * STAGE;
-        const uint4* Vs = Ks + NKC;
-        uint4 kf[KD], vf[2][DB];
-#pragma unroll
-        for (int kd = 0; kd < KD; ++kd) {
-            const int c = 2 * kd + lg;
-            kf[kd] = Ks[key_off * KSTR + (CK_POW2 ? (c ^ (key_off & (CK - 1))) : c)];
-        }
-#pragma unroll
-        for (int j = 0; j < 2; ++j)
-#pragma unroll
-            for (int d = 0; d < DB; ++d) vf[j][d] = Vs[(d * 32 + lr) * 4 + ((2 * j + lg) ^ ((lr >> 2) & 3))];
-        if (kt + 32 > seq_len) {               // the request's last tile: slots past its end hold old data
-#pragma unroll
-            for (int j = 0; j < 2; ++j) {
-                const int k8 = kt + 16 * j + 8 * lg;
-                uint32_t mk[4];
-#pragma unroll
-                for (int e = 0; e < 4; ++e)
-                    mk[e] = (k8 + 2 * e < seq_len ? 0x0000FFFFu : 0u) | (k8 + 2 * e + 1 < seq_len ? 0xFFFF0000u : 0u);
-#pragma unroll
-                for (int d = 0; d < DB; ++d) {
-                    vf[j][d].x &= mk[0]; vf[j][d].y &= mk[1]; vf[j][d].z &= mk[2]; vf[j][d].w &= mk[3];
-                }
-            }
-        }
-        f32x16 s_[RB];
-#pragma unroll
-        for (int rb = 0; rb < RB; ++rb)
-#pragma unroll
-            for (int e = 0; e < 16; ++e) s_[rb][e] = 0.f;
-#pragma unroll
-        for (int kd = 0; kd < KD; ++kd)
-#pragma unroll
-            for (int rb = 0; rb < RB; ++rb)
-                s_[rb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16x8(kf[kd]), qf[rb][kd], s_[rb], 0, 0, 0);
-#pragma unroll
-        for (int rb = 0; rb < RB; ++rb) {
-            f32x16& s = s_[rb];
-            f32x16 (&o)[DB] = o_[rb];
-            float& m = m_[rb];
-            float& l = l_[rb];
-            const bool row_ok = ok_[rb];
-            const int pos = pos_[rb], lo = lo_[rb], pos_min = pmin_[rb], lo_max = lmax_[rb];
-            float p[16];
-            float corr;
-            ATTN_SOFTMAX_STEP(kt, kend)
-#pragma unroll
-            for (int j = 0; j < 2; ++j) {
-                uint4 pk = make_uint4(pack2(p[8 * j + 0], p[8 * j + 1]), pack2(p[8 * j + 2], p[8 * j + 3]),
-                                      pack2(p[8 * j + 4], p[8 * j + 5]), pack2(p[8 * j + 6], p[8 * j + 7]));
-                const bf16x8 pf = as_bf16x8(pk);
-#pragma unroll
-                for (int d = 0; d < DB; ++d)
-                    o[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16x8(vf[j][d]), pf, o[d], 0, 0, 0);
-            }
-        }
+    // Step v of a wave touches place v of the ring only, so the places are filled and waited for two
+    // at a time as before: at the barrier before steps v and v+1 every wave has done with places v-2
+    // and v-1, which then take what steps v+2 and v+3 will read.  A set's tiles take two steps more than
+    // it has tiles; both sets go through the loops as often as the first, every wave through the same
+    // number of steps, whichever loop it does them in.
+    static_assert(LOADS * 2 < 64, "two places' copies are counted at once");
+    const int n_steps = nt_first + 2;
+    // steps [v1, v2), in pairs: the wave's whole steps.  The steps with a tile v-1 that all rows see
+    // whole and tiles v, v-2 that exist are consecutive (each condition holds for a range of v), so
+    // both ends are tried and nothing between them.
+    auto whole_step = [&](int v) { return w.sees(v) && w.sees(v - 1) && w.sees(v - 2) && w.whole(v - 1); };
+    int v1, v2;
+    {
+        // the first and the last tile that all rows see whole, from the same comparisons as CtaWave::whole
+        const int up = min(min(kend - kbeg, w.pos_min + 1 - kbeg), nt * 32);
+        const int t_last = up >= 32 ? (up >> 5) - 1 : -1;
+        const int t_first = w.lo_max > kbeg ? (w.lo_max - kbeg + 31) >> 5 : 0;
+        v1 = (max(t_first + 1, 2) + 1) & ~1;
+        v2 = min(t_last + 2, n_steps) & ~1;
+        while (v1 < v2 && !(whole_step(v1) && whole_step(v1 + 1))) v1 += 2;
+        while (v1 < v2 && !(whole_step(v2 - 2) && whole_step(v2 - 1))) v2 -= 2;
+        if (v1 >= v2) v1 = v2 = 0;
     }
-#undef CTA_ISSUE
+    f32x16 s_even, s_odd;                    // the scores of the tiles with even and with odd numbers
+    uint4 pf_even[2] = {}, pf_odd[2] = {};   // and their weights, rounded, as the value product takes them
+    STEPS_ISSUE(0)
+    STEPS_ISSUE(1)
+#define STEPS_SYNC(V)                                                                                    \
+        wait_vmcnt<0>();                                                                                 \
+        __builtin_amdgcn_s_barrier();                                                                    \
+        STEPS_ISSUE((V) + 2)                                                                             \
+        STEPS_ISSUE((V) + 3)
+    int v = 0;
+    for (; v < v1; v += 2) {
+        STEPS_SYNC(v)
+        cta_step_edge<STAGE>(w, v, s_even, s_odd, pf_odd, pf_even, o, m, l);
+        cta_step_edge<STAGE>(w, v + 1, s_odd, s_even, pf_even, pf_odd, o, m, l);
+    }
+    for (; v < v2; v += 2) {
+        STEPS_SYNC(v)
+        cta_step_whole<STAGE>(w, v, s_even, s_odd, pf_odd, pf_even, o, m, l);
+        cta_step_whole<STAGE>(w, v + 1, s_odd, s_even, pf_even, pf_odd, o, m, l);
+    }
+    for (; v < n_steps; v += 2) {
+        STEPS_SYNC(v)
+        cta_step_edge<STAGE>(w, v, s_even, s_odd, pf_odd, pf_even, o, m, l);
+        cta_step_edge<STAGE>(w, v + 1, s_odd, s_even, pf_even, pf_odd, o, m, l);
+    }
+#undef STEPS_SYNC
+#undef STEPS_ISSUE
     wait_vmcnt<0>();                                     // the trailing copies of zeros
-#pragma unroll
-    for (int rb = 0; rb < RB; ++rb) l_[rb] += __shfl_xor(l_[rb], 32, 64);      // the row's sum from its two lanes
+    l += __shfl_xor(l, 32, 64);                          // the row's sum from its two lanes
 
+    // (the row's place in the output is worked out again here, from a lane number the compiler cannot
+    // trace back, rather than kept in registers through the loop)
+    int lane_after = lane;
+    asm volatile("" : "+v"(lane_after));
+    const int lr = lane_after & 31, lg = lane_after >> 5;
+    const int rho = it[1] + wave * ROWS + lr;
+    const int tok = rho / G, hg = rho - tok * G;
+    const int slot = it[4] < 0 ? -1 : it[4] + wave;
+    const bool row_ok = tok < q_len;
+    const int t = it[5] + tok, h = kvh * G + hg;
     if (SETS == 2) {
         // the second set hands its rows' maxima, sums and unnormalised outputs to the first
         __syncthreads();                                 // the rings are free
         float* xo = reinterpret_cast<float*>(lds_all);   // [4 row blocks][ROWS][HD + 4]
         float* xml = xo + 4 * ROWS * (HD + 4);           // [4 row blocks][ROWS][2]
+        float* mine = xo + (wave * ROWS + lr) * (HD + 4);
         if (set == 1) {
-#pragma unroll
-            for (int rb = 0; rb < RB; ++rb) {
-                float* mine = xo + ((wave * RB + rb) * ROWS + lr) * (HD + 4);
-#pragma unroll
-                for (int d = 0; d < DB; ++d)
-#pragma unroll
-                    for (int e4 = 0; e4 < 4; ++e4) {
-                        const int dd = d * 32 + e4 * 8 + lg * 4;
-                        if (dd < HD)
-                            *reinterpret_cast<float4*>(mine + dd) = make_float4(o_[rb][d][e4 * 4 + 0], o_[rb][d][e4 * 4 + 1],
-                                                                                o_[rb][d][e4 * 4 + 2], o_[rb][d][e4 * 4 + 3]);
-                    }
-                if (lg == 0) {
-                    xml[((wave * RB + rb) * ROWS + lr) * 2] = m_[rb];
-                    xml[((wave * RB + rb) * ROWS + lr) * 2 + 1] = l_[rb];
-                }
-            }
-        }
-        __syncthreads();
-        if (set == 1) return;
-#pragma unroll
-        for (int rb = 0; rb < RB; ++rb) {
-            const float* mine = xo + ((wave * RB + rb) * ROWS + lr) * (HD + 4);
-            const float m1 = xml[((wave * RB + rb) * ROWS + lr) * 2], l1 = xml[((wave * RB + rb) * ROWS + lr) * 2 + 1];
-            const float mn = fmaxf(m_[rb], m1);
-            const float f0 = m_[rb] == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(m_[rb] - mn);
-            const float f1 = m1 == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(m1 - mn);
-            l_[rb] = l_[rb] * f0 + l1 * f1;
-            m_[rb] = mn;
 #pragma unroll
             for (int d = 0; d < DB; ++d)
 #pragma unroll
                 for (int e4 = 0; e4 < 4; ++e4) {
                     const int dd = d * 32 + e4 * 8 + lg * 4;
-                    if (dd < HD) {
-                        const float4 x = *reinterpret_cast<const float4*>(mine + dd);
-                        o_[rb][d][e4 * 4 + 0] = o_[rb][d][e4 * 4 + 0] * f0 + x.x * f1;
-                        o_[rb][d][e4 * 4 + 1] = o_[rb][d][e4 * 4 + 1] * f0 + x.y * f1;
-                        o_[rb][d][e4 * 4 + 2] = o_[rb][d][e4 * 4 + 2] * f0 + x.z * f1;
-                        o_[rb][d][e4 * 4 + 3] = o_[rb][d][e4 * 4 + 3] * f0 + x.w * f1;
-                    }
+                    if (dd < HD)
+                        *reinterpret_cast<float4*>(mine + dd) = make_float4(o[d][e4 * 4 + 0], o[d][e4 * 4 + 1], o[d][e4 * 4 + 2], o[d][e4 * 4 + 3]);
                 }
+            if (lg == 0) {
+                xml[(wave * ROWS + lr) * 2] = m;
+                xml[(wave * ROWS + lr) * 2 + 1] = l;
+            }
         }
-    }
+        __syncthreads();
+        if (set == 1) return;
+        const float m1 = xml[(wave * ROWS + lr) * 2], l1 = xml[(wave * ROWS + lr) * 2 + 1];
+        const float mn = fmaxf(m, m1);
+        const float f0 = m == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(m - mn);
+        const float f1 = m1 == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(m1 - mn);
+        l = l * f0 + l1 * f1;
+        m = mn;
 #pragma unroll
-    for (int rb = 0; rb < RB; ++rb)
-        cta_write_out(a, o_[rb], m_[rb], l_[rb], ok_[rb], t_[rb], h_[rb], kvh, lr, lg, slot_[rb]);
+        for (int d = 0; d < DB; ++d)
+#pragma unroll
+            for (int e4 = 0; e4 < 4; ++e4) {
+                const int dd = d * 32 + e4 * 8 + lg * 4;
+                if (dd < HD) {
+                    const float4 x = *reinterpret_cast<const float4*>(mine + dd);
+                    o[d][e4 * 4 + 0] = o[d][e4 * 4 + 0] * f0 + x.x * f1;
+                    o[d][e4 * 4 + 1] = o[d][e4 * 4 + 1] * f0 + x.y * f1;
+                    o[d][e4 * 4 + 2] = o[d][e4 * 4 + 2] * f0 + x.z * f1;
+                    o[d][e4 * 4 + 3] = o[d][e4 * 4 + 3] * f0 + x.w * f1;
+                }
+            }
+    }
+    cta_write_out(a, o, m, l, row_ok, t, h, kvh, lr, lg, slot);
 }
 
 // ------------------------------------------------------------------------------ streaming kernel
@@ -867,15 +1060,15 @@ extern "C" int xr_attention_mfma(void* out, const void* q, const void* k_cache, 
     a.part_o = part_o; a.part_ml = part_ml; a.n_items = n_items; a.H = H; a.Hk = Hk;
     a.page_shift = shift; a.page_mask = page_size - 1; a.page_size = page_size; a.scale = scale; a.window = window;
     if (n_cta_items > 0) {
-        constexpr int smem = CtaShape<1>::LDS_BYTES;
+        constexpr int smem = CtaShape::LDS_BYTES;
         static bool attr_set = false;
         if (!attr_set) {
-            hipError_t e = hipFuncSetAttribute((const void*)k_attn_cta<1>, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+            hipError_t e = hipFuncSetAttribute((const void*)k_attn_cta, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
             if (e != hipSuccess) (void)hipGetLastError();     // or the next launch's check would report this refusal
             XR_REQUIRE(e == hipSuccess, "attention: %d bytes of LDS refused: %s", smem, hipGetErrorString(e));
             attr_set = true;
         }
-        k_attn_cta<1><<<dim3((unsigned)n_cta_items * (unsigned)Hk), CtaShape<1>::THREADS, smem, stream>>>(a);
+        k_attn_cta<<<dim3((unsigned)n_cta_items * (unsigned)Hk), CtaShape::THREADS, smem, stream>>>(a);
         XR_CHECK_LAUNCH("attention_cta");
     }
     if (n_items > 0) {

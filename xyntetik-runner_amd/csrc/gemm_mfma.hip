@@ -1291,6 +1291,8 @@ static int launch_tile_variant(int variant, const GemmArgs& g, hipStream_t strea
         xr_set_error("gemm: the four-wave kernel does not take K %d in %d ranges, lda %d, or a rotation", g.K, g.splits, g.lda);
         return XR_BAD_ARG;
     }
+    // (the 256x192 tile with four waves and the rotation, 12 tiles a wave: 27.0 ms for the prompt step
+    // of 2,048 rows against 26.8 with eight)
     if (variant == 26) return launch_tile_async<256, 192, 4, 2, 2>(g, stream);
     xr_set_error("gemm: unknown variant %d", variant);
     return XR_BAD_ARG;
