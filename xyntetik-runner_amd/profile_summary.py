@@ -9,7 +9,16 @@ embedding begins a prompt step).  ``--grid N`` takes only spans whose marker dis
 at least N threads (the embedding of a 2,048-row step, 256 threads a row, among those of decode
 steps); ``--index``
 counts spans from the end (-1: the last).  The table is markdown, as the files under ``profiles/``
-hold it.  The reference prints per-op timings of a decode step from inside its engine
+hold it.
+
+    rocprofv3 --pmc SQ_CYCLES SQ_INSTS_MFMA SQ_VALU_MFMA_BUSY_CYCLES --kernel-trace --output-format csv -d OUT -- python3 bench.py ...
+    python -m xyntetik_runner_amd.profile_summary OUT --counters --kernel k_attn_cta --kernel k_gemm_tile
+
+``--counters`` reads the counters of such a run instead: for every kernel whose name holds one of the
+``--kernel`` strings (all kernels without), the dispatches (``--grid N``: those of at least N
+threads), their mean time and the mean of every counter per dispatch.
+
+The reference prints per-op timings of a decode step from inside its engine
 (src/main.c:1435-1515 for its own bench); here the profiler's trace is the source.
 """
 from __future__ import annotations
@@ -72,13 +81,49 @@ def summarize(rows, first: int, last: int) -> str:
     return "\n".join(lines)
 
 
+def read_counters(folder: str, min_grid: int = 0) -> Dict[str, Dict[str, List[float]]]:
+    """kernel name -> counter name -> one value per dispatch (and "us": the dispatches' times)."""
+    files = sorted(glob.glob(os.path.join(folder, "**", "*counter_collection.csv"), recursive=True), key=os.path.getmtime)
+    if not files:
+        raise SystemExit(f"no *counter_collection.csv under {folder}")
+    out: Dict[str, Dict[str, List[float]]] = {}
+    seen = set()
+    with open(files[-1], newline="") as f:
+        for r in csv.DictReader(f):
+            if int(r.get("Grid_Size") or 0) < min_grid:
+                continue
+            k = out.setdefault(short_name(r["Kernel_Name"]), {})
+            k.setdefault(r["Counter_Name"], []).append(float(r["Counter_Value"]))
+            if r["Dispatch_Id"] not in seen:             # a dispatch has a row per counter, with the same times
+                seen.add(r["Dispatch_Id"])
+                k.setdefault("us", []).append((int(r["End_Timestamp"]) - int(r["Start_Timestamp"])) / 1e3)
+    return out
+
+
+def counter_table(counters: Dict[str, Dict[str, List[float]]], kernels: List[str]) -> str:
+    names = [n for n in counters if not kernels or any(k in n for k in kernels)]
+    cols = sorted({c for n in names for c in counters[n] if c != "us"})
+    lines = ["| kernel | dispatches | mean us | " + " | ".join(cols) + " |", "|--------|-----------:|--------:|" + "|".join("-" * (len(c) + 1) + ":" for c in cols) + "|"]
+    for n in sorted(names, key=lambda n: -sum(counters[n].get("us", [0]))):
+        c = counters[n]
+        us = c.get("us", [0.0])
+        cells = [f"{sum(c[x]) / len(c[x]):,.0f}" if x in c else "" for x in cols]
+        lines.append(f"| `{n}` | {len(us)} | {sum(us) / len(us):,.1f} | " + " | ".join(cells) + " |")
+    return "\n".join(lines)
+
+
 def main(argv=None) -> int:
     ap = argparse.ArgumentParser(prog="profile_summary", description=__doc__.split("\n\n")[0])
     ap.add_argument("folder", help="the -d folder of the rocprofv3 run")
     ap.add_argument("--marker", default="k_sample", help="part of the name of the kernel that separates steps")
     ap.add_argument("--grid", type=int, default=0, help="only spans whose marker dispatch has at least this many threads")
     ap.add_argument("--index", type=int, default=-1, help="which span, counted from the end (-1: the last)")
+    ap.add_argument("--counters", action="store_true", help="the means of a --pmc run's counters per kernel instead of a step's times")
+    ap.add_argument("--kernel", action="append", default=[], help="with --counters: only kernels whose name holds this (may be given again)")
     args = ap.parse_args(argv)
+    if args.counters:
+        print(counter_table(read_counters(args.folder, args.grid), args.kernel))
+        return 0
     rows = read_trace(args.folder)
     found = spans(rows, args.marker, args.grid)
     if not found:
