@@ -24,7 +24,9 @@
 // results that k_attn_merge combines (src/kernels.cu:2171-2270 does this
 // with 8 fixed slices for decoding).  Page sizes are powers of two from 16; a key that does
 // not exist (past the request's end, or in a page the window has given back) is copied from
-// a block of zeros, and the words of V^T past the end in the last tile are masked on use.
+// a block of zeros, and the words of V^T past the end in the last tile are masked on use
+// (k_attn_cta copies a tile that exists whole where the head size allows, never reads a tile
+// it did not copy, and chooses among the scores instead of multiplying them: see there).
 #include <type_traits>
 
 #include "common.h"
@@ -532,6 +534,9 @@ __global__ __launch_bounds__(CtaShape::THREADS, 1) void k_attn_cta(AttnArgs a) {
     }
     const int nt = kend > kbeg ? (kend - kbeg + 31) >> 5 : 0;
     // place u of the ring: K of tile u, V^T of tile u-2 (zeros for tiles that do not exist)
+    // (A page number below 0, which the table holds for pages a window has given back, is read as
+    // the null page: the host lists no keys from such pages, and a list that did would get wrong
+    // values from here, not a fault.)
     // Place u of the ring: K of tile u and V^T of tile u-2.  A tile that does not exist (before the first,
     // past the set's last) is never read and is not copied.  Where every copy instruction brings pieces
     // of keys only or of values only, a tile that exists is copied whole, the slots past the request's
@@ -555,13 +560,13 @@ __global__ __launch_bounds__(CtaShape::THREADS, 1) void k_attn_cta(AttnArgs a) {
         if (CTA_FAST) {                                                                                  \
             if (k_there_) {                                                                              \
                 const int pg_ = __builtin_amdgcn_readlane(my_page, (ktk_ >> a.page_shift) - pages_base); \
-                const char* kb_ = kc_head + (size_t)(uint32_t)pg_ * page_bytes + (uint32_t)(ktk_ & a.page_mask) * (HD * 2); \
+                const char* kb_ = kc_head + (size_t)(uint32_t)max(pg_, 0) * page_bytes + (uint32_t)(ktk_ & a.page_mask) * (HD * 2); \
                 _Pragma("unroll") for (int i = 0; i < LOADS; ++i)                                        \
                     if (i * SET_THREADS < NKC) lds_dma16_base(kb_, fast_off[i % N_OFF], dst_ + i * SET_THREADS * 16); \
             }                                                                                            \
             if (v_there_) {                                                                              \
                 const int pg_ = __builtin_amdgcn_readlane(my_page, (ktv_ >> a.page_shift) - pages_base); \
-                const char* vb_ = vc_head + (size_t)(uint32_t)pg_ * page_bytes + (uint32_t)(ktv_ & a.page_mask) * 2; \
+                const char* vb_ = vc_head + (size_t)(uint32_t)max(pg_, 0) * page_bytes + (uint32_t)(ktv_ & a.page_mask) * 2; \
                 _Pragma("unroll") for (int i = 0; i < LOADS; ++i)                                        \
                     if (i * SET_THREADS >= NKC) lds_dma16_base(vb_, fast_off[i % N_OFF], dst_ + i * SET_THREADS * 16); \
             }                                                                                            \
