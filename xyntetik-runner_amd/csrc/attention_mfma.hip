@@ -626,7 +626,7 @@ __global__ __launch_bounds__(CtaShape::THREADS, 1) void k_attn_cta(AttnArgs a) {
     int v1, v2;
     {
         // the first and the last tile that all rows see whole, from the same comparisons as CtaWave::whole
-        const int up = min(min(kend - kbeg, w.pos_min + 1 - kbeg), nt * 32);
+        const int up = min(min(kend - kbeg, min(w.pos_min, kend) + 1 - kbeg), nt * 32);      // (a wave without rows has pos_min at the largest int)
         const int t_last = up >= 32 ? (up >> 5) - 1 : -1;
         const int t_first = w.lo_max > kbeg ? (w.lo_max - kbeg + 31) >> 5 : 0;
         v1 = (max(t_first + 1, 2) + 1) & ~1;
