@@ -929,6 +929,41 @@ def test_attention_two_wave_sets_share_an_item(ops, start, far):
     assert sees and rel(got[sees], v.bfloat16().float()[far].expand(len(sees), H, D)) < 1e-2
 
 
+@pytest.mark.parametrize("H,Hk,D,ps,window,start", [(1, 1, 128, 64, None, 1111), (4, 1, 128, 32, None, 1111), (2, 2, 64, 64, None, 600),
+                                                      (1, 1, 128, 64, 700, 1111), (2, 1, 256, 64, None, 500)])
+def test_attention_every_token_has_a_far_key_of_its_own(ops, H, Hk, D, ps, window, start):
+    """A step of the workgroup kernel works on three tiles at once (the scores of one, the softmax of
+    the one before, the value product of the one before that) out of four places of a ring in LDS.  Here
+    every token of a 160-token portion has one key that stands out, and these keys are spread over all the
+    tiles the token may see (with a window: over the tiles inside it): whichever tile, place of the ring,
+    step of the loop or set of waves a key falls to, its token must come back with that key's value."""
+    n_new = 160
+    n = start + n_new
+    g = torch.Generator().manual_seed(D + ps + start)
+    u = (torch.randint(0, 2, (n_new, D), generator=g).float() * 2 - 1) * 1.5      # q . k = 2.25 D for a token's own key
+    span = window if window else start
+    far = [start + t - (t * 37) % span if window else (t * 37) % start for t in range(n_new)]
+    assert len(set(p // 32 for p in far)) >= min(20, span // 32)      # many different tiles
+    k = torch.randn(n, Hk, D, generator=g) * 0.1
+    v = torch.randn(n, Hk, D, generator=g)
+    q = u[:, None, :].expand(n_new, H, D).contiguous()
+    for t, p in enumerate(far):
+        k[p] = u[t]
+    tables, n_pages = scatter_pages([n], ps, 5)
+    kc, vc = fill_cache([k], [v], tables, n_pages, ps, torch.bfloat16)
+    ctx = FakeCtx([start], [n_new], tables, ps, cta_tiles=1000)
+    plan = ctx.attention_plan(0, H // Hk, window, Hk, ps)
+    assert plan.n_cta_items >= 1 and plan.n_jobs == 0
+    scale = 1 / math.sqrt(D)
+    got = ops.attention(q.bfloat16().to(DEV).reshape(n_new, H * D), kc, vc, ctx, 0, H, Hk, D, ps, scale, window)
+    got = got.cpu().reshape(n_new, H, D).float()
+    want = ref_attention(q.bfloat16().float(), [k.bfloat16().float()], [v.bfloat16().float()], [start], [n_new], scale, window)
+    err = (got.double() - want).abs().amax(dim=(1, 2)) / want.abs().amax()
+    assert err.max() < 1.2e-2, f"token {int(err.argmax())} (its key at {far[int(err.argmax())]}): {float(err.max())}"
+    own = torch.stack([v.bfloat16().float()[p] for p in far]).repeat_interleave(H // Hk, dim=1)
+    assert rel(got, own) < 2e-2
+
+
 @pytest.mark.parametrize("dt", ["float32", "bfloat16"])
 def test_attention_window_edge(ops, dt):
     """The key just outside the window is made huge: it must not be seen; the one just inside must."""
